@@ -1,0 +1,138 @@
+/*
+ * slowrun_ce.h - C ABI of libslowrun_ce.so: fused fp8 LM-head + tanh-softcap +
+ * cross-entropy, forward and backward, for AMD MI355X (gfx950).
+ *
+ * The reference has no FFI for this path: its "binding" is a CUDA source string
+ * compiled at import time (tiny/cuda_kernels.py:305-312) and wrapped as the
+ * custom op nanogpt::ce_fwd_bwd (tiny/cuda_kernels.py:314-334), called from
+ * FusedSoftcappedCrossEntropy.forward/backward (tiny/cuda_kernels.py:336-414).
+ * The entry points below are what a binding for that autograd Function needs:
+ * plain pointers and sizes, no framework types.
+ *
+ * Conventions
+ *  - every pointer is a device pointer on `device`; the caller owns all memory,
+ *    including the saved state and the workspaces; the library allocates no
+ *    device memory and keeps no pointer after a call returns;
+ *  - all work is enqueued on `stream` (a hipStream_t, NULL = default stream);
+ *    no call synchronises with the host;
+ *  - return value 0 = success, otherwise an SCE_E* code; sce_last_error() gives
+ *    a message for the calling thread;
+ *  - X is (N, d) row-major, W is (d, V) row-major (the layout of the reference's
+ *    CastedLinearT, tiny/train.py:489-497), targets are int64 with
+ *    `ignore_index` marking rows that take no part (tiny/train.py:743).
+ */
+#ifndef SLOWRUN_CE_H
+#define SLOWRUN_CE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SCE_VERSION 1
+
+enum { SCE_F32 = 0, SCE_BF16 = 1 };               /* element types of X, W, dX, dW          */
+enum { SCE_REDUCE_NONE = 0, SCE_REDUCE_MEAN = 1 }; /* F.cross_entropy(reduction=...)         */
+
+enum {
+  SCE_OK = 0,
+  SCE_EINVAL = 1,      /* bad shape, dtype, alignment, null pointer, workspace too small     */
+  SCE_EARCH = 2,       /* device is not gfx950                                               */
+  SCE_EHIP = 3         /* a HIP runtime call failed                                          */
+};
+
+typedef struct sce_shape {
+  int64_t N;           /* rows (tokens)                         */
+  int64_t d;           /* hidden size, multiple of 16           */
+  int64_t V;           /* vocabulary (columns of W), < 2^31     */
+  int32_t n_predict;   /* number of MTP offsets, 1..4           */
+  int32_t reserved;
+} sce_shape;
+
+typedef struct sce_sizes {
+  size_t saved_bytes;        /* state written by sce_forward and read by sce_backward        */
+  size_t fwd_workspace_bytes;
+  size_t bwd_workspace_min_bytes;   /* backward with the smallest row panel (256 rows)       */
+  size_t bwd_workspace_bytes;       /* backward with the default row panel                   */
+  int64_t bwd_panel_rows;           /* the default row panel                                 */
+} sce_sizes;
+
+typedef struct sce_args {
+  uint32_t struct_size;      /* sizeof(sce_args), checked                                    */
+  int32_t device;            /* HIP device ordinal the pointers live on                      */
+  void* stream;              /* hipStream_t                                                  */
+  sce_shape shape;
+
+  /* ---- inputs (forward) ---- */
+  const void* x;  int32_t x_dtype;  int32_t pad0;  int64_t x_ld;   /* (N,d), row stride in elements */
+  const void* w;  int32_t w_dtype;  int32_t pad1;  int64_t w_ld;   /* (d,V), row stride in elements */
+  const int64_t* targets;    /* (N,)                                                         */
+  const float* mtp_weights;  /* (n_predict,) on the device, or NULL for a single weight 1    */
+  float x_s, w_s;            /* fp8 scales: X_q = e4m3(X / x_s), W_q = e4m3(W / w_s)         */
+  float cap;                 /* z = cap * tanh(u / cap), 0 < cap <= 40                       */
+  float grad_scale;          /* multiplies every gradient (tiny/cuda_kernels.py:265)         */
+  int64_t ignore_index;
+  int32_t reduction;         /* SCE_REDUCE_*                                                 */
+  int32_t pad2;
+
+  /* ---- outputs (forward) ---- */
+  float* loss;               /* [1] mean over valid rows (written when reduction = mean)     */
+  float* losses;             /* (N,) per-row loss, 0 at ignored rows; may be NULL for mean   */
+  float* lse;                /* (N,) log-sum-exp of the capped logits; optional              */
+  int32_t* argmax;           /* (N,) argmax over V of the uncapped logits; optional          */
+  int32_t* n_valid;          /* [2]: number of valid rows, number of out-of-range targets    */
+
+  /* ---- state and scratch ---- */
+  void* saved;      size_t saved_bytes;
+  void* workspace;  size_t workspace_bytes;
+
+  /* ---- backward ---- */
+  const float* grad_output;  /* [1] for reduction = mean, (N,) for reduction = none          */
+  void* dx;  int32_t dx_dtype;  int32_t pad3;  int64_t dx_ld;      /* (N,d)                  */
+  void* dw;  int32_t dw_dtype;  int32_t pad4;  int64_t dw_ld;      /* (d,V)                  */
+  int64_t panel_rows;        /* 0 = as many rows per panel as the workspace allows           */
+} sce_args;
+
+/* Library / ABI version (SCE_VERSION of the build). */
+int sce_version(void);
+
+/* Message for the last non-zero return code on this thread ("" if none). */
+const char* sce_last_error(void);
+
+/* Buffer sizes for a problem shape.  Replaces the torch.empty calls in
+ * FusedSoftcappedCrossEntropy.forward/backward (tiny/cuda_kernels.py:359-366,398-401). */
+int sce_sizes_for(const sce_shape* shape, sce_sizes* out);
+
+/* Per-tensor scaled cast to OCP e4m3: dst[i] = e4m3_rne(src[i] / scale), NaN code above
+ * 464 like Tensor.to(float8_e4m3fn); bf16 input is divided in fp32 and rounded to bf16
+ * first, as torch does.  Replaces x.div(x_s).to(torch.float8_e4m3fn)
+ * (tiny/cuda_kernels.py:340-341). */
+int sce_quantize_e4m3(const void* src, int32_t src_dtype, void* dst, float scale, size_t n,
+                      int32_t device, void* stream);
+
+/* dst (cols, rows) = transpose of src (rows, cols), one byte per element.  Replaces
+ * transpose_copy (tiny/cuda_kernels.py:56-78) for callers that still want it; the fused
+ * path itself never materialises a transposed N x V matrix. */
+int sce_transpose_bytes(const void* src, void* dst, int64_t rows, int64_t cols,
+                        int32_t device, void* stream);
+
+/* Forward: quantise X and W, contract on fp8 MFMA, softcap, online log-sum-exp, loss.
+ * Replaces FusedSoftcappedCrossEntropy.forward (tiny/cuda_kernels.py:336-373) and the
+ * kernel it launches (tiny/cuda_kernels.py:125-240).  Uses args->workspace
+ * (fwd_workspace_bytes) and fills args->saved. */
+int sce_forward(const sce_args* args);
+
+/* Backward: recompute logit tiles from the saved fp8 operands, form dlogits on chip,
+ * dX = dlogits * W_q^T, dW = X_q^T * dlogits.  Replaces
+ * FusedSoftcappedCrossEntropy.backward (tiny/cuda_kernels.py:375-414) and the dlogits half
+ * of the reference kernel (tiny/cuda_kernels.py:242-301).  Needs the `saved` buffer of the
+ * matching sce_forward call, the same shape/scales/cap/targets, and a workspace of at
+ * least bwd_workspace_min_bytes. */
+int sce_backward(const sce_args* args);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

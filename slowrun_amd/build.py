@@ -1,0 +1,53 @@
+"""Compiles libslowrun_ce.so (gfx950) in-tree with hipcc.
+
+``python -m slowrun_amd.build`` or ``build_library()``.  The library is loaded by
+``slowrun_amd._lib``; nothing is compiled at import time.
+"""
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_PATH = os.path.join(HERE, "libslowrun_ce.so")
+SOURCES = ["sce_kernels.hip", "sce_sort.hip"]
+# packed fp32 math is kept off for every device function in this library
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             "-Wno-unused-command-line-argument"]
+
+
+def build_library(verbose=True, jobs=2):
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    objs, procs = [], []
+    for src in SOURCES:
+        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+        cmd = [hipcc, *HIP_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        objs.append(obj)
+        if len(procs) >= jobs:
+            _wait(procs, verbose)
+    _wait(procs, verbose)
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return LIB_PATH
+
+
+def _wait(procs, verbose):
+    while procs:
+        src, p = procs.pop(0)
+        out, _ = p.communicate()
+        out = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l)
+        if p.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src}:\n{out}")
+        if verbose and out.strip():
+            print(out, flush=True)
+
+
+if __name__ == "__main__":
+    print(build_library())
+    sys.exit(0)

@@ -1,0 +1,1067 @@
+// gfx950 (MI355X, CDNA4) kernels for the fused fp8 LM-head + tanh-softcap + cross-entropy
+// loss head, and the C ABI declared in include/slowrun_ce.h.
+//
+// Replaces, in the reference: the quantise / _scaled_mm / ce_fwd_bwd / transpose_copy chain of
+// FusedSoftcappedCrossEntropy (tiny/cuda_kernels.py:336-414, kernel at :125-302).
+//
+// Data flow
+//   forward : X, W --quantise--> X_q [Np][dp], W_q^T [Vp][dp], W_q [dq][Vp]   (OCP e4m3, zero padded)
+//             fwd_kernel: 256x256 logit tiles on v_mfma_f32_32x32x64_f8f6f4, epilogue keeps
+//             per-row sum exp(z - cap), max/argmax of u and the target logit in registers;
+//             the logits never leave the chip.  Partials per (row, V-split) -> combine.
+//   backward: per panel of P rows: recompute the logit tiles, turn them in registers into
+//             G = 256 * (1 - t^2) * exp(z - zmax_row) (e4m3), written once row-major and once
+//             transposed into a panel-sized scratch; dX = rho_row * G W_q^T and
+//             dW += (rho X_q)^T G run on the same MFMA main loop.  The one-hot part of
+//             dlogits never goes through fp8: it is applied in fp32 in the dX epilogue
+//             (gather of W_q^T rows) and in the dW finalisation (rows grouped by target).
+#include "sce_common.h"
+#include "../../include/slowrun_ce.h"
+
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+#include <mutex>
+
+namespace sce {
+
+// ------------------------------------------------------------------------------------------
+// small device helpers
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {   // round to nearest even
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);   // NaN stays NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float round_to_bf16(float f) { return bf16_bits_to_float(float_to_bf16_bits(f)); }
+
+// two floats -> two e4m3 bytes (low half of the result).  v_cvt_pk_fp8_f32 on gfx950 is OCP
+// e4m3fn, round to nearest even, 464 -> 448 and anything larger -> NaN code: the same rule as
+// Tensor.to(torch.float8_e4m3fn).
+__device__ __forceinline__ uint32_t cvt2_e4m3(float a, float b) {
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xffffu;
+}
+__device__ __forceinline__ uint32_t cvt4_e4m3(float a, float b, float c, float d) {
+  int w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+  return (uint32_t)w;
+}
+template <int SEL>
+__device__ __forceinline__ float e4m3_to_float(uint32_t word) { return __builtin_amdgcn_cvt_f32_fp8((int)word, SEL); }
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+  static __device__ __forceinline__ float load(const float* p) { return *p; }
+  static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+  static __device__ __forceinline__ float div_round(float x, float s) { return x / s; }
+};
+struct bf16_t { uint16_t bits; };
+template <> struct Elem<bf16_t> {
+  static __device__ __forceinline__ float load(const bf16_t* p) { return bf16_bits_to_float(p->bits); }
+  static __device__ __forceinline__ void store(bf16_t* p, float v) { p->bits = float_to_bf16_bits(v); }
+  // torch divides a bf16 tensor in fp32 and rounds the quotient back to bf16 before the fp8 cast
+  static __device__ __forceinline__ float div_round(float x, float s) { return round_to_bf16(x / s); }
+};
+
+// XCD-aware tile order.  Consecutive workgroup ids go round-robin to the 8 XCDs, each with its
+// own L2; the 32 workgroups resident on one XCD are given a 4 x 8 block of tiles so that they
+// share A-side and B-side rows through that L2.
+__device__ __forceinline__ bool map_tile(int bid, int RT, int CT, int& rt, int& ct) {
+  const int xcd = bid & 7, slot = bid >> 3;
+  const int c = slot >> 5, w = slot & 31;
+  const int st = c * 8 + xcd;
+  const int SC = (CT + 7) >> 3;
+  const int sr = st / SC, sc = st - sr * SC;
+  rt = sr * 4 + (w >> 3);
+  ct = sc * 8 + (w & 7);
+  return rt < RT && ct < CT;
+}
+static inline int map_tile_grid(int RT, int CT) {
+  const int SR = (RT + 3) / 4, SC = (CT + 7) / 8;
+  return 8 * 32 * ((SR * SC + 7) / 8);
+}
+
+// ------------------------------------------------------------------------------------------
+// MFMA main loop: acc[a][b] (32x32 blocks) += A_tile[256][K] * B_tile[256][K]^T, fp8 e4m3.
+// Wave (wa, wb) of the 2 x 2 wave grid owns A rows [128 wa, +128) and B rows [128 wb, +128).
+// Global -> registers -> LDS, two LDS stages, one barrier per 128 bytes of K.
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, int64_t lda,
+                                              const uint8_t* __restrict__ Bg, int64_t ldb, int KT,
+                                              uint8_t* smem, v16f (&acc)[4][4]) {
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
+  const int lrow = t >> 3, lcol = (t & 7) * 16;
+  const uint8_t* ap = Ag + (int64_t)lrow * lda + lcol;
+  const uint8_t* bp = Bg + (int64_t)lrow * ldb + lcol;
+  v4i ra[8], rb[8];
+
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  auto gload = [&](int kt) {
+#pragma unroll
+    for (int n = 0; n < 8; ++n) {
+      ra[n] = *reinterpret_cast<const v4i*>(ap + (int64_t)(32 * n) * lda + (int64_t)kt * BK);
+      rb[n] = *reinterpret_cast<const v4i*>(bp + (int64_t)(32 * n) * ldb + (int64_t)kt * BK);
+    }
+  };
+  auto swrite = [&](int stage) {
+    uint8_t* sa = smem + stage * STAGE_BYTES + lrow * PITCH + lcol;
+    uint8_t* sb = sa + TM * PITCH;
+#pragma unroll
+    for (int n = 0; n < 8; ++n) {
+      *reinterpret_cast<v4i*>(sa + 32 * n * PITCH) = ra[n];
+      *reinterpret_cast<v4i*>(sb + 32 * n * PITCH) = rb[n];
+    }
+  };
+
+  gload(0);
+  swrite(0);
+  __syncthreads();
+  const int frag_off = (lane & 31) * PITCH + (lane >> 5) * 32;
+  for (int kt = 0; kt < KT; ++kt) {
+    const bool more = kt + 1 < KT;
+    if (more) gload(kt + 1);
+    const uint8_t* sa = smem + (kt & 1) * STAGE_BYTES + wa * 128 * PITCH + frag_off;
+    const uint8_t* sb = smem + (kt & 1) * STAGE_BYTES + (TM + wb * 128) * PITCH + frag_off;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      v8i fa[4], fb[4];
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const v4i lo = *reinterpret_cast<const v4i*>(sa + a * 32 * PITCH + s * 64);
+        const v4i hi = *reinterpret_cast<const v4i*>(sa + a * 32 * PITCH + s * 64 + 16);
+        fa[a] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const v4i lo = *reinterpret_cast<const v4i*>(sb + b * 32 * PITCH + s * 64);
+        const v4i hi = *reinterpret_cast<const v4i*>(sb + b * 32 * PITCH + s * 64 + 16);
+        fb[b] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[a], fb[b], acc[a][b], 0, 0, 0, 0, 0, 0);
+    }
+    if (more) swrite((kt + 1) & 1);
+    __syncthreads();
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// quantisation
+// ------------------------------------------------------------------------------------------
+// dst [rows_p][cols_p] e4m3 = src [rows][cols] / scale, zero outside; 16 outputs per thread.
+template <typename T>
+__global__ __launch_bounds__(256) void quantize_pad_kernel(const T* __restrict__ src, int64_t ld, int64_t rows,
+                                                          int64_t cols, uint8_t* __restrict__ dst,
+                                                          int64_t rows_p, int64_t cols_p, float scale) {
+  const int64_t chunks_per_row = cols_p / 16;
+  const int64_t total = rows_p * chunks_per_row;
+  for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < total; q += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = q / chunks_per_row, c0 = (q - r * chunks_per_row) * 16;
+    uint32_t out[4] = {0, 0, 0, 0};
+    if (r < rows && c0 < cols) {
+      float v[16];
+#pragma unroll
+      for (int m = 0; m < 16; ++m)
+        v[m] = (c0 + m < cols) ? Elem<T>::div_round(Elem<T>::load(src + r * ld + c0 + m), scale) : 0.f;
+#pragma unroll
+      for (int m = 0; m < 4; ++m) out[m] = cvt4_e4m3(v[4 * m], v[4 * m + 1], v[4 * m + 2], v[4 * m + 3]);
+    }
+    *reinterpret_cast<v4i*>(dst + r * cols_p + c0) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
+  }
+}
+
+// W (d, V) -> W_q [dq][Vp] (same orientation) and W_q^T [Vp][dp]; 64 x 64 tiles through LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void quantize_w_kernel(const T* __restrict__ w, int64_t ld, int64_t d, int64_t V,
+                                                        uint8_t* __restrict__ wq, uint8_t* __restrict__ wqt,
+                                                        int64_t dp, int64_t Vp, float scale) {
+  __shared__ uint8_t tile[64][68];
+  const int t = threadIdx.x;
+  const int64_t j0 = (int64_t)blockIdx.y * 64, v0 = (int64_t)blockIdx.x * 64;
+  {
+    const int r = t >> 2, c = (t & 3) * 16;
+    const int64_t j = j0 + r, v = v0 + c;
+    uint32_t out[4] = {0, 0, 0, 0};
+    if (j < d && v < V) {
+      float x[16];
+#pragma unroll
+      for (int m = 0; m < 16; ++m)
+        x[m] = (v + m < V) ? Elem<T>::div_round(Elem<T>::load(w + j * ld + v + m), scale) : 0.f;
+#pragma unroll
+      for (int m = 0; m < 4; ++m) out[m] = cvt4_e4m3(x[4 * m], x[4 * m + 1], x[4 * m + 2], x[4 * m + 3]);
+    }
+    *reinterpret_cast<v4i*>(wq + j * Vp + v) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
+#pragma unroll
+    for (int m = 0; m < 4; ++m) *reinterpret_cast<uint32_t*>(&tile[r][c + 4 * m]) = out[m];
+  }
+  __syncthreads();
+  if (j0 < dp) {
+    const int vr = t >> 2, jc = (t & 3) * 16;
+    uint32_t out[4];
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      out[m] = (uint32_t)tile[jc + 4 * m][vr] | ((uint32_t)tile[jc + 4 * m + 1][vr] << 8) |
+               ((uint32_t)tile[jc + 4 * m + 2][vr] << 16) | ((uint32_t)tile[jc + 4 * m + 3][vr] << 24);
+    }
+    *reinterpret_cast<v4i*>(wqt + (v0 + vr) * dp + j0 + jc) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
+  }
+}
+
+// flat cast, for the standalone sce_quantize_e4m3 entry point
+template <typename T>
+__global__ __launch_bounds__(256) void quantize_flat_kernel(const T* __restrict__ src, uint8_t* __restrict__ dst,
+                                                           size_t n, float scale) {
+  for (size_t q = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; q < n; q += (size_t)gridDim.x * blockDim.x * 4) {
+    float v[4];
+#pragma unroll
+    for (int m = 0; m < 4; ++m) v[m] = (q + m < n) ? Elem<T>::div_round(Elem<T>::load(src + q + m), scale) : 0.f;
+    const uint32_t w = cvt4_e4m3(v[0], v[1], v[2], v[3]);
+    if (q + 4 <= n && (((uintptr_t)(dst + q)) & 3) == 0) {
+      *reinterpret_cast<uint32_t*>(dst + q) = w;
+    } else {
+      for (int m = 0; m < 4 && q + m < n; ++m) dst[q + m] = (uint8_t)(w >> (8 * m));
+    }
+  }
+}
+
+// dst (cols, rows) = src (rows, cols)^T, bytes.
+__global__ __launch_bounds__(256) void transpose_bytes_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                             int64_t rows, int64_t cols) {
+  __shared__ uint8_t tile[64][68];
+  const int t = threadIdx.x;
+  const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+  for (int e = t; e < 64 * 64; e += 256) {
+    const int r = e >> 6, c = e & 63;
+    tile[r][c] = (r0 + r < rows && c0 + c < cols) ? src[(r0 + r) * cols + c0 + c] : 0;
+  }
+  __syncthreads();
+  for (int e = t; e < 64 * 64; e += 256) {
+    const int c = e >> 6, r = e & 63;
+    if (r0 + r < rows && c0 + c < cols) dst[(c0 + c) * rows + r0 + r] = tile[r][c];
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// forward
+// ------------------------------------------------------------------------------------------
+struct FwdParams {
+  const uint8_t* xq;       // [Np][dp]
+  const uint8_t* wqt;      // [Vp][dp]
+  const int64_t* targets;  // [N]
+  float4* partials;        // [S][Np]: sum exp(z - cap), max u, argmax u (bits), z at target (-inf if not seen)
+  int64_t dp;
+  int N, V, Np, RT, CT, S;
+  float sc;                // x_s * w_s
+  float c1;                // 2 log2(e) / cap
+  float c2;                // -2 cap log2(e)
+  float cap;
+};
+
+template <bool EDGE>
+__device__ __forceinline__ void fwd_epilogue(const v16f (&acc)[4][4], const FwdParams& p, int vbase, const int (&dy)[4],
+                                             float (&sum)[4], float (&umax)[4], int (&uarg)[4], float (&zy)[4]) {
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    float tmax = -INFINITY, rry = 2.0f;     // best u of this tile and its offset; 1/(E+1) at the target (2 = not here)
+    int targ = 0;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int vo = a * 32 + 8 * (r >> 2) + (r & 3);
+        float u = acc[a][b][r] * p.sc;
+        const float rr = fast_rcp(fast_exp2(u * p.c1) + 1.0f);   // 1 / (e^{2u/cap} + 1), so tanh = 1 - 2 rr
+        float pt = fast_exp2(p.c2 * rr);                          // e^{z - cap}
+        if (EDGE) {
+          if (vo >= p.V - vbase) { pt = 0.f; u = -INFINITY; }
+        }
+        sum[b] += pt;
+        if (u > tmax) { tmax = u; targ = vo; }
+        if (dy[b] == vo) rry = rr;
+      }
+    }
+    if (tmax > umax[b]) { umax[b] = tmax; uarg[b] = vbase + targ; }
+    if (rry < 2.0f) zy[b] = p.cap - 2.0f * p.cap * rry;
+  }
+}
+
+__global__ __launch_bounds__(256) void fwd_kernel(FwdParams p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int bid = blockIdx.x, xcd = bid & 7, slot = bid >> 3;
+  const int s = slot % p.S, rt = (slot / p.S) * 8 + xcd;
+  if (rt >= p.RT) return;
+  const int ct0 = (int)((int64_t)p.CT * s / p.S), ct1 = (int)((int64_t)p.CT * (s + 1) / p.S);
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
+
+  int y[4];
+  float sum[4], umax[4], zy[4];
+  int uarg[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int i = rt * 256 + wb * 128 + b * 32 + (lane & 31);
+    int64_t yy = (i < p.N) ? p.targets[i] : -1;
+    y[b] = (yy >= 0 && yy < p.V) ? (int)yy : -0x40000000;
+    sum[b] = 0.f; umax[b] = -INFINITY; uarg[b] = 0x7fffffff; zy[b] = -INFINITY;
+  }
+  v16f acc[4][4];
+  const uint8_t* Bg = p.xq + (int64_t)rt * 256 * p.dp;
+  const int KT = (int)(p.dp / BK);
+  for (int ct = ct0; ct < ct1; ++ct) {
+    mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.dp, p.dp, Bg, p.dp, KT, smem, acc);
+    const int vbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
+    int dy[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) dy[b] = y[b] - vbase;
+    if (ct * 256 + 256 > p.V) fwd_epilogue<true>(acc, p, vbase, dy, sum, umax, uarg, zy);
+    else fwd_epilogue<false>(acc, p, vbase, dy, sum, umax, uarg, zy);
+  }
+  // the two half-waves hold different columns of the same rows
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const float s2 = __shfl_xor(sum[b], 32), um2 = __shfl_xor(umax[b], 32), zy2 = __shfl_xor(zy[b], 32);
+    const int ua2 = __shfl_xor(uarg[b], 32);
+    sum[b] += s2;
+    if (um2 > umax[b] || (um2 == umax[b] && ua2 < uarg[b])) { umax[b] = um2; uarg[b] = ua2; }
+    zy[b] = fmaxf(zy[b], zy2);
+  }
+  // waves wa = 0 and wa = 1 hold different columns of the same rows
+  float4* red = reinterpret_cast<float4*>(smem);
+  if (wa == 1 && lane < 32) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) red[wb * 128 + b * 32 + lane] = make_float4(sum[b], umax[b], __int_as_float(uarg[b]), zy[b]);
+  }
+  __syncthreads();
+  if (wa == 0 && lane < 32) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const float4 o = red[wb * 128 + b * 32 + lane];
+      const int ua2 = __float_as_int(o.z);
+      sum[b] += o.x;
+      if (o.y > umax[b] || (o.y == umax[b] && ua2 < uarg[b])) { umax[b] = o.y; uarg[b] = ua2; }
+      zy[b] = fmaxf(zy[b], o.w);
+      p.partials[(int64_t)s * p.Np + rt * 256 + wb * 128 + b * 32 + lane] =
+          make_float4(sum[b], umax[b], __int_as_float(uarg[b]), zy[b]);
+    }
+  }
+}
+
+// one thread per row: fold the V-splits, write lse / loss / argmax and the saved row statistics
+__global__ __launch_bounds__(256) void fwd_combine_kernel(const float4* __restrict__ partials, int S, int N, int Np, int V,
+                                                         const int64_t* __restrict__ targets, int64_t ignore_index, float cap,
+                                                         float* __restrict__ s_lse, float* __restrict__ s_umax,
+                                                         float* __restrict__ s_zy, float* __restrict__ losses,
+                                                         float* __restrict__ lse_out, int32_t* __restrict__ argmax_out) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= Np) return;
+  if (i >= N) { s_lse[i] = 0.f; s_umax[i] = 0.f; s_zy[i] = 0.f; return; }
+  float sum = 0.f, umax = -INFINITY, zy = -INFINITY;
+  int uarg = 0x7fffffff;
+  for (int s = 0; s < S; ++s) {
+    const float4 o = partials[(int64_t)s * Np + i];
+    const int ua = __float_as_int(o.z);
+    sum += o.x;
+    if (o.y > umax || (o.y == umax && ua < uarg)) { umax = o.y; uarg = ua; }
+    zy = fmaxf(zy, o.w);
+  }
+  const float lse = cap + logf(sum);
+  const int64_t y = targets[i];
+  const bool valid = (y != ignore_index) && y >= 0 && y < V;
+  s_lse[i] = lse; s_umax[i] = umax; s_zy[i] = valid ? zy : 0.f;
+  if (losses) losses[i] = valid ? (lse - zy) : 0.f;
+  if (lse_out) lse_out[i] = lse;
+  if (argmax_out) argmax_out[i] = (uarg == 0x7fffffff) ? 0 : uarg;
+}
+
+// single workgroup: n_valid, number of out-of-range targets, mean loss (deterministic order)
+__global__ __launch_bounds__(1024) void fwd_reduce_kernel(const float* __restrict__ s_lse, const float* __restrict__ s_zy,
+                                                         const int64_t* __restrict__ targets, int64_t ignore_index, int N, int V,
+                                                         int32_t* __restrict__ hdr, float* __restrict__ loss_out,
+                                                         int32_t* __restrict__ nvalid_out) {
+  __shared__ double ssum[1024];
+  __shared__ int scnt[1024], sbad[1024];
+  const int t = threadIdx.x;
+  double acc = 0.0;
+  int cnt = 0, bad = 0;
+  for (int i = t; i < N; i += 1024) {
+    const int64_t y = targets[i];
+    if (y == ignore_index) continue;
+    if (y < 0 || y >= V) { ++bad; continue; }
+    acc += (double)(s_lse[i] - s_zy[i]);
+    ++cnt;
+  }
+  ssum[t] = acc; scnt[t] = cnt; sbad[t] = bad;
+  __syncthreads();
+  for (int w = 512; w > 0; w >>= 1) {
+    if (t < w) { ssum[t] += ssum[t + w]; scnt[t] += scnt[t + w]; sbad[t] += sbad[t + w]; }
+    __syncthreads();
+  }
+  if (t == 0) {
+    hdr[0] = scnt[0]; hdr[1] = sbad[0];
+    const float mean = (float)(ssum[0] / (double)scnt[0]);   // 0/0 = NaN, as F.cross_entropy gives
+    reinterpret_cast<float*>(hdr)[2] = mean;
+    if (loss_out) *loss_out = mean;
+    if (nvalid_out) { nvalid_out[0] = scnt[0]; nvalid_out[1] = sbad[0]; }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// backward
+// ------------------------------------------------------------------------------------------
+// per row: c_row (exponent offset of G), rho (row scale of G), h (one-hot coefficient)
+__global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__ s_lse, const float* __restrict__ s_umax,
+                                                      const float* __restrict__ s_zy, const int64_t* __restrict__ targets,
+                                                      int64_t ignore_index, const int32_t* __restrict__ hdr,
+                                                      const float* __restrict__ grad_output, int per_row, float grad_scale,
+                                                      float cap, int N, int Np, int V, float* __restrict__ crow,
+                                                      float* __restrict__ rho, float* __restrict__ hcoef,
+                                                      float* __restrict__ blockmax) {
+  __shared__ float smax[256];
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  float c = -INFINITY, r = 0.f, h = 0.f;
+  if (i < N) {
+    const int64_t y = targets[i];
+    const bool valid = (y != ignore_index) && y >= 0 && y < V;
+    if (valid) {
+      const float g = (per_row ? grad_output[i] : grad_output[0] / (float)hdr[0]) * grad_scale;
+      const float zmax = cap * tanhf(s_umax[i] / cap);
+      c = (cap - zmax) * LOG2E + 10.0f;        // G = 2^c * r(1-r) * e^{z-cap} = 256 (1-t^2) e^{z-zmax}
+      r = g * expf(zmax - s_lse[i]) * (1.0f / 256.0f);
+      const float ty = s_zy[i] / cap;
+      h = g * (1.0f - ty * ty);
+    }
+  }
+  if (i < Np) { crow[i] = c; rho[i] = r; hcoef[i] = h; }
+  smax[threadIdx.x] = fabsf(r);
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if (threadIdx.x < w) smax[threadIdx.x] = fmaxf(smax[threadIdx.x], smax[threadIdx.x + w]);
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) blockmax[blockIdx.x] = smax[0];
+}
+
+__global__ __launch_bounds__(1024) void bwd_xi_kernel(const float* __restrict__ blockmax, int n, float* __restrict__ xi) {
+  __shared__ float smax[1024];
+  float m = 0.f;
+  for (int i = threadIdx.x; i < n; i += 1024) m = fmaxf(m, blockmax[i]);
+  smax[threadIdx.x] = m;
+  __syncthreads();
+  for (int w = 512; w > 0; w >>= 1) {
+    if (threadIdx.x < w) smax[threadIdx.x] = fmaxf(smax[threadIdx.x], smax[threadIdx.x + w]);
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) xi[0] = (smax[0] > 0.f && isfinite(smax[0])) ? smax[0] : 1.0f;
+}
+
+// Xt [dq][Np] = e4m3( X_q[i][j] * rho_i / xi ), transposed through LDS in 64 x 64 tiles.
+__global__ __launch_bounds__(256) void bwd_xt_kernel(const uint8_t* __restrict__ xq, int64_t dp, int64_t Np,
+                                                    const float* __restrict__ rho, const float* __restrict__ xi,
+                                                    uint8_t* __restrict__ xt) {
+  __shared__ uint8_t tile[64][68];
+  const int t = threadIdx.x;
+  const int64_t i0 = (int64_t)blockIdx.x * 64, j0 = (int64_t)blockIdx.y * 64;
+  if (j0 < dp) {
+    const int r = t >> 2, c = (t & 3) * 16;
+    const v4i raw = *reinterpret_cast<const v4i*>(xq + (i0 + r) * dp + j0 + c);
+    const float f = rho[i0 + r] / xi[0];
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const uint32_t w = (uint32_t)raw[m];
+      const uint32_t o = cvt4_e4m3(e4m3_to_float<0>(w) * f, e4m3_to_float<1>(w) * f, e4m3_to_float<2>(w) * f,
+                                   e4m3_to_float<3>(w) * f);
+      *reinterpret_cast<uint32_t*>(&tile[r][c + 4 * m]) = o;
+    }
+  } else {
+    for (int e = t; e < 64 * 17; e += 256) reinterpret_cast<uint32_t*>(&tile[0][0])[e] = 0;
+  }
+  __syncthreads();
+  const int jr = t >> 2, ic = (t & 3) * 16;
+  uint32_t out[4];
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    out[m] = (uint32_t)tile[ic + 4 * m][jr] | ((uint32_t)tile[ic + 4 * m + 1][jr] << 8) |
+             ((uint32_t)tile[ic + 4 * m + 2][jr] << 16) | ((uint32_t)tile[ic + 4 * m + 3][jr] << 24);
+  }
+  *reinterpret_cast<v4i*>(xt + (j0 + jr) * Np + i0 + ic) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
+}
+
+struct RecomputeParams {
+  const uint8_t* xq;     // [Np][dp], already offset to the panel's first row
+  const uint8_t* wqt;    // [Vp][dp]
+  const float* crow;     // offset to the panel's first row
+  uint8_t* ghat;         // [P][Vp]
+  uint8_t* ghat_t;       // [Vp][P]
+  int64_t dp, Vp, P;
+  int RT, CT, V;
+  float sc, c1, c2;
+};
+
+// Recompute a 256 x 256 logit tile and leave G = 256 (1 - t^2) e^{z - zmax_row} in e4m3, once
+// row-major (operand of dX) and once transposed (operand of dW).
+__global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  int rt, ct;
+  if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
+  v16f acc[4][4];
+  mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.dp, p.dp, p.xq + (int64_t)rt * 256 * p.dp, p.dp, (int)(p.dp / BK), smem, acc);
+  const int vbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
+  const bool edge = ct * 256 + 256 > p.V;
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int il = rt * 256 + wb * 128 + b * 32 + (lane & 31);      // row within the panel
+    const float c = p.crow[il];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float g[4];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          const float u = acc[a][b][4 * q + m] * p.sc;
+          const float rr = fast_rcp(fast_exp2(u * p.c1) + 1.0f);
+          g[m] = fast_exp2(fmaf(p.c2, rr, c)) * (rr - rr * rr);
+        }
+        const int v = vbase + a * 32 + 8 * q;
+        if (edge) {
+#pragma unroll
+          for (int m = 0; m < 4; ++m) if (v + m >= p.V) g[m] = 0.f;
+        }
+        const uint32_t w = cvt4_e4m3(g[0], g[1], g[2], g[3]);
+        *reinterpret_cast<uint32_t*>(p.ghat + (int64_t)il * p.Vp + v) = w;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) p.ghat_t[(int64_t)(v + m) * p.P + il] = (uint8_t)(w >> (8 * m));
+      }
+    }
+  }
+}
+
+struct DxParams {
+  const uint8_t* wq;      // [dq][Vp]   A side (rows j)
+  const uint8_t* ghat;    // [P][Vp]    B side (rows i of the panel)
+  const uint8_t* wqt;     // [Vp][dp]   for the one-hot gather
+  const float* rho;       // offset to the panel
+  const float* hcoef;     // offset to the panel
+  const int64_t* targets; // offset to the panel
+  void* dx;               // offset to the panel's first row
+  int64_t dx_ld, Vp, dp;
+  int RT, CT, rows, d, V;  // rows: valid rows in this panel
+  float w_s;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  int rt, ct;
+  if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
+  v16f acc[4][4];
+  mfma_mainloop(p.wq + (int64_t)ct * 256 * p.Vp, p.Vp, p.ghat + (int64_t)rt * 256 * p.Vp, p.Vp, (int)(p.Vp / BK), smem, acc);
+  const int jbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
+  T* dx = reinterpret_cast<T*>(p.dx);
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int il = rt * 256 + wb * 128 + b * 32 + (lane & 31);
+    if (il >= p.rows) continue;
+    const float rs = p.rho[il] * p.w_s;
+    const float hs = p.hcoef[il] * p.w_s;
+    const int64_t y = p.targets[il];
+    const uint8_t* wrow = p.wqt + ((hs != 0.f && y >= 0 && y < p.V) ? y : 0) * p.dp;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int j = jbase + a * 32 + 8 * q;
+        if (j >= p.d) continue;                       // d is a multiple of 4, so j..j+3 are in range together
+        const uint32_t w = *reinterpret_cast<const uint32_t*>(wrow + j);
+        const float o0 = acc[a][b][4 * q + 0] * rs - hs * e4m3_to_float<0>(w);
+        const float o1 = acc[a][b][4 * q + 1] * rs - hs * e4m3_to_float<1>(w);
+        const float o2 = acc[a][b][4 * q + 2] * rs - hs * e4m3_to_float<2>(w);
+        const float o3 = acc[a][b][4 * q + 3] * rs - hs * e4m3_to_float<3>(w);
+        T* dst = dx + (int64_t)il * p.dx_ld + j;
+        Elem<T>::store(dst + 0, o0); Elem<T>::store(dst + 1, o1);
+        Elem<T>::store(dst + 2, o2); Elem<T>::store(dst + 3, o3);
+      }
+    }
+  }
+}
+
+struct DwParams {
+  const uint8_t* xt;      // [dq][Np], offset to the panel's first column   A side (rows j)
+  const uint8_t* ghat_t;  // [Vp][P]                                         B side (rows v)
+  float* dwacc;           // [dq][Vp] fp32
+  int64_t Np, P, Vp;
+  int RT, CT, KT, accumulate;
+};
+
+__global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  int rt, ct;
+  if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
+  v16f acc[4][4];
+  mfma_mainloop(p.xt + (int64_t)rt * 256 * p.Np, p.Np, p.ghat_t + (int64_t)ct * 256 * p.P, p.P, p.KT, smem, acc);
+  const int jbase = rt * 256 + wa * 128 + 4 * (lane >> 5);
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int v = ct * 256 + wb * 128 + b * 32 + (lane & 31);
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int j = jbase + a * 32 + 8 * (r >> 2) + (r & 3);
+        float* dst = p.dwacc + (int64_t)j * p.Vp + v;
+        *dst = p.accumulate ? (*dst + acc[a][b][r]) : acc[a][b][r];
+      }
+    }
+  }
+}
+
+// sort keys: target (V for rows that take no part), value = row
+__global__ __launch_bounds__(256) void bwd_keys_kernel(const int64_t* __restrict__ targets, int64_t ignore_index, int N, int V,
+                                                      int32_t* __restrict__ keys, int32_t* __restrict__ vals) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= N) return;
+  const int64_t y = targets[i];
+  keys[i] = ((y != ignore_index) && y >= 0 && y < V) ? (int32_t)y : V;
+  vals[i] = i;
+}
+
+// segoff[v] = first sorted position whose key >= v, v = 0..V+1
+__global__ __launch_bounds__(256) void bwd_segoff_kernel(const int32_t* __restrict__ skeys, int N, int V,
+                                                        int32_t* __restrict__ segoff) {
+  const int pos = blockIdx.x * 256 + threadIdx.x;
+  if (pos > N) return;
+  const int k = (pos < N) ? skeys[pos] : V + 1;
+  const int kprev = (pos > 0) ? skeys[pos - 1] : -1;
+  for (int v = kprev + 1; v <= k; ++v) segoff[v] = pos;
+}
+
+constexpr int LONG_SEG = 64;
+
+// Columns that are the target of many rows: dwacc[:, v] -= sum_i h_i X_q[i, :] / xi, one
+// workgroup per column, rows split over 16 row-lanes and folded in a fixed order.
+__global__ __launch_bounds__(256) void bwd_dw_long_kernel(const int32_t* __restrict__ segoff, const int32_t* __restrict__ perm,
+                                                         const float* __restrict__ hcoef, const uint8_t* __restrict__ xq,
+                                                         int64_t dp, int64_t dq, int64_t Vp, const float* __restrict__ xi,
+                                                         float* __restrict__ dwacc) {
+  __shared__ float red[16][256];
+  const int v = blockIdx.x;
+  const int s0 = segoff[v], L = segoff[v + 1] - s0;
+  if (L < LONG_SEG) return;
+  const int t = threadIdx.x, c = t & 15, rl = t >> 4;
+  const float inv_xi = 1.0f / xi[0];
+  for (int64_t jb = 0; jb < dq; jb += 256) {
+    float a[16];
+#pragma unroll
+    for (int m = 0; m < 16; ++m) a[m] = 0.f;
+    if (jb + c * 16 < dp) {
+      for (int n = rl; n < L; n += 16) {
+        const int i = perm[s0 + n];
+        const float h = hcoef[i];
+        const v4i raw = *reinterpret_cast<const v4i*>(xq + (int64_t)i * dp + jb + c * 16);
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          const uint32_t w = (uint32_t)raw[m];
+          a[4 * m + 0] = fmaf(h, e4m3_to_float<0>(w), a[4 * m + 0]);
+          a[4 * m + 1] = fmaf(h, e4m3_to_float<1>(w), a[4 * m + 1]);
+          a[4 * m + 2] = fmaf(h, e4m3_to_float<2>(w), a[4 * m + 2]);
+          a[4 * m + 3] = fmaf(h, e4m3_to_float<3>(w), a[4 * m + 3]);
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int m = 0; m < 16; ++m) red[rl][c * 16 + m] = a[m];
+    __syncthreads();
+    float sfold = 0.f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) sfold += red[k][t];
+    float* dst = dwacc + (jb + t) * Vp + v;
+    *dst -= sfold * inv_xi;
+  }
+}
+
+// dW = x_s * ( xi * dwacc - sum over the (short) target segment of h_i X_q[i, :] ), cast to the
+// output type.  A thread owns one column v and 16 consecutive rows j.
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restrict__ dwacc, int64_t Vp, const int32_t* __restrict__ segoff,
+                                                          const int32_t* __restrict__ perm, const float* __restrict__ hcoef,
+                                                          const uint8_t* __restrict__ xq, int64_t dp, const float* __restrict__ xi,
+                                                          float x_s, int d, int V, T* __restrict__ dw, int64_t dw_ld) {
+  const int t = threadIdx.x;
+  const int v = blockIdx.x * 64 + (t & 63);
+  const int j0 = blockIdx.y * 64 + (t >> 6) * 16;
+  if (v >= V || j0 >= d) return;
+  const float scale = x_s * xi[0];
+  float o[16];
+#pragma unroll
+  for (int m = 0; m < 16; ++m) o[m] = dwacc[(int64_t)(j0 + m) * Vp + v] * scale;
+  const int s0 = segoff[v], L = segoff[v + 1] - s0;
+  if (L > 0 && L < LONG_SEG) {
+    for (int n = 0; n < L; ++n) {
+      const int i = perm[s0 + n];
+      const float h = hcoef[i] * x_s;
+      const v4i raw = *reinterpret_cast<const v4i*>(xq + (int64_t)i * dp + j0);
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const uint32_t w = (uint32_t)raw[m];
+        o[4 * m + 0] -= h * e4m3_to_float<0>(w);
+        o[4 * m + 1] -= h * e4m3_to_float<1>(w);
+        o[4 * m + 2] -= h * e4m3_to_float<2>(w);
+        o[4 * m + 3] -= h * e4m3_to_float<3>(w);
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < 16; ++m)
+    if (j0 + m < d) Elem<T>::store(dw + (int64_t)(j0 + m) * dw_ld + v, o[m]);
+}
+
+}  // namespace sce
+
+// ==========================================================================================
+// host side: C ABI
+// ==========================================================================================
+namespace sce {
+int sort_pairs(void* tmp, size_t* tmp_bytes, const int32_t* kin, int32_t* kout, const int32_t* vin, int32_t* vout,
+               size_t n, int end_bit, hipStream_t stream);   // sce_sort.hip
+}
+
+using namespace sce;
+
+static thread_local char g_err[512] = "";
+
+static int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define HIP_TRY(expr)                                                                              \
+  do {                                                                                             \
+    hipError_t e_ = (expr);                                                                        \
+    if (e_ != hipSuccess) return fail(SCE_EHIP, "%s failed: %s", #expr, hipGetErrorString(e_));    \
+  } while (0)
+
+struct DeviceGuard {
+  int prev = -1;
+  bool ok = true;
+  explicit DeviceGuard(int dev) {
+    if (hipGetDevice(&prev) != hipSuccess) { ok = false; return; }
+    if (prev != dev && hipSetDevice(dev) != hipSuccess) ok = false;
+  }
+  ~DeviceGuard() { if (prev >= 0) (void)hipSetDevice(prev); }
+};
+
+static std::mutex g_mu;
+static int g_arch_ok[64];   // 0 unknown, 1 gfx950, -1 other
+
+static int check_device(int dev) {
+  if (dev < 0 || dev >= 64) return fail(SCE_EINVAL, "device %d out of range", dev);
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (g_arch_ok[dev] == 0) {
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    g_arch_ok[dev] = strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : -1;
+    if (g_arch_ok[dev] == 1) {
+      // the MFMA kernels hold two 72 KB stages in LDS
+      HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_recompute_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+    }
+  }
+  if (g_arch_ok[dev] != 1) return fail(SCE_EARCH, "device %d is not gfx950", dev);
+  return SCE_OK;
+}
+
+static int check_shape(const sce_shape* s) {
+  if (!s) return fail(SCE_EINVAL, "shape is NULL");
+  if (s->N <= 0 || s->d <= 0 || s->V <= 0) return fail(SCE_EINVAL, "N, d, V must be positive (got %lld, %lld, %lld)",
+                                                       (long long)s->N, (long long)s->d, (long long)s->V);
+  if (s->d % 16 != 0) return fail(SCE_EINVAL, "d = %lld must be a multiple of 16", (long long)s->d);
+  if (s->N >= (1ll << 31) - 512 || s->V >= (1ll << 31) - 512) return fail(SCE_EINVAL, "N and V must be below 2^31");
+  if (s->n_predict != 1) return fail(SCE_EINVAL, "n_predict = %d: only a single offset is built into the kernels", s->n_predict);
+  return SCE_OK;
+}
+
+static size_t sort_tmp_bytes(int64_t N, int64_t V) {
+  size_t bytes = 0;
+  int bits = 1;
+  while ((1ll << bits) <= V) ++bits;
+  (void)sce::sort_pairs(nullptr, &bytes, nullptr, nullptr, nullptr, nullptr, (size_t)N, bits, nullptr);
+  return bytes;
+}
+
+static BwdLayout bwd_layout(const SavedLayout& S, int64_t P) {
+  BwdLayout B;
+  B.P = P;
+  size_t o = 0;
+  auto take = [&](size_t bytes) { size_t r = o; o += (bytes + 255) / 256 * 256; return r; };
+  B.off_crow = take((size_t)S.Np * 4);
+  B.off_rho = take((size_t)S.Np * 4);
+  B.off_hcoef = take((size_t)S.Np * 4);
+  B.off_blockmax = take((size_t)(S.Np / 256) * 4);
+  B.off_xi = take(256);
+  B.off_xt = take((size_t)S.dq * S.Np);
+  B.off_dwacc = take((size_t)S.dq * S.Vp * 4);
+  B.off_perm = take((size_t)S.N * 4 * 2);      // sorted values + unsorted values
+  B.off_keys = take((size_t)S.N * 4 * 2);      // sorted keys + unsorted keys
+  B.off_segoff = take((size_t)(S.V + 2) * 4);
+  B.sorttmp_bytes = sort_tmp_bytes(S.N, S.V);
+  B.off_sorttmp = take(B.sorttmp_bytes);
+  B.fixed = o;
+  B.off_ghat = take((size_t)P * S.Vp);
+  B.off_ghat_t = take((size_t)S.Vp * P);
+  B.total = o;
+  return B;
+}
+
+static int64_t default_panel(const SavedLayout& S) { return S.Np < 8192 ? S.Np : 8192; }
+
+extern "C" int sce_version(void) { return SCE_VERSION; }
+extern "C" const char* sce_last_error(void) { return g_err; }
+
+extern "C" int sce_sizes_for(const sce_shape* shape, sce_sizes* out) {
+  if (int rc = check_shape(shape)) return rc;
+  if (!out) return fail(SCE_EINVAL, "out is NULL");
+  const SavedLayout S = saved_layout(shape->N, shape->d, shape->V, shape->n_predict);
+  out->saved_bytes = S.total;
+  out->fwd_workspace_bytes = (size_t)8 * S.Np * 16 + 256;
+  out->bwd_workspace_min_bytes = bwd_layout(S, 256).total;
+  out->bwd_panel_rows = default_panel(S);
+  out->bwd_workspace_bytes = bwd_layout(S, out->bwd_panel_rows).total;
+  return SCE_OK;
+}
+
+static int grid_for(size_t work_items, int per_block) {
+  size_t g = (work_items + per_block - 1) / per_block;
+  if (g > 65536 * 16) g = 65536 * 16;
+  if (g == 0) g = 1;
+  return (int)g;
+}
+
+extern "C" int sce_quantize_e4m3(const void* src, int32_t src_dtype, void* dst, float scale, size_t n, int32_t device,
+                                 void* stream) {
+  if (!src || !dst) return fail(SCE_EINVAL, "src/dst is NULL");
+  if (!(scale > 0.f)) return fail(SCE_EINVAL, "scale must be positive");
+  if (int rc = check_device(device)) return rc;
+  if (n == 0) return SCE_OK;
+  DeviceGuard guard(device);
+  if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", device);
+  hipStream_t st = (hipStream_t)stream;
+  const int grid = grid_for((n + 3) / 4, 256);
+  if (src_dtype == SCE_F32) quantize_flat_kernel<float><<<grid, 256, 0, st>>>((const float*)src, (uint8_t*)dst, n, scale);
+  else if (src_dtype == SCE_BF16) quantize_flat_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)src, (uint8_t*)dst, n, scale);
+  else return fail(SCE_EINVAL, "unsupported dtype %d", src_dtype);
+  HIP_TRY(hipGetLastError());
+  return SCE_OK;
+}
+
+extern "C" int sce_transpose_bytes(const void* src, void* dst, int64_t rows, int64_t cols, int32_t device, void* stream) {
+  if (!src || !dst) return fail(SCE_EINVAL, "src/dst is NULL");
+  if (rows <= 0 || cols <= 0) return fail(SCE_EINVAL, "rows and cols must be positive");
+  if ((rows + 63) / 64 > 65535) return fail(SCE_EINVAL, "too many rows (%lld)", (long long)rows);
+  if (int rc = check_device(device)) return rc;
+  DeviceGuard guard(device);
+  if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", device);
+  dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
+  transpose_bytes_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint8_t*)src, (uint8_t*)dst, rows, cols);
+  HIP_TRY(hipGetLastError());
+  return SCE_OK;
+}
+
+static int check_common(const sce_args* a) {
+  if (!a) return fail(SCE_EINVAL, "args is NULL");
+  if (a->struct_size != sizeof(sce_args)) return fail(SCE_EINVAL, "struct_size %u != %zu (ABI mismatch)", a->struct_size, sizeof(sce_args));
+  if (int rc = check_shape(&a->shape)) return rc;
+  if (!a->targets) return fail(SCE_EINVAL, "targets is NULL");
+  if (!(a->cap > 0.f) || a->cap > 40.f) return fail(SCE_EINVAL, "cap = %g must be in (0, 40]", (double)a->cap);
+  if (!(a->x_s > 0.f) || !(a->w_s > 0.f)) return fail(SCE_EINVAL, "x_s and w_s must be positive");
+  if (a->reduction != SCE_REDUCE_NONE && a->reduction != SCE_REDUCE_MEAN) return fail(SCE_EINVAL, "bad reduction %d", a->reduction);
+  if (!a->saved) return fail(SCE_EINVAL, "saved is NULL");
+  if (((uintptr_t)a->saved & 255) || ((uintptr_t)a->workspace & 255)) return fail(SCE_EINVAL, "saved and workspace must be 256-byte aligned");
+  return check_device(a->device);
+}
+
+extern "C" int sce_forward(const sce_args* a) {
+  if (int rc = check_common(a)) return rc;
+  const int64_t N = a->shape.N, d = a->shape.d, V = a->shape.V;
+  if (!a->x || !a->w) return fail(SCE_EINVAL, "x or w is NULL");
+  if (a->x_ld < d || a->w_ld < V) return fail(SCE_EINVAL, "row strides smaller than the row length");
+  if (a->reduction == SCE_REDUCE_NONE && !a->losses) return fail(SCE_EINVAL, "losses is NULL with reduction = none");
+  if (a->reduction == SCE_REDUCE_MEAN && !a->loss) return fail(SCE_EINVAL, "loss is NULL with reduction = mean");
+  const SavedLayout S = saved_layout(N, d, V, a->shape.n_predict);
+  if (a->saved_bytes < S.total) return fail(SCE_EINVAL, "saved buffer too small: %zu < %zu", a->saved_bytes, S.total);
+  const int RT = (int)(S.Np / 256), CT = (int)(S.Vp / 256);
+  const int nsplit = CT < 8 ? CT : 8;
+  const size_t need_ws = (size_t)nsplit * S.Np * 16;
+  if (!a->workspace || a->workspace_bytes < need_ws) return fail(SCE_EINVAL, "forward workspace too small: %zu < %zu", a->workspace_bytes, need_ws);
+  DeviceGuard guard(a->device);
+  if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", a->device);
+  hipStream_t st = (hipStream_t)a->stream;
+  uint8_t* sv = (uint8_t*)a->saved;
+  uint8_t* xq = sv + S.off_xq;
+  uint8_t* wqt = sv + S.off_wqt;
+  uint8_t* wq = sv + S.off_wq;
+
+  {
+    const int grid = grid_for((size_t)S.Np * (S.dp / 16), 256);
+    if (a->x_dtype == SCE_F32)
+      quantize_pad_kernel<float><<<grid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, a->x_s);
+    else if (a->x_dtype == SCE_BF16)
+      quantize_pad_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, a->x_s);
+    else return fail(SCE_EINVAL, "unsupported x dtype %d", a->x_dtype);
+    dim3 gw((unsigned)(S.Vp / 64), (unsigned)(S.dq / 64));
+    if (a->w_dtype == SCE_F32)
+      quantize_w_kernel<float><<<gw, 256, 0, st>>>((const float*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.Vp, a->w_s);
+    else if (a->w_dtype == SCE_BF16)
+      quantize_w_kernel<bf16_t><<<gw, 256, 0, st>>>((const bf16_t*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.Vp, a->w_s);
+    else return fail(SCE_EINVAL, "unsupported w dtype %d", a->w_dtype);
+  }
+  FwdParams p;
+  p.xq = xq; p.wqt = wqt; p.targets = a->targets; p.partials = (float4*)a->workspace;
+  p.dp = S.dp; p.N = (int)N; p.V = (int)V; p.Np = (int)S.Np; p.RT = RT; p.CT = CT; p.S = nsplit;
+  p.sc = a->x_s * a->w_s; p.c1 = 2.0f * LOG2E / a->cap; p.c2 = -2.0f * a->cap * LOG2E; p.cap = a->cap;
+  const int grid = 8 * nsplit * ((RT + 7) / 8);
+  fwd_kernel<<<grid, NTHREADS, SMEM_BYTES, st>>>(p);
+  float* s_lse = (float*)(sv + S.off_lse);
+  float* s_umax = (float*)(sv + S.off_umax);
+  float* s_zy = (float*)(sv + S.off_zy);
+  fwd_combine_kernel<<<(int)(S.Np / 256), 256, 0, st>>>(p.partials, nsplit, (int)N, (int)S.Np, (int)V, a->targets, a->ignore_index,
+                                                       a->cap, s_lse, s_umax, s_zy, a->losses, a->lse, a->argmax);
+  fwd_reduce_kernel<<<1, 1024, 0, st>>>(s_lse, s_zy, a->targets, a->ignore_index, (int)N, (int)V, (int32_t*)(sv + S.off_hdr),
+                                        a->reduction == SCE_REDUCE_MEAN ? a->loss : nullptr, a->n_valid);
+  HIP_TRY(hipGetLastError());
+  return SCE_OK;
+}
+
+extern "C" int sce_backward(const sce_args* a) {
+  if (int rc = check_common(a)) return rc;
+  const int64_t N = a->shape.N, d = a->shape.d, V = a->shape.V;
+  if (!a->grad_output) return fail(SCE_EINVAL, "grad_output is NULL");
+  if (!a->dx || !a->dw) return fail(SCE_EINVAL, "dx or dw is NULL");
+  if (a->dx_ld < d || a->dw_ld < V) return fail(SCE_EINVAL, "row strides smaller than the row length");
+  if ((a->dx_dtype != SCE_F32 && a->dx_dtype != SCE_BF16) || (a->dw_dtype != SCE_F32 && a->dw_dtype != SCE_BF16))
+    return fail(SCE_EINVAL, "unsupported gradient dtype");
+  const SavedLayout S = saved_layout(N, d, V, a->shape.n_predict);
+  if (a->saved_bytes < S.total) return fail(SCE_EINVAL, "saved buffer too small: %zu < %zu", a->saved_bytes, S.total);
+  if (!a->workspace) return fail(SCE_EINVAL, "workspace is NULL");
+  const BwdLayout Bmin = bwd_layout(S, 256);
+  if (a->workspace_bytes < Bmin.total) return fail(SCE_EINVAL, "backward workspace too small: %zu < %zu", a->workspace_bytes, Bmin.total);
+  int64_t P = (int64_t)((a->workspace_bytes - Bmin.fixed) / (2 * (size_t)S.Vp)) / 256 * 256;
+  if (P > S.Np) P = S.Np;
+  if (a->panel_rows > 0) {
+    if (a->panel_rows % 256) return fail(SCE_EINVAL, "panel_rows must be a multiple of 256");
+    if (a->panel_rows < P) P = a->panel_rows;
+  }
+  if (P < 256) return fail(SCE_EINVAL, "backward workspace too small for one 256-row panel");
+  const BwdLayout B = bwd_layout(S, P);
+  if (B.total > a->workspace_bytes) return fail(SCE_EINVAL, "internal: panel layout exceeds workspace");
+  DeviceGuard guard(a->device);
+  if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", a->device);
+  hipStream_t st = (hipStream_t)a->stream;
+  uint8_t* sv = (uint8_t*)a->saved;
+  uint8_t* ws = (uint8_t*)a->workspace;
+  const uint8_t* xq = sv + S.off_xq;
+  const uint8_t* wqt = sv + S.off_wqt;
+  const uint8_t* wq = sv + S.off_wq;
+  const float* s_lse = (const float*)(sv + S.off_lse);
+  const float* s_umax = (const float*)(sv + S.off_umax);
+  const float* s_zy = (const float*)(sv + S.off_zy);
+  const int32_t* hdr = (const int32_t*)(sv + S.off_hdr);
+  float* crow = (float*)(ws + B.off_crow);
+  float* rho = (float*)(ws + B.off_rho);
+  float* hcoef = (float*)(ws + B.off_hcoef);
+  float* blockmax = (float*)(ws + B.off_blockmax);
+  float* xi = (float*)(ws + B.off_xi);
+  uint8_t* xt = ws + B.off_xt;
+  float* dwacc = (float*)(ws + B.off_dwacc);
+  int32_t* perm = (int32_t*)(ws + B.off_perm);
+  int32_t* vals_in = perm + N;
+  int32_t* skeys = (int32_t*)(ws + B.off_keys);
+  int32_t* keys_in = skeys + N;
+  int32_t* segoff = (int32_t*)(ws + B.off_segoff);
+  uint8_t* ghat = ws + B.off_ghat;
+  uint8_t* ghat_t = ws + B.off_ghat_t;
+
+  const int nblk = (int)(S.Np / 256);
+  bwd_prep_kernel<<<nblk, 256, 0, st>>>(s_lse, s_umax, s_zy, a->targets, a->ignore_index, hdr, a->grad_output,
+                                        a->reduction == SCE_REDUCE_NONE ? 1 : 0, a->grad_scale, a->cap, (int)N, (int)S.Np, (int)V,
+                                        crow, rho, hcoef, blockmax);
+  bwd_xi_kernel<<<1, 1024, 0, st>>>(blockmax, nblk, xi);
+  {
+    dim3 g((unsigned)(S.Np / 64), (unsigned)(S.dq / 64));
+    bwd_xt_kernel<<<g, 256, 0, st>>>(xq, S.dp, S.Np, rho, xi, xt);
+  }
+  // rows grouped by target, for the one-hot part of dW
+  {
+    bwd_keys_kernel<<<(int)((N + 255) / 256), 256, 0, st>>>(a->targets, a->ignore_index, (int)N, (int)V, keys_in, vals_in);
+    int bits = 1;
+    while ((1ll << bits) <= V) ++bits;
+    size_t tmp = B.sorttmp_bytes;
+    if (sce::sort_pairs(ws + B.off_sorttmp, &tmp, keys_in, skeys, vals_in, perm, (size_t)N, bits, st) != 0)
+      return fail(SCE_EHIP, "radix sort of the targets failed");
+    bwd_segoff_kernel<<<(int)((N + 256) / 256), 256, 0, st>>>(skeys, (int)N, (int)V, segoff);
+  }
+  const float sc = a->x_s * a->w_s, c1 = 2.0f * LOG2E / a->cap, c2 = -2.0f * a->cap * LOG2E;
+  const int CTv = (int)(S.Vp / 256), CTd = (int)(S.dq / 256);
+  int first = 1;
+  for (int64_t p0 = 0; p0 < S.Np; p0 += P) {
+    const int64_t prow = (S.Np - p0 < P) ? (S.Np - p0) : P;     // multiple of 256
+    const int RTp = (int)(prow / 256);
+    RecomputeParams rp;
+    rp.xq = xq + p0 * S.dp; rp.wqt = wqt; rp.crow = crow + p0; rp.ghat = ghat; rp.ghat_t = ghat_t;
+    rp.dp = S.dp; rp.Vp = S.Vp; rp.P = P; rp.RT = RTp; rp.CT = CTv; rp.V = (int)V; rp.sc = sc; rp.c1 = c1; rp.c2 = c2;
+    bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_BYTES, st>>>(rp);
+
+    DxParams dp_;
+    dp_.wq = wq; dp_.ghat = ghat; dp_.wqt = wqt; dp_.rho = rho + p0; dp_.hcoef = hcoef + p0; dp_.targets = a->targets + p0;
+    dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.dp = S.dp; dp_.RT = RTp; dp_.CT = CTd;
+    dp_.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); dp_.d = (int)d; dp_.V = (int)V; dp_.w_s = a->w_s;
+    if (a->dx_dtype == SCE_F32) {
+      dp_.dx = (float*)a->dx + p0 * a->dx_ld;
+      bwd_dx_kernel<float><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_BYTES, st>>>(dp_);
+    } else {
+      dp_.dx = (bf16_t*)a->dx + p0 * a->dx_ld;
+      bwd_dx_kernel<bf16_t><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_BYTES, st>>>(dp_);
+    }
+
+    DwParams wp;
+    wp.xt = xt + p0; wp.ghat_t = ghat_t; wp.dwacc = dwacc; wp.Np = S.Np; wp.P = P; wp.Vp = S.Vp;
+    wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(prow / BK); wp.accumulate = first ? 0 : 1;
+    bwd_dw_kernel<<<map_tile_grid(CTd, CTv), NTHREADS, SMEM_BYTES, st>>>(wp);
+    first = 0;
+  }
+  bwd_dw_long_kernel<<<(int)V, 256, 0, st>>>(segoff, perm, hcoef, xq, S.dp, S.dq, S.Vp, xi, dwacc);
+  {
+    dim3 g((unsigned)((V + 63) / 64), (unsigned)((d + 63) / 64));
+    if (a->dw_dtype == SCE_F32)
+      bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, S.Vp, segoff, perm, hcoef, xq, S.dp, xi, a->x_s, (int)d, (int)V,
+                                                   (float*)a->dw, a->dw_ld);
+    else
+      bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, S.Vp, segoff, perm, hcoef, xq, S.dp, xi, a->x_s, (int)d, (int)V,
+                                                    (bf16_t*)a->dw, a->dw_ld);
+  }
+  HIP_TRY(hipGetLastError());
+  return SCE_OK;
+}

@@ -1,0 +1,181 @@
+"""Drop-in for the reference's ``tiny/cuda_kernels.py`` on MI355X.
+
+Exports the same names the trainer imports (tiny/train.py:47):
+
+    from cuda_kernels import CE_KERNEL_VOCAB_SIZE, FusedSoftcappedCrossEntropy
+
+``FusedSoftcappedCrossEntropy.apply(x, targets, mtp_weights, lm_head_weight, x_s,
+w_s, grad_s, grad_scale[, cap])`` keeps the positional signature of
+tiny/cuda_kernels.py:338 and returns the per-row losses (N,), which the caller
+reduces with ``.mean()`` (tiny/train.py:1417).  Underneath, the work is done by the
+HIP kernels of libslowrun_ce.so through its C ABI; the N x V logits are never
+stored, and nothing N x V sized is kept for backward.
+
+Differences from the reference that a caller can see:
+  * V is a runtime size (CE_KERNEL_VOCAB_SIZE is kept only for the trainer's asserts);
+  * ``reduction='mean'`` is available (mean over rows whose target is not -1, like
+    F.cross_entropy(ignore_index=-1) in the eager head, tiny/train.py:743);
+  * rows with target -1 give loss 0 and zero gradient;
+  * ``grad_s`` is accepted and unused: the reference needs it to fit dlogits into
+    e5m2 (tiny/cuda_kernels.py:265); here each row of the on-chip dlogits carries its
+    own scale;
+  * dW is returned in the weight's dtype and uses the upstream gradient of every row,
+    not its mean (tiny/cuda_kernels.py:412 assumes it is uniform).
+"""
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._lib import SceArgs, SceShape
+
+CE_KERNEL_VOCAB_SIZE = 50304          # tiny/cuda_kernels.py:82
+IGNORE_INDEX = -1                     # tiny/train.py:743
+
+_DTYPES = {torch.float32: _lib.SCE_F32, torch.bfloat16: _lib.SCE_BF16}
+
+
+def _scale_value(s, like):
+    """Python float, or a 0-dim tensor.  torch casts a 0-dim tensor operand to the
+    dtype of the tensor it divides, so the same rounding is applied here."""
+    if isinstance(s, torch.Tensor):
+        return float(s.detach().to(like.dtype))
+    return float(s)
+
+
+def _dtype_code(t, what):
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError(f"{what} must be float32 or bfloat16, got {t.dtype}") from None
+
+
+def _stream_ptr(device):
+    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _base_args(x_like, N, d, V, x_s, w_s, cap, grad_scale, reduction, targets):
+    a = SceArgs()
+    a.struct_size = C.sizeof(SceArgs)
+    a.device = x_like.device.index if x_like.device.index is not None else torch.cuda.current_device()
+    a.stream = _stream_ptr(x_like.device)
+    a.shape = SceShape(N, d, V, 1, 0)
+    a.targets = targets.data_ptr()
+    a.mtp_weights = None
+    a.x_s, a.w_s, a.cap, a.grad_scale = x_s, w_s, cap, grad_scale
+    a.ignore_index = IGNORE_INDEX
+    a.reduction = _lib.SCE_REDUCE_MEAN if reduction == "mean" else _lib.SCE_REDUCE_NONE
+    return a
+
+
+def _check_inputs(x, w, targets):
+    if not x.is_cuda:
+        raise RuntimeError("FusedSoftcappedCrossEntropy runs on an MI355X GPU only; got a CPU tensor")
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[0]:
+        raise ValueError(f"expected x (N, d) and lm_head_weight (d, V), got {tuple(x.shape)} and {tuple(w.shape)}")
+    if targets.dim() != 1 or targets.shape[0] != x.shape[0] or targets.dtype != torch.int64:
+        raise ValueError("targets must be int64 of shape (N,)")
+
+
+def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False):
+    """One call of sce_forward.  Returns (out, saved, lse, argmax, n_valid)."""
+    _check_inputs(x, w, targets)
+    x = x if x.stride(1) == 1 else x.contiguous()
+    w = w if w.stride(1) == 1 else w.contiguous()
+    targets = targets.contiguous()
+    N, d = x.shape
+    V = w.shape[1]
+    dev = x.device
+    sz = _lib.sizes_for(N, d, V)
+    saved = torch.empty(sz.saved_bytes, dtype=torch.uint8, device=dev)
+    ws = torch.empty(sz.fwd_workspace_bytes, dtype=torch.uint8, device=dev)
+    losses = torch.empty(N, dtype=torch.float32, device=dev)
+    lse = torch.empty(N, dtype=torch.float32, device=dev)
+    loss = torch.empty(1, dtype=torch.float32, device=dev)
+    n_valid = torch.empty(2, dtype=torch.int32, device=dev)
+    argmax = torch.empty(N, dtype=torch.int32, device=dev) if want_argmax else None
+    a = _base_args(x, N, d, V, x_s, w_s, cap, 1.0, reduction, targets)
+    a.x, a.x_dtype, a.x_ld = x.data_ptr(), _dtype_code(x, "x"), x.stride(0)
+    a.w, a.w_dtype, a.w_ld = w.data_ptr(), _dtype_code(w, "lm_head_weight"), w.stride(0)
+    a.loss, a.losses, a.lse, a.n_valid = loss.data_ptr(), losses.data_ptr(), lse.data_ptr(), n_valid.data_ptr()
+    a.argmax = argmax.data_ptr() if want_argmax else None
+    a.saved, a.saved_bytes = saved.data_ptr(), saved.numel()
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    _lib.check(_lib.lib().sce_forward(C.byref(a)), "sce_forward")
+    out = loss.reshape(()) if reduction == "mean" else losses
+    return out, saved, lse, argmax, n_valid
+
+
+def ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale, reduction, x_dtype, w_dtype,
+                panel_rows=0, workspace_bytes=None):
+    """One call of sce_backward.  Returns (dx (N,d) in x_dtype, dw (d,V) in w_dtype)."""
+    dev = saved.device
+    sz = _lib.sizes_for(N, d, V)
+    nbytes = sz.bwd_workspace_bytes if workspace_bytes is None else workspace_bytes
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    dx = torch.empty(N, d, dtype=x_dtype, device=dev)
+    dw = torch.empty(d, V, dtype=w_dtype, device=dev)
+    go = grad_output.detach().to(torch.float32).contiguous().reshape(-1)
+    if reduction == "mean":
+        if go.numel() != 1:
+            raise ValueError("grad_output must be a scalar for reduction='mean'")
+    elif go.numel() != N:
+        raise ValueError("grad_output must have one element per row for reduction='none'")
+    a = _base_args(saved, N, d, V, x_s, w_s, cap, grad_scale, reduction, targets)
+    a.saved, a.saved_bytes = saved.data_ptr(), saved.numel()
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    a.grad_output = go.data_ptr()
+    a.dx, a.dx_dtype, a.dx_ld = dx.data_ptr(), _DTYPES[x_dtype], d
+    a.dw, a.dw_dtype, a.dw_ld = dw.data_ptr(), _DTYPES[w_dtype], V
+    a.panel_rows = panel_rows
+    _lib.check(_lib.lib().sce_backward(C.byref(a)), "sce_backward")
+    return dx, dw
+
+
+class FusedSoftcappedCrossEntropy(torch.autograd.Function):
+    """Same call as tiny/cuda_kernels.py:336-414; see the module docstring."""
+
+    @staticmethod
+    def forward(ctx, x, targets, mtp_weights, lm_head_weight, x_s, w_s, grad_s, grad_scale, cap=15.0, reduction="none"):
+        if mtp_weights is not None and mtp_weights.numel() != 1:
+            raise NotImplementedError("multi-token prediction (more than one offset) is not built into the kernels yet")
+        if reduction not in ("none", "mean"):
+            raise ValueError("reduction must be 'none' or 'mean'")
+        w0 = 1.0 if mtp_weights is None else float(mtp_weights.reshape(-1)[0])
+        xs, ws_ = _scale_value(x_s, x), _scale_value(w_s, lm_head_weight)
+        out, saved, _lse, _am, _nv = ce_forward(x.detach(), lm_head_weight.detach(), targets, xs, ws_, float(cap), reduction)
+        ctx.save_for_backward(saved, targets)
+        ctx.params = (x.shape[0], x.shape[1], lm_head_weight.shape[1], xs, ws_, float(cap), float(grad_scale) * w0,
+                      reduction, x.dtype, lm_head_weight.dtype)
+        return out * w0 if w0 != 1.0 else out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        saved, targets = ctx.saved_tensors
+        N, d, V, xs, ws_, cap, gscale, reduction, x_dtype, w_dtype = ctx.params
+        dx, dw = ce_backward(saved, targets, grad_output, N, d, V, xs, ws_, cap, gscale, reduction, x_dtype, w_dtype)
+        return dx, None, None, dw, None, None, None, None, None, None
+
+
+def quantize_e4m3(t, scale):
+    """``t.div(scale).to(torch.float8_e4m3fn)`` (tiny/cuda_kernels.py:340-341) on the HIP quantiser."""
+    if not t.is_cuda:
+        raise RuntimeError("quantize_e4m3 needs a GPU tensor")
+    t = t.contiguous()
+    out = torch.empty(t.shape, dtype=torch.uint8, device=t.device)
+    _lib.check(_lib.lib().sce_quantize_e4m3(t.data_ptr(), _dtype_code(t, "t"), out.data_ptr(), _scale_value(scale, t),
+                                           t.numel(), t.device.index, _stream_ptr(t.device)), "sce_quantize_e4m3")
+    return out.view(torch.float8_e4m3fn)
+
+
+def transpose_copy(src, dst):
+    """dst = src.T for one-byte element types (tiny/cuda_kernels.py:56-78)."""
+    assert src.ndim == 2 and dst.ndim == 2
+    M, Nn = src.shape
+    assert dst.shape == (Nn, M), f"Expected dst shape ({Nn}, {M}), got {dst.shape}"
+    if src.element_size() != 1 or dst.element_size() != 1:
+        raise TypeError("transpose_copy handles one-byte element types (fp8)")
+    if not (src.is_contiguous() and dst.is_contiguous()):
+        raise ValueError("transpose_copy needs contiguous tensors")
+    _lib.check(_lib.lib().sce_transpose_bytes(src.data_ptr(), dst.data_ptr(), M, Nn, src.device.index,
+                                             _stream_ptr(src.device)), "sce_transpose_bytes")

@@ -1,0 +1,77 @@
+"""Shared helpers for the GPU parity tests: run the HIP path and the oracle on the
+same inputs and compare to the tolerances the task states."""
+import torch
+
+from oracle import eager
+
+LOSS_RTOL = 1e-3          # loss: relative error
+GRAD_MAXREL = 2e-2        # dX, dW: max |delta| / max |ref|
+GRAD_COS = 0.9995         # dX, dW: cosine similarity
+
+
+def maxrel(a, b):
+    return float((a.double() - b.double()).abs().max() / b.double().abs().max().clamp_min(1e-300))
+
+
+def cosine(a, b):
+    a, b = a.double().flatten(), b.double().flatten()
+    return float((a @ b) / (a.norm() * b.norm()).clamp_min(1e-300))
+
+
+def run_ours(inp, reduction="mean", x_dtype=torch.bfloat16, w_dtype=torch.bfloat16, grad_output=None, device="cuda",
+             want_argmax=True, panel_rows=0):
+    from slowrun_amd import cuda_kernels as ck
+    x = inp.x.to(device=device, dtype=x_dtype)
+    w = inp.w.to(device=device, dtype=w_dtype)
+    y = inp.targets.to(device)
+    N, d = x.shape
+    V = w.shape[1]
+    out, saved, lse, argmax, n_valid = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, reduction, want_argmax=want_argmax)
+    if grad_output is None:
+        grad_output = torch.ones((), device=device) if reduction == "mean" else torch.full((N,), 1.0 / N, device=device)
+    dx, dw = ck.ce_backward(saved, y, grad_output, N, d, V, inp.x_s, inp.w_s, inp.cap, 1.0, reduction, x_dtype, w_dtype,
+                            panel_rows=panel_rows)
+    torch.cuda.synchronize()
+    return dict(loss=out, lse=lse, argmax=argmax, n_valid=n_valid, dx=dx, dw=dw, x=x, w=w, y=y)
+
+
+def run_oracle(inp, ours, reduction="mean", grad_output=None, row_chunk=4096):
+    """Oracle on the same device and on the very tensors handed to the HIP path
+    (already cast to bf16 if that is what it got)."""
+    go = grad_output
+    if reduction == "mean" and go is not None:
+        go = float(go)
+    return eager.softcapped_ce(ours["x"], ours["w"], ours["y"], inp.x_s, inp.w_s, cap=inp.cap, reduction=reduction,
+                               grad_output=go, row_chunk=row_chunk)
+
+
+def check_parity(ours, ref, reduction="mean", check_argmax=True):
+    report = {}
+    lo, lr = ours["loss"].float(), ref["loss"].float()
+    if reduction == "mean":
+        rel = abs(float(lo) - float(lr)) / abs(float(lr))
+    else:
+        rel = float((lo - lr).abs().max() / lr.abs().max())
+    report["loss_rel"] = rel
+    assert rel <= LOSS_RTOL, f"loss rel err {rel}"
+    lse_err = float((ours["lse"] - ref["lse"]).abs().max())
+    report["lse_abs"] = lse_err
+    assert lse_err <= 1e-3 * float(ref["lse"].abs().max()), f"lse err {lse_err}"
+    for k in ("dx", "dw"):
+        mr, cs = maxrel(ours[k].float(), ref[k]), cosine(ours[k].float(), ref[k])
+        report[k + "_maxrel"], report[k + "_cos"] = mr, cs
+        assert mr <= GRAD_MAXREL, f"{k} max-rel {mr}"
+        assert cs > GRAD_COS, f"{k} cosine {cs}"
+    # ignore handling, bit exact: ignored rows have zero loss and zero dX rows
+    ign = ours["y"] == -1
+    report["n_ignored"] = int(ign.sum())
+    assert int(ours["n_valid"][0]) == int((~ign).sum()) == ref["n_valid"]
+    if ign.any():
+        assert float(ours["dx"][ign].float().abs().max()) == 0.0
+        if reduction == "none":
+            assert float(ours["loss"][ign].abs().max()) == 0.0
+    if check_argmax and ours["argmax"] is not None:
+        mism = ours["argmax"].long() != ref["argmax"]
+        report["argmax_mismatch"] = int(mism.sum())
+        assert report["argmax_mismatch"] == 0, f"{report['argmax_mismatch']} argmax mismatches"
+    return report

@@ -1,0 +1,99 @@
+"""GPU parity of the HIP path against the oracle on small and ragged shapes,
+through the C ABI (slowrun_amd.cuda_kernels -> libslowrun_ce.so)."""
+import pytest
+import torch
+
+from slowrun_amd import configs
+from tests import parity_util as pu
+
+pytestmark = pytest.mark.gpu
+
+
+def _small(name, N, d, V):
+    return configs.make_inputs(name, N=N, d=d, V=V)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_quantize_matches_torch_cast_bit_exact(dtype):
+    from slowrun_amd import cuda_kernels as ck
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn(1 << 20, generator=g) * 3).to(dtype).cuda()
+    x[:8] = torch.tensor([448., 449., 464., 465., 1e4, -1e4, 2.0 ** -10, 0.0], dtype=dtype)
+    for s in (100 / 448, 1.6 / 448, 0.0123, 1.0):
+        ours = ck.quantize_e4m3(x, s).view(torch.uint8)
+        ref = x.div(s).to(torch.float8_e4m3fn).view(torch.uint8)      # tiny/cuda_kernels.py:340
+        assert torch.equal(ours, ref), f"scale {s}: {(ours != ref).sum().item()} bytes differ"
+
+
+def test_transpose_copy():
+    from slowrun_amd import cuda_kernels as ck
+    src = torch.randint(0, 255, (1000, 333), dtype=torch.uint8, device="cuda").view(torch.float8_e4m3fn)
+    dst = torch.empty(333, 1000, dtype=torch.float8_e4m3fn, device="cuda")
+    ck.transpose_copy(src, dst)
+    assert torch.equal(dst.view(torch.uint8), src.view(torch.uint8).T.contiguous())
+
+
+@pytest.mark.parametrize("N,d,V", [(256, 128, 256), (300, 128, 1000), (1000, 80, 777), (513, 272, 2049), (64, 16, 50304)])
+@pytest.mark.parametrize("reduction", ["mean", "none"])
+def test_small_shapes(N, d, V, reduction):
+    inp = _small("tiny_track", N, d, V)
+    ours = pu.run_ours(inp, reduction)
+    ref = pu.run_oracle(inp, ours, reduction)
+    print(pu.check_parity(ours, ref, reduction))
+
+
+def test_small_fp32_inputs_and_ignored_rows():
+    inp = _small("irregular", 700, 128, 1500)
+    ours = pu.run_ours(inp, "mean", x_dtype=torch.float32, w_dtype=torch.float32)
+    ref = pu.run_oracle(inp, ours, "mean")
+    rep = pu.check_parity(ours, ref, "mean")
+    assert rep["n_ignored"] > 0
+    print(rep)
+
+
+def test_small_panels_and_upstream_gradient():
+    inp = _small("limited_2p7b", 1100, 256, 3000)
+    go = torch.rand(1100, generator=torch.Generator().manual_seed(9)).cuda() * 2e-3
+    ours = pu.run_ours(inp, "none", grad_output=go, panel_rows=256)
+    ref = pu.run_oracle(inp, ours, "none", grad_output=go)
+    print(pu.check_parity(ours, ref, "none"))
+    ours2 = pu.run_ours(inp, "none", grad_output=go, panel_rows=0)
+    assert pu.maxrel(ours2["dw"].float(), ours["dw"].float()) < 1e-2
+    assert torch.equal(ours2["dx"], ours["dx"])
+
+
+def test_all_rows_ignored():
+    inp = _small("tiny_track", 300, 128, 512)
+    inp.targets[:] = -1
+    ours = pu.run_ours(inp, "mean")
+    assert torch.isnan(ours["loss"])
+    assert float(ours["dx"].float().abs().max()) == 0 and float(ours["dw"].float().abs().max()) == 0
+    assert int(ours["n_valid"][0]) == 0
+
+
+def test_out_of_range_targets_are_ignored_and_counted():
+    inp = _small("tiny_track", 300, 128, 512)
+    inp.targets[5] = 512
+    inp.targets[7] = -7
+    ours = pu.run_ours(inp, "none")
+    assert int(ours["n_valid"][1]) == 2 and int(ours["n_valid"][0]) == 298
+    assert float(ours["loss"][5]) == 0 and float(ours["loss"][7]) == 0
+    assert float(ours["dx"][5].float().abs().max()) == 0
+
+
+def test_autograd_function_signature():
+    from slowrun_amd.cuda_kernels import CE_KERNEL_VOCAB_SIZE, FusedSoftcappedCrossEntropy
+    assert CE_KERNEL_VOCAB_SIZE == 50304
+    inp = _small("tiny_track", 512, 128, 1024)
+    x = inp.x.cuda().bfloat16().requires_grad_(True)
+    w = inp.w.cuda().bfloat16().requires_grad_(True)
+    y = inp.targets.cuda()
+    # the trainer's call (tiny/train.py:694-696) and reduction (tiny/train.py:1417-1419)
+    losses = FusedSoftcappedCrossEntropy.apply(x, y, torch.tensor([1.0], device="cuda"), w, inp.x_s, inp.w_s, 0.75 / 448, 1.0)
+    assert losses.shape == (512,)
+    losses.mean().backward()
+    assert x.grad.shape == x.shape and w.grad.shape == w.shape and w.grad.dtype == torch.bfloat16
+    from oracle import eager
+    ref = eager.softcapped_ce(x.detach(), w.detach(), y, inp.x_s, inp.w_s, cap=15.0, reduction="none")
+    assert float((losses.detach() - ref["loss"]).abs().max() / ref["loss"].abs().max()) < 1e-3
+    assert pu.cosine(x.grad.float(), ref["dx"]) > pu.GRAD_COS and pu.cosine(w.grad.float(), ref["dw"]) > pu.GRAD_COS
