@@ -1,0 +1,139 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused fp8 LM-head + softcap + cross-entropy path on one MI355X.
+
+A step is one forward + backward of the loss head over one batch of synthetic
+input (resident in HBM before the timed region).  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload limited_2p7b]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0        # MI355X dense fp8 MFMA, published
+
+
+def cpu_baseline(inp, rows, threads):
+    """The eager reference path (oracle/eager.py) on the host cores, forward + backward,
+    on the first `rows` rows against the full W."""
+    import torch
+    from oracle import eager
+    torch.set_num_threads(threads)
+    x = inp.x[:rows].bfloat16()
+    w = inp.w.bfloat16()
+    y = inp.targets[:rows]
+    t0 = time.time()
+    eager.softcapped_ce(x, w, y, inp.x_s, inp.w_s, cap=inp.cap, reduction="mean", row_chunk=1024)
+    dt = time.time() - t0
+    return rows / dt, dt
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="limited_2p7b")
+    ap.add_argument("--rows", type=int, default=None, help="override N (debugging only; the result is then not the headline)")
+    ap.add_argument("--panel-rows", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-rows", type=int, default=2048)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (one process, one MI355X); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from slowrun_amd import _lib, configs
+    from slowrun_amd import cuda_kernels as ck
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    _lib.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    inp = configs.make_inputs(args.workload, N=args.rows)
+    N, d, V = inp.shape
+    x = inp.x.to(dev, torch.bfloat16)
+    w = inp.w.to(dev, torch.bfloat16)
+    y = inp.targets.to(dev)
+    go = torch.ones((), device=dev)
+
+    def step():
+        loss, saved, _lse, _am, _nv = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, "mean")
+        dx, dw = ck.ce_backward(saved, y, go, N, d, V, inp.x_s, inp.w_s, inp.cap, 1.0, "mean", torch.bfloat16, torch.bfloat16,
+                                panel_rows=args.panel_rows)
+        return loss, dx, dw
+
+    for _ in range(args.warmup):
+        out = step()
+    torch.cuda.synchronize()
+    _lib.timing_enable(True)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.time()
+    e0.record()
+    for _ in range(args.steps):
+        out = step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.time() - t0
+    ms_total = e0.elapsed_time(e1)
+    kt = _lib.timing_read()
+    _lib.timing_enable(False)
+    ms_per_step = ms_total / args.steps
+    loss = float(out[0])
+
+    flops_step = 6.0 * N * d * V                      # algorithmic: logits + dX + dW, no recompute
+    tokens_per_s = N / (ms_per_step * 1e-3)
+    # per-kernel achieved rate: algorithmic flops of the launches of that kind / their time
+    algo = {"fwd": 2.0 * N * d * V, "recompute": 2.0 * N * d * V, "dx": 2.0 * N * d * V, "dw": 2.0 * N * d * V}
+    kernels = {}
+    for k, (ms, n) in kt.items():
+        if n == 0:
+            continue
+        per_step_ms = ms / args.steps
+        ent = {"ms_per_step": round(per_step_ms, 4), "launches_per_step": n / args.steps, "avg_launch_ms": round(ms / n, 4)}
+        if k in algo:
+            ent["tflops"] = round(algo[k] / (per_step_ms * 1e-3) * 1e-12, 1)
+        kernels[k] = ent
+    dom = max((k for k in kernels if k in algo), key=lambda k: kernels[k]["ms_per_step"])
+    roofline = {
+        "bound": "mfma", "kernel": dom, "achieved": kernels[dom]["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(kernels[dom]["tflops"] / PEAK_FP8_TFLOPS, 4), "traffic": None,
+        "avg_launch_ms": kernels[dom]["avg_launch_ms"],
+    }
+    result = {
+        "metric": "fp8 lm-head+softcap CE fwd+bwd tokens/s at d=2560,V=50304; % fp8 MFMA peak",
+        "value": round(tokens_per_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3", "data": "synthetic",
+        "config": {"workload": f"{inp.name}: N={N}, d={d}, V={V}, cap={inp.cap}, fp8 e4m3 amax scales, bf16 dX/dW, mean reduction"},
+        "algorithmic_tflops": round(flops_step / (ms_per_step * 1e-3) * 1e-12, 1),
+        "frac_fp8_mfma_peak": round(flops_step / (ms_per_step * 1e-3) * 1e-12 / PEAK_FP8_TFLOPS, 4),
+        "hardware_flops_per_step": 8.0 * N * d * V,
+        "loss": loss,
+        "wall_s_timed_region": round(wall, 3),
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        threads = min(16, os.cpu_count() or 1)
+        rows = min(args.cpu_rows, N)
+        tps, dt = cpu_baseline(inp, rows, threads)
+        result["cpu_baseline"] = {
+            "value": round(tps, 1), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"eager fp8-quantise + fp32 matmul + softcap + F.cross_entropy fwd+bwd on the first {rows} rows "
+                      f"against the full (d,V) weight, {dt:.1f} s, torch {torch.__version__} with {threads} threads",
+        }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

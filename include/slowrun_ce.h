@@ -132,6 +132,29 @@ int sce_forward(const sce_args* args);
  * least bwd_workspace_min_bytes. */
 int sce_backward(const sce_args* args);
 
+/* ---- optional per-kernel timing (off by default) --------------------------------------
+ * No counterpart in the reference (it times whole steps with torch.cuda.synchronize,
+ * tiny/train.py:1408-1452).  While enabled, sce_forward / sce_backward record a HIP event
+ * pair on the caller's stream around each group of launches; sce_timing_read waits for the
+ * recorded events and returns the accumulated time and number of groups per kind. */
+enum {
+  SCE_K_QUANT = 0,       /* X and W quantisation                                             */
+  SCE_K_FWD = 1,         /* fused logits + softcap + online LSE (one launch per forward)     */
+  SCE_K_FWD_REDUCE = 2,  /* combine of the V-splits and the mean                             */
+  SCE_K_BWD_PREP = 3,    /* row scales, scaled X^T, rows grouped by target                   */
+  SCE_K_RECOMPUTE = 4,   /* logit recompute -> on-chip dlogits panel (one launch per panel)  */
+  SCE_K_DX = 5,          /* dX panel GEMM                                                    */
+  SCE_K_DW = 6,          /* dW panel GEMM                                                    */
+  SCE_K_DW_FINAL = 7,    /* one-hot part of dW, scaling, cast                                */
+  SCE_K_COUNT = 8
+};
+typedef struct sce_timing {
+  double ms[SCE_K_COUNT];
+  int64_t launches[SCE_K_COUNT];
+} sce_timing;
+int sce_timing_enable(int on);            /* also clears the accumulators */
+int sce_timing_read(sce_timing* out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -14,7 +14,9 @@ SCE_REDUCE_NONE, SCE_REDUCE_MEAN = 0, 1
 SCE_VERSION = 1
 
 EXPORTS = ("sce_version", "sce_last_error", "sce_sizes_for", "sce_quantize_e4m3", "sce_transpose_bytes",
-           "sce_forward", "sce_backward")
+           "sce_forward", "sce_backward", "sce_timing_enable", "sce_timing_read")
+
+KERNEL_KINDS = ("quantize", "fwd", "fwd_reduce", "bwd_prep", "recompute", "dx", "dw", "dw_final")
 
 
 class SceShape(C.Structure):
@@ -44,6 +46,10 @@ class SceArgs(C.Structure):
     ]
 
 
+class SceTiming(C.Structure):
+    _fields_ = [("ms", C.c_double * 8), ("launches", C.c_int64 * 8)]
+
+
 _LIB = None
 
 
@@ -63,6 +69,8 @@ def lib():
         L.sce_transpose_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int32, C.c_void_p]
         L.sce_forward.argtypes = [C.POINTER(SceArgs)]
         L.sce_backward.argtypes = [C.POINTER(SceArgs)]
+        L.sce_timing_enable.argtypes = [C.c_int]
+        L.sce_timing_read.argtypes = [C.POINTER(SceTiming)]
         if L.sce_version() != SCE_VERSION:
             raise RuntimeError(f"libslowrun_ce.so has ABI version {L.sce_version()}, expected {SCE_VERSION}")
         _LIB = L
@@ -80,3 +88,14 @@ def sizes_for(N, d, V, n_predict=1):
     out = SceSizes()
     check(lib().sce_sizes_for(C.byref(shape), C.byref(out)), "sce_sizes_for")
     return out
+
+
+def timing_enable(on):
+    check(lib().sce_timing_enable(1 if on else 0), "sce_timing_enable")
+
+
+def timing_read():
+    """{kind: (total_ms, launches)} accumulated since timing_enable(True)."""
+    t = SceTiming()
+    check(lib().sce_timing_read(C.byref(t)), "sce_timing_read")
+    return {k: (t.ms[i], t.launches[i]) for i, k in enumerate(KERNEL_KINDS)}

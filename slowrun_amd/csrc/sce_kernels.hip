@@ -23,6 +23,7 @@
 #include <stdio.h>
 #include <string.h>
 #include <mutex>
+#include <vector>
 
 namespace sce {
 
@@ -774,6 +775,44 @@ struct DeviceGuard {
 static std::mutex g_mu;
 static int g_arch_ok[64];   // 0 unknown, 1 gfx950, -1 other
 
+// Optional per-kernel timing with HIP events on the caller's stream (off by default).
+struct TimingState {
+  bool on = false;
+  std::vector<hipEvent_t> pool;                       // unused events
+  std::vector<hipEvent_t> begin[SCE_K_COUNT], end[SCE_K_COUNT];
+  double ms[SCE_K_COUNT] = {0};
+  int64_t launches[SCE_K_COUNT] = {0};
+};
+static TimingState g_timing;
+static std::mutex g_timing_mu;
+
+static hipEvent_t timing_event() {
+  if (!g_timing.pool.empty()) { hipEvent_t e = g_timing.pool.back(); g_timing.pool.pop_back(); return e; }
+  hipEvent_t e = nullptr;
+  (void)hipEventCreate(&e);
+  return e;
+}
+struct KernelTimer {   // records an event pair around the launches made while it lives
+  int kind; hipStream_t st; bool active;
+  KernelTimer(int k, hipStream_t s) : kind(k), st(s), active(false) {
+    std::lock_guard<std::mutex> lk(g_timing_mu);
+    if (!g_timing.on) return;
+    hipEvent_t e = timing_event();
+    if (!e) return;
+    (void)hipEventRecord(e, st);
+    g_timing.begin[kind].push_back(e);
+    active = true;
+  }
+  ~KernelTimer() {
+    if (!active) return;
+    std::lock_guard<std::mutex> lk(g_timing_mu);
+    hipEvent_t e = timing_event();
+    if (!e) { g_timing.pool.push_back(g_timing.begin[kind].back()); g_timing.begin[kind].pop_back(); return; }
+    (void)hipEventRecord(e, st);
+    g_timing.end[kind].push_back(e);
+  }
+};
+
 static int check_device(int dev) {
   if (dev < 0 || dev >= 64) return fail(SCE_EINVAL, "device %d out of range", dev);
   std::lock_guard<std::mutex> lk(g_mu);
@@ -839,6 +878,36 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P) {
 static int64_t default_panel(const SavedLayout& S) { return S.Np < 8192 ? S.Np : 8192; }
 
 extern "C" int sce_version(void) { return SCE_VERSION; }
+
+extern "C" int sce_timing_enable(int on) {
+  std::lock_guard<std::mutex> lk(g_timing_mu);
+  for (int k = 0; k < SCE_K_COUNT; ++k) {
+    for (hipEvent_t e : g_timing.begin[k]) g_timing.pool.push_back(e);
+    for (hipEvent_t e : g_timing.end[k]) g_timing.pool.push_back(e);
+    g_timing.begin[k].clear(); g_timing.end[k].clear();
+    g_timing.ms[k] = 0.0; g_timing.launches[k] = 0;
+  }
+  g_timing.on = on != 0;
+  return SCE_OK;
+}
+
+extern "C" int sce_timing_read(sce_timing* out) {
+  if (!out) return fail(SCE_EINVAL, "out is NULL");
+  std::lock_guard<std::mutex> lk(g_timing_mu);
+  for (int k = 0; k < SCE_K_COUNT; ++k) {
+    const size_t n = g_timing.end[k].size();
+    for (size_t i = 0; i < n; ++i) {
+      float ms = 0.f;
+      HIP_TRY(hipEventSynchronize(g_timing.end[k][i]));
+      HIP_TRY(hipEventElapsedTime(&ms, g_timing.begin[k][i], g_timing.end[k][i]));
+      g_timing.ms[k] += ms; g_timing.launches[k] += 1;
+      g_timing.pool.push_back(g_timing.begin[k][i]); g_timing.pool.push_back(g_timing.end[k][i]);
+    }
+    g_timing.begin[k].clear(); g_timing.end[k].clear();
+    out->ms[k] = g_timing.ms[k]; out->launches[k] = g_timing.launches[k];
+  }
+  return SCE_OK;
+}
 extern "C" const char* sce_last_error(void) { return g_err; }
 
 extern "C" int sce_sizes_for(const sce_shape* shape, sce_sizes* out) {
@@ -925,6 +994,7 @@ extern "C" int sce_forward(const sce_args* a) {
   uint8_t* wq = sv + S.off_wq;
 
   {
+    KernelTimer tm(SCE_K_QUANT, st);
     const int grid = grid_for((size_t)S.Np * (S.dp / 16), 256);
     if (a->x_dtype == SCE_F32)
       quantize_pad_kernel<float><<<grid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, a->x_s);
@@ -943,7 +1013,11 @@ extern "C" int sce_forward(const sce_args* a) {
   p.dp = S.dp; p.N = (int)N; p.V = (int)V; p.Np = (int)S.Np; p.RT = RT; p.CT = CT; p.S = nsplit;
   p.sc = a->x_s * a->w_s; p.c1 = 2.0f * LOG2E / a->cap; p.c2 = -2.0f * a->cap * LOG2E; p.cap = a->cap;
   const int grid = 8 * nsplit * ((RT + 7) / 8);
-  fwd_kernel<<<grid, NTHREADS, SMEM_BYTES, st>>>(p);
+  {
+    KernelTimer tm(SCE_K_FWD, st);
+    fwd_kernel<<<grid, NTHREADS, SMEM_BYTES, st>>>(p);
+  }
+  KernelTimer tm_red(SCE_K_FWD_REDUCE, st);
   float* s_lse = (float*)(sv + S.off_lse);
   float* s_umax = (float*)(sv + S.off_umax);
   float* s_zy = (float*)(sv + S.off_zy);
@@ -1005,6 +1079,7 @@ extern "C" int sce_backward(const sce_args* a) {
   uint8_t* ghat_t = ws + B.off_ghat_t;
 
   const int nblk = (int)(S.Np / 256);
+  KernelTimer* tm_prep = new KernelTimer(SCE_K_BWD_PREP, st);
   bwd_prep_kernel<<<nblk, 256, 0, st>>>(s_lse, s_umax, s_zy, a->targets, a->ignore_index, hdr, a->grad_output,
                                         a->reduction == SCE_REDUCE_NONE ? 1 : 0, a->grad_scale, a->cap, (int)N, (int)S.Np, (int)V,
                                         crow, rho, hcoef, blockmax);
@@ -1020,9 +1095,10 @@ extern "C" int sce_backward(const sce_args* a) {
     while ((1ll << bits) <= V) ++bits;
     size_t tmp = B.sorttmp_bytes;
     if (sce::sort_pairs(ws + B.off_sorttmp, &tmp, keys_in, skeys, vals_in, perm, (size_t)N, bits, st) != 0)
-      return fail(SCE_EHIP, "radix sort of the targets failed");
+    { delete tm_prep; return fail(SCE_EHIP, "radix sort of the targets failed"); }
     bwd_segoff_kernel<<<(int)((N + 256) / 256), 256, 0, st>>>(skeys, (int)N, (int)V, segoff);
   }
+  delete tm_prep;
   const float sc = a->x_s * a->w_s, c1 = 2.0f * LOG2E / a->cap, c2 = -2.0f * a->cap * LOG2E;
   const int CTv = (int)(S.Vp / 256), CTd = (int)(S.dq / 256);
   int first = 1;
@@ -1032,26 +1108,36 @@ extern "C" int sce_backward(const sce_args* a) {
     RecomputeParams rp;
     rp.xq = xq + p0 * S.dp; rp.wqt = wqt; rp.crow = crow + p0; rp.ghat = ghat; rp.ghat_t = ghat_t;
     rp.dp = S.dp; rp.Vp = S.Vp; rp.P = P; rp.RT = RTp; rp.CT = CTv; rp.V = (int)V; rp.sc = sc; rp.c1 = c1; rp.c2 = c2;
-    bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_BYTES, st>>>(rp);
+    {
+      KernelTimer tm(SCE_K_RECOMPUTE, st);
+      bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_BYTES, st>>>(rp);
+    }
 
     DxParams dp_;
     dp_.wq = wq; dp_.ghat = ghat; dp_.wqt = wqt; dp_.rho = rho + p0; dp_.hcoef = hcoef + p0; dp_.targets = a->targets + p0;
     dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.dp = S.dp; dp_.RT = RTp; dp_.CT = CTd;
     dp_.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); dp_.d = (int)d; dp_.V = (int)V; dp_.w_s = a->w_s;
-    if (a->dx_dtype == SCE_F32) {
-      dp_.dx = (float*)a->dx + p0 * a->dx_ld;
-      bwd_dx_kernel<float><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_BYTES, st>>>(dp_);
-    } else {
-      dp_.dx = (bf16_t*)a->dx + p0 * a->dx_ld;
-      bwd_dx_kernel<bf16_t><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_BYTES, st>>>(dp_);
+    {
+      KernelTimer tm(SCE_K_DX, st);
+      if (a->dx_dtype == SCE_F32) {
+        dp_.dx = (float*)a->dx + p0 * a->dx_ld;
+        bwd_dx_kernel<float><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_BYTES, st>>>(dp_);
+      } else {
+        dp_.dx = (bf16_t*)a->dx + p0 * a->dx_ld;
+        bwd_dx_kernel<bf16_t><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_BYTES, st>>>(dp_);
+      }
     }
 
     DwParams wp;
     wp.xt = xt + p0; wp.ghat_t = ghat_t; wp.dwacc = dwacc; wp.Np = S.Np; wp.P = P; wp.Vp = S.Vp;
     wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(prow / BK); wp.accumulate = first ? 0 : 1;
-    bwd_dw_kernel<<<map_tile_grid(CTd, CTv), NTHREADS, SMEM_BYTES, st>>>(wp);
+    {
+      KernelTimer tm(SCE_K_DW, st);
+      bwd_dw_kernel<<<map_tile_grid(CTd, CTv), NTHREADS, SMEM_BYTES, st>>>(wp);
+    }
     first = 0;
   }
+  KernelTimer tm_fin(SCE_K_DW_FINAL, st);
   bwd_dw_long_kernel<<<(int)V, 256, 0, st>>>(segoff, perm, hcoef, xq, S.dp, S.dq, S.Vp, xi, dwacc);
   {
     dim3 g((unsigned)((V + 63) / 64), (unsigned)((d + 63) / 64));

@@ -32,7 +32,7 @@ def run_ours(inp, reduction="mean", x_dtype=torch.bfloat16, w_dtype=torch.bfloat
     dx, dw = ck.ce_backward(saved, y, grad_output, N, d, V, inp.x_s, inp.w_s, inp.cap, 1.0, reduction, x_dtype, w_dtype,
                             panel_rows=panel_rows)
     torch.cuda.synchronize()
-    return dict(loss=out, lse=lse, argmax=argmax, n_valid=n_valid, dx=dx, dw=dw, x=x, w=w, y=y)
+    return dict(loss=out, lse=lse, argmax=argmax, n_valid=n_valid, dx=dx, dw=dw, x=x, w=w, y=y, x_s=inp.x_s, w_s=inp.w_s)
 
 
 def run_oracle(inp, ours, reduction="mean", grad_output=None, row_chunk=4096):
@@ -71,7 +71,24 @@ def check_parity(ours, ref, reduction="mean", check_argmax=True):
         if reduction == "none":
             assert float(ours["loss"][ign].abs().max()) == 0.0
     if check_argmax and ours["argmax"] is not None:
-        mism = ours["argmax"].long() != ref["argmax"]
-        report["argmax_mismatch"] = int(mism.sum())
-        assert report["argmax_mismatch"] == 0, f"{report['argmax_mismatch']} argmax mismatches"
+        # Bit-exact except on genuine near-ties: fp8 x fp8 products are exact in fp32, so two correct
+        # evaluations differ only by the order of the fp32 accumulation.  A differing row is accepted
+        # only if, with the logits recomputed exactly (float64 sums of exact products), our argmax is
+        # within the accumulation error of the true maximum: 32 * 2^-24 * sum_k |x_k w_k| (the MFMA's
+        # fp32 accumulation was measured at up to ~12 * 2^-24 of that sum; a gap of this size is a few
+        # parts in 10^6 of the logit).  The number of such rows is reported.
+        mism = (ours["argmax"].long() != ref["argmax"]).nonzero().flatten()
+        report["argmax_near_ties"] = int(mism.numel())
+        if mism.numel():
+            assert mism.numel() <= max(4, ours["argmax"].numel() // 2000), f"{mism.numel()} argmax mismatches"
+            xq = eager.dequantize(eager.quantize_e4m3(ours["x"][mism], inp_scales(ours)[0]), inp_scales(ours)[0]).double()
+            wq = eager.dequantize(eager.quantize_e4m3(ours["w"], inp_scales(ours)[1]), inp_scales(ours)[1]).double()
+            u = xq @ wq
+            bound = 32 * 2.0 ** -24 * (xq.abs() @ wq.abs()).max(dim=1).values
+            got = u.gather(1, ours["argmax"][mism].long()[:, None])[:, 0]
+            assert bool((got >= u.max(dim=1).values - bound).all()), "argmax differs on a row that is not a near-tie"
     return report
+
+
+def inp_scales(ours):
+    return ours["x_s"], ours["w_s"]
