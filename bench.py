@@ -42,7 +42,7 @@ def main():
     ap.add_argument("--rows", type=int, default=None, help="override N (debugging only; the result is then not the headline)")
     ap.add_argument("--panel-rows", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-rows", type=int, default=2048)
+    ap.add_argument("--cpu-rows", type=int, default=16384)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (one process, one MI355X); run with --gpus 1", file=sys.stderr)

@@ -46,7 +46,7 @@ enum {
 typedef struct sce_shape {
   int64_t N;           /* rows (tokens)                         */
   int64_t d;           /* hidden size, multiple of 16           */
-  int64_t V;           /* vocabulary (columns of W), < 2^31     */
+  int64_t V;           /* vocabulary (columns of W); N, d, V < 2^24 */
   int32_t n_predict;   /* number of MTP offsets, 1..4           */
   int32_t reserved;
 } sce_shape;

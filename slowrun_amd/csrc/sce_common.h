@@ -17,10 +17,9 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 // 8*(r/4) + 4*(l/32) + r%4, r = 0..15).
 constexpr int TM = 256;          // A-side rows per tile
 constexpr int TN = 256;          // B-side rows per tile
-constexpr int BK = 128;          // K bytes per pipeline stage
-constexpr int PITCH = BK + 16;   // LDS row pitch: 16 lanes x 16 B then cover all 64 banks
-constexpr int STAGE_BYTES = (TM + TN) * PITCH;
-constexpr int SMEM_BYTES = 2 * STAGE_BYTES;     // 147456 of the 163840 B a workgroup may hold
+constexpr int BK = 128;          // K bytes per LDS slot row
+constexpr int SLOT_BYTES = (TM + TN) * BK;      // 65536
+constexpr int SMEM_BYTES = 2 * SLOT_BYTES;      // 131072 of the 163840 B a workgroup may hold
 constexpr int NTHREADS = 256;
 
 constexpr float LOG2E = 1.4426950408889634f;
@@ -29,7 +28,7 @@ static inline int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * 
 
 // Layout of the state sce_forward saves for sce_backward (byte offsets into `saved`).
 struct SavedLayout {
-  int64_t N, d, V, Np, dp, dq, Vp;   // Np, Vp: multiples of 256; dp: of 128; dq: of 256
+  int64_t N, d, V, Np, dp, dq, Vp;   // Np, Vp: multiples of 256; dp: of 128, at least 256; dq: of 256
   size_t off_hdr, off_xq, off_wqt, off_wq, off_lse, off_umax, off_zy, total;
 };
 // hdr: int32 n_valid, int32 n_bad_targets, float loss_sum, float pad
@@ -37,7 +36,7 @@ struct SavedLayout {
 static inline SavedLayout saved_layout(int64_t N, int64_t d, int64_t V, int n_predict) {
   SavedLayout L;
   L.N = N; L.d = d; L.V = V;
-  L.Np = round_up(N, 256); L.dp = round_up(d, 128); L.dq = round_up(d, 256); L.Vp = round_up(V, 256);
+  L.Np = round_up(N, 256); L.dp = round_up(d, 128) < 256 ? 256 : round_up(d, 128); L.dq = round_up(d, 256); L.Vp = round_up(V, 256);
   size_t o = 0;
   auto take = [&](size_t bytes) { size_t r = o; o += (bytes + 255) / 256 * 256; return r; };
   L.off_hdr = take(256);
@@ -52,7 +51,7 @@ static inline SavedLayout saved_layout(int64_t N, int64_t d, int64_t V, int n_pr
 }
 
 struct BwdLayout {
-  int64_t P;                         // rows per panel (multiple of 256)
+  int64_t P, Pw;                     // rows per recompute/dX panel and per dW launch (multiples of 256, Pw of P)
   size_t off_crow, off_rho, off_hcoef, off_blockmax, off_xi, off_xt, off_dwacc, off_perm, off_keys,
       off_segoff, off_sorttmp, off_ghat, off_ghat_t, fixed, total;
   size_t sorttmp_bytes;

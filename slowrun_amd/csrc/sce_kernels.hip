@@ -16,6 +16,7 @@
 //             dlogits never goes through fp8: it is applied in fp32 in the dX epilogue
 //             (gather of W_q^T rows) and in the dW finalisation (rows grouped by target).
 #include "sce_common.h"
+#include "sce_mainloop.h"
 #include "../../include/slowrun_ce.h"
 
 #include <math.h>
@@ -71,95 +72,25 @@ template <> struct Elem<bf16_t> {
 };
 
 // XCD-aware tile order.  Consecutive workgroup ids go round-robin to the 8 XCDs, each with its
-// own L2; the 32 workgroups resident on one XCD are given a 4 x 8 block of tiles so that they
-// share A-side and B-side rows through that L2.
+// own L2.  The tiles are put in a locality-preserving order (groups of 8 columns, walked row by
+// row, so that 32 consecutive tiles form a 4 x 8 block sharing A-side and B-side rows) and every
+// XCD takes one contiguous eighth of that order: equal shares, and neighbours in the order run on
+// the same L2 at about the same time.
 __device__ __forceinline__ bool map_tile(int bid, int RT, int CT, int& rt, int& ct) {
-  const int xcd = bid & 7, slot = bid >> 3;
-  const int c = slot >> 5, w = slot & 31;
-  const int st = c * 8 + xcd;
-  const int SC = (CT + 7) >> 3;
-  const int sr = st / SC, sc = st - sr * SC;
-  rt = sr * 4 + (w >> 3);
-  ct = sc * 8 + (w & 7);
-  return rt < RT && ct < CT;
+  const int T = RT * CT;
+  const int per = (T + 7) >> 3;
+  const int xcd = bid & 7, local = bid >> 3;
+  if (local >= per) return false;
+  const int idx = xcd * per + local;
+  if (idx >= T) return false;
+  const int gsz = 8 * RT;                 // tiles in a full group of 8 columns
+  const int g = idx / gsz, rem = idx - g * gsz;
+  const int gw = (CT - g * 8) < 8 ? (CT - g * 8) : 8;
+  rt = rem / gw;
+  ct = g * 8 + (rem - rt * gw);
+  return true;
 }
-static inline int map_tile_grid(int RT, int CT) {
-  const int SR = (RT + 3) / 4, SC = (CT + 7) / 8;
-  return 8 * 32 * ((SR * SC + 7) / 8);
-}
-
-// ------------------------------------------------------------------------------------------
-// MFMA main loop: acc[a][b] (32x32 blocks) += A_tile[256][K] * B_tile[256][K]^T, fp8 e4m3.
-// Wave (wa, wb) of the 2 x 2 wave grid owns A rows [128 wa, +128) and B rows [128 wb, +128).
-// Global -> registers -> LDS, two LDS stages, one barrier per 128 bytes of K.
-// ------------------------------------------------------------------------------------------
-__device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, int64_t lda,
-                                              const uint8_t* __restrict__ Bg, int64_t ldb, int KT,
-                                              uint8_t* smem, v16f (&acc)[4][4]) {
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
-  const int lrow = t >> 3, lcol = (t & 7) * 16;
-  const uint8_t* ap = Ag + (int64_t)lrow * lda + lcol;
-  const uint8_t* bp = Bg + (int64_t)lrow * ldb + lcol;
-  v4i ra[8], rb[8];
-
-#pragma unroll
-  for (int a = 0; a < 4; ++a)
-#pragma unroll
-    for (int b = 0; b < 4; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
-
-  auto gload = [&](int kt) {
-#pragma unroll
-    for (int n = 0; n < 8; ++n) {
-      ra[n] = *reinterpret_cast<const v4i*>(ap + (int64_t)(32 * n) * lda + (int64_t)kt * BK);
-      rb[n] = *reinterpret_cast<const v4i*>(bp + (int64_t)(32 * n) * ldb + (int64_t)kt * BK);
-    }
-  };
-  auto swrite = [&](int stage) {
-    uint8_t* sa = smem + stage * STAGE_BYTES + lrow * PITCH + lcol;
-    uint8_t* sb = sa + TM * PITCH;
-#pragma unroll
-    for (int n = 0; n < 8; ++n) {
-      *reinterpret_cast<v4i*>(sa + 32 * n * PITCH) = ra[n];
-      *reinterpret_cast<v4i*>(sb + 32 * n * PITCH) = rb[n];
-    }
-  };
-
-  gload(0);
-  swrite(0);
-  __syncthreads();
-  const int frag_off = (lane & 31) * PITCH + (lane >> 5) * 32;
-  for (int kt = 0; kt < KT; ++kt) {
-    const bool more = kt + 1 < KT;
-    if (more) gload(kt + 1);
-    const uint8_t* sa = smem + (kt & 1) * STAGE_BYTES + wa * 128 * PITCH + frag_off;
-    const uint8_t* sb = smem + (kt & 1) * STAGE_BYTES + (TM + wb * 128) * PITCH + frag_off;
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      v8i fa[4], fb[4];
-#pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        const v4i lo = *reinterpret_cast<const v4i*>(sa + a * 32 * PITCH + s * 64);
-        const v4i hi = *reinterpret_cast<const v4i*>(sa + a * 32 * PITCH + s * 64 + 16);
-        fa[a] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      }
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const v4i lo = *reinterpret_cast<const v4i*>(sb + b * 32 * PITCH + s * 64);
-        const v4i hi = *reinterpret_cast<const v4i*>(sb + b * 32 * PITCH + s * 64 + 16);
-        fb[b] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      }
-#pragma unroll
-      for (int a = 0; a < 4; ++a)
-#pragma unroll
-        for (int b = 0; b < 4; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[a], fb[b], acc[a][b], 0, 0, 0, 0, 0, 0);
-    }
-    if (more) swrite((kt + 1) & 1);
-    __syncthreads();
-  }
-}
+static inline int map_tile_grid(int RT, int CT) { return 8 * ((RT * CT + 7) / 8); }
 
 // ------------------------------------------------------------------------------------------
 // quantisation
@@ -506,8 +437,8 @@ struct RecomputeParams {
   const uint8_t* wqt;    // [Vp][dp]
   const float* crow;     // offset to the panel's first row
   uint8_t* ghat;         // [P][Vp]
-  uint8_t* ghat_t;       // [Vp][P]
-  int64_t dp, Vp, P;
+  uint8_t* ghat_t;       // [Vp][Pw], already offset to this panel's first column
+  int64_t dp, Vp, Pw;
   int RT, CT, V;
   float sc, c1, c2;
 };
@@ -546,7 +477,7 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
         const uint32_t w = cvt4_e4m3(g[0], g[1], g[2], g[3]);
         *reinterpret_cast<uint32_t*>(p.ghat + (int64_t)il * p.Vp + v) = w;
 #pragma unroll
-        for (int m = 0; m < 4; ++m) p.ghat_t[(int64_t)(v + m) * p.P + il] = (uint8_t)(w >> (8 * m));
+        for (int m = 0; m < 4; ++m) p.ghat_t[(int64_t)(v + m) * p.Pw + il] = (uint8_t)(w >> (8 * m));
       }
     }
   }
@@ -603,10 +534,10 @@ __global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p) {
 }
 
 struct DwParams {
-  const uint8_t* xt;      // [dq][Np], offset to the panel's first column   A side (rows j)
-  const uint8_t* ghat_t;  // [Vp][P]                                         B side (rows v)
+  const uint8_t* xt;      // [dq][Np], offset to the first row of the dW panel   A side (rows j)
+  const uint8_t* ghat_t;  // [Vp][Pw]                                             B side (rows v)
   float* dwacc;           // [dq][Vp] fp32
-  int64_t Np, P, Vp;
+  int64_t Np, Pw, Vp;
   int RT, CT, KT, accumulate;
 };
 
@@ -616,7 +547,7 @@ __global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
   if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
-  mfma_mainloop(p.xt + (int64_t)rt * 256 * p.Np, p.Np, p.ghat_t + (int64_t)ct * 256 * p.P, p.P, p.KT, smem, acc);
+  mfma_mainloop(p.xt + (int64_t)rt * 256 * p.Np, p.Np, p.ghat_t + (int64_t)ct * 256 * p.Pw, p.Pw, p.KT, smem, acc);
   const int jbase = rt * 256 + wa * 128 + 4 * (lane >> 5);
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
@@ -655,47 +586,45 @@ __global__ __launch_bounds__(256) void bwd_segoff_kernel(const int32_t* __restri
 
 constexpr int LONG_SEG = 64;
 
-// Columns that are the target of many rows: dwacc[:, v] -= sum_i h_i X_q[i, :] / xi, one
-// workgroup per column, rows split over 16 row-lanes and folded in a fixed order.
+// Columns that are the target of many rows: dwacc[:, v] -= sum_i h_i X_q[i, :] / xi.  One
+// workgroup per (column, block of 256 rows of dW); the rows of the segment are split over 16
+// row-lanes and folded in a fixed order, so the result does not depend on scheduling.
 __global__ __launch_bounds__(256) void bwd_dw_long_kernel(const int32_t* __restrict__ segoff, const int32_t* __restrict__ perm,
                                                          const float* __restrict__ hcoef, const uint8_t* __restrict__ xq,
-                                                         int64_t dp, int64_t dq, int64_t Vp, const float* __restrict__ xi,
+                                                         int64_t dp, int64_t Vp, const float* __restrict__ xi,
                                                          float* __restrict__ dwacc) {
   __shared__ float red[16][256];
   const int v = blockIdx.x;
   const int s0 = segoff[v], L = segoff[v + 1] - s0;
   if (L < LONG_SEG) return;
   const int t = threadIdx.x, c = t & 15, rl = t >> 4;
-  const float inv_xi = 1.0f / xi[0];
-  for (int64_t jb = 0; jb < dq; jb += 256) {
-    float a[16];
+  const int64_t jb = (int64_t)blockIdx.y * 256;
+  float a[16];
 #pragma unroll
-    for (int m = 0; m < 16; ++m) a[m] = 0.f;
-    if (jb + c * 16 < dp) {
-      for (int n = rl; n < L; n += 16) {
-        const int i = perm[s0 + n];
-        const float h = hcoef[i];
-        const v4i raw = *reinterpret_cast<const v4i*>(xq + (int64_t)i * dp + jb + c * 16);
+  for (int m = 0; m < 16; ++m) a[m] = 0.f;
+  if (jb + c * 16 < dp) {
+    for (int n = rl; n < L; n += 16) {
+      const int i = perm[s0 + n];
+      const float h = hcoef[i];
+      const v4i raw = *reinterpret_cast<const v4i*>(xq + (int64_t)i * dp + jb + c * 16);
 #pragma unroll
-        for (int m = 0; m < 4; ++m) {
-          const uint32_t w = (uint32_t)raw[m];
-          a[4 * m + 0] = fmaf(h, e4m3_to_float<0>(w), a[4 * m + 0]);
-          a[4 * m + 1] = fmaf(h, e4m3_to_float<1>(w), a[4 * m + 1]);
-          a[4 * m + 2] = fmaf(h, e4m3_to_float<2>(w), a[4 * m + 2]);
-          a[4 * m + 3] = fmaf(h, e4m3_to_float<3>(w), a[4 * m + 3]);
-        }
+      for (int m = 0; m < 4; ++m) {
+        const uint32_t w = (uint32_t)raw[m];
+        a[4 * m + 0] = fmaf(h, e4m3_to_float<0>(w), a[4 * m + 0]);
+        a[4 * m + 1] = fmaf(h, e4m3_to_float<1>(w), a[4 * m + 1]);
+        a[4 * m + 2] = fmaf(h, e4m3_to_float<2>(w), a[4 * m + 2]);
+        a[4 * m + 3] = fmaf(h, e4m3_to_float<3>(w), a[4 * m + 3]);
       }
     }
-    __syncthreads();
-#pragma unroll
-    for (int m = 0; m < 16; ++m) red[rl][c * 16 + m] = a[m];
-    __syncthreads();
-    float sfold = 0.f;
-#pragma unroll
-    for (int k = 0; k < 16; ++k) sfold += red[k][t];
-    float* dst = dwacc + (jb + t) * Vp + v;
-    *dst -= sfold * inv_xi;
   }
+#pragma unroll
+  for (int m = 0; m < 16; ++m) red[rl][c * 16 + m] = a[m];
+  __syncthreads();
+  float sfold = 0.f;
+#pragma unroll
+  for (int k = 0; k < 16; ++k) sfold += red[k][t];
+  float* dst = dwacc + (jb + t) * Vp + v;
+  *dst -= sfold / xi[0];
 }
 
 // dW = x_s * ( xi * dwacc - sum over the (short) target segment of h_i X_q[i, :] ), cast to the
@@ -821,7 +750,7 @@ static int check_device(int dev) {
     HIP_TRY(hipGetDeviceProperties(&prop, dev));
     g_arch_ok[dev] = strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : -1;
     if (g_arch_ok[dev] == 1) {
-      // the MFMA kernels hold two 72 KB stages in LDS
+      // the MFMA kernels hold two 64 KB K-slots in LDS
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_recompute_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
@@ -838,7 +767,8 @@ static int check_shape(const sce_shape* s) {
   if (s->N <= 0 || s->d <= 0 || s->V <= 0) return fail(SCE_EINVAL, "N, d, V must be positive (got %lld, %lld, %lld)",
                                                        (long long)s->N, (long long)s->d, (long long)s->V);
   if (s->d % 16 != 0) return fail(SCE_EINVAL, "d = %lld must be a multiple of 16", (long long)s->d);
-  if (s->N >= (1ll << 31) - 512 || s->V >= (1ll << 31) - 512) return fail(SCE_EINVAL, "N and V must be below 2^31");
+  if (s->N > (1ll << 24) - 256 || s->V > (1ll << 24) - 256 || s->d > (1ll << 24) - 256)
+    return fail(SCE_EINVAL, "N, d and V must be below 2^24 (32-bit tile offsets)");
   if (s->n_predict != 1) return fail(SCE_EINVAL, "n_predict = %d: only a single offset is built into the kernels", s->n_predict);
   return SCE_OK;
 }
@@ -851,9 +781,9 @@ static size_t sort_tmp_bytes(int64_t N, int64_t V) {
   return bytes;
 }
 
-static BwdLayout bwd_layout(const SavedLayout& S, int64_t P) {
+static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw) {
   BwdLayout B;
-  B.P = P;
+  B.P = P; B.Pw = Pw;
   size_t o = 0;
   auto take = [&](size_t bytes) { size_t r = o; o += (bytes + 255) / 256 * 256; return r; };
   B.off_crow = take((size_t)S.Np * 4);
@@ -870,12 +800,29 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P) {
   B.off_sorttmp = take(B.sorttmp_bytes);
   B.fixed = o;
   B.off_ghat = take((size_t)P * S.Vp);
-  B.off_ghat_t = take((size_t)S.Vp * P);
+  B.off_ghat_t = take((size_t)S.Vp * Pw);
   B.total = o;
   return B;
 }
 
-static int64_t default_panel(const SavedLayout& S) { return S.Np < 8192 ? S.Np : 8192; }
+// Rows per panel: as many 256-row tiles as give the dX kernel one full round of tiles on the
+// 256 CUs (its tile count is (P / 256) * (dq / 256)), capped by the problem size.
+static int64_t default_panel(const SavedLayout& S) {
+  int64_t rt = 256 / (S.dq / 256);
+  if (rt < 1) rt = 1;
+  if (rt > 64) rt = 64;
+  const int64_t P = rt * 256;
+  return S.Np < P ? S.Np : P;
+}
+// Rows per dW launch: several dX panels are gathered (transposed) before dW runs, so that its
+// fp32 accumulator is read and rewritten less often and its K loop is long.
+static int64_t default_dw_panel(const SavedLayout& S, int64_t P) {
+  int64_t m = 24576 / P;
+  if (m < 1) m = 1;
+  int64_t Pw = m * P;
+  const int64_t cap = round_up(S.Np, P);
+  return Pw < cap ? Pw : cap;
+}
 
 extern "C" int sce_version(void) { return SCE_VERSION; }
 
@@ -916,9 +863,9 @@ extern "C" int sce_sizes_for(const sce_shape* shape, sce_sizes* out) {
   const SavedLayout S = saved_layout(shape->N, shape->d, shape->V, shape->n_predict);
   out->saved_bytes = S.total;
   out->fwd_workspace_bytes = (size_t)8 * S.Np * 16 + 256;
-  out->bwd_workspace_min_bytes = bwd_layout(S, 256).total;
+  out->bwd_workspace_min_bytes = bwd_layout(S, 256, 256).total;
   out->bwd_panel_rows = default_panel(S);
-  out->bwd_workspace_bytes = bwd_layout(S, out->bwd_panel_rows).total;
+  out->bwd_workspace_bytes = bwd_layout(S, out->bwd_panel_rows, default_dw_panel(S, out->bwd_panel_rows)).total;
   return SCE_OK;
 }
 
@@ -1040,16 +987,21 @@ extern "C" int sce_backward(const sce_args* a) {
   const SavedLayout S = saved_layout(N, d, V, a->shape.n_predict);
   if (a->saved_bytes < S.total) return fail(SCE_EINVAL, "saved buffer too small: %zu < %zu", a->saved_bytes, S.total);
   if (!a->workspace) return fail(SCE_EINVAL, "workspace is NULL");
-  const BwdLayout Bmin = bwd_layout(S, 256);
+  const BwdLayout Bmin = bwd_layout(S, 256, 256);
   if (a->workspace_bytes < Bmin.total) return fail(SCE_EINVAL, "backward workspace too small: %zu < %zu", a->workspace_bytes, Bmin.total);
-  int64_t P = (int64_t)((a->workspace_bytes - Bmin.fixed) / (2 * (size_t)S.Vp)) / 256 * 256;
-  if (P > S.Np) P = S.Np;
+  // panel sizes from what the caller gave: P rows per recompute/dX panel, Pw = m * P rows per dW launch
+  const size_t room = (a->workspace_bytes - Bmin.fixed) / (size_t)S.Vp;     // rows of e4m3 scratch available
+  int64_t P = default_panel(S);
   if (a->panel_rows > 0) {
     if (a->panel_rows % 256) return fail(SCE_EINVAL, "panel_rows must be a multiple of 256");
-    if (a->panel_rows < P) P = a->panel_rows;
+    P = a->panel_rows < S.Np ? a->panel_rows : S.Np;
   }
+  if ((int64_t)(room / 2) < P) P = (int64_t)(room / 2) / 256 * 256;
   if (P < 256) return fail(SCE_EINVAL, "backward workspace too small for one 256-row panel");
-  const BwdLayout B = bwd_layout(S, P);
+  int64_t Pw = default_dw_panel(S, P);
+  if ((int64_t)room - P < Pw) Pw = ((int64_t)room - P) / P * P;
+  if (Pw < P) return fail(SCE_EINVAL, "internal: dW panel smaller than the dX panel");
+  const BwdLayout B = bwd_layout(S, P, Pw);
   if (B.total > a->workspace_bytes) return fail(SCE_EINVAL, "internal: panel layout exceeds workspace");
   DeviceGuard guard(a->device);
   if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", a->device);
@@ -1102,12 +1054,13 @@ extern "C" int sce_backward(const sce_args* a) {
   const float sc = a->x_s * a->w_s, c1 = 2.0f * LOG2E / a->cap, c2 = -2.0f * a->cap * LOG2E;
   const int CTv = (int)(S.Vp / 256), CTd = (int)(S.dq / 256);
   int first = 1;
+  int64_t w0 = 0;                      // first row of the rows gathered for the next dW launch
   for (int64_t p0 = 0; p0 < S.Np; p0 += P) {
     const int64_t prow = (S.Np - p0 < P) ? (S.Np - p0) : P;     // multiple of 256
     const int RTp = (int)(prow / 256);
     RecomputeParams rp;
-    rp.xq = xq + p0 * S.dp; rp.wqt = wqt; rp.crow = crow + p0; rp.ghat = ghat; rp.ghat_t = ghat_t;
-    rp.dp = S.dp; rp.Vp = S.Vp; rp.P = P; rp.RT = RTp; rp.CT = CTv; rp.V = (int)V; rp.sc = sc; rp.c1 = c1; rp.c2 = c2;
+    rp.xq = xq + p0 * S.dp; rp.wqt = wqt; rp.crow = crow + p0; rp.ghat = ghat; rp.ghat_t = ghat_t + (p0 - w0);
+    rp.dp = S.dp; rp.Vp = S.Vp; rp.Pw = Pw; rp.RT = RTp; rp.CT = CTv; rp.V = (int)V; rp.sc = sc; rp.c1 = c1; rp.c2 = c2;
     {
       KernelTimer tm(SCE_K_RECOMPUTE, st);
       bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_BYTES, st>>>(rp);
@@ -1128,17 +1081,21 @@ extern "C" int sce_backward(const sce_args* a) {
       }
     }
 
-    DwParams wp;
-    wp.xt = xt + p0; wp.ghat_t = ghat_t; wp.dwacc = dwacc; wp.Np = S.Np; wp.P = P; wp.Vp = S.Vp;
-    wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(prow / BK); wp.accumulate = first ? 0 : 1;
-    {
-      KernelTimer tm(SCE_K_DW, st);
-      bwd_dw_kernel<<<map_tile_grid(CTd, CTv), NTHREADS, SMEM_BYTES, st>>>(wp);
+    const int64_t gathered = p0 + prow - w0;
+    if (gathered + P > Pw || p0 + prow >= S.Np) {      // the transposed scratch is full, or this was the last panel
+      DwParams wp;
+      wp.xt = xt + w0; wp.ghat_t = ghat_t; wp.dwacc = dwacc; wp.Np = S.Np; wp.Pw = Pw; wp.Vp = S.Vp;
+      wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(gathered / BK); wp.accumulate = first ? 0 : 1;
+      {
+        KernelTimer tm(SCE_K_DW, st);
+        bwd_dw_kernel<<<map_tile_grid(CTd, CTv), NTHREADS, SMEM_BYTES, st>>>(wp);
+      }
+      first = 0;
+      w0 = p0 + prow;
     }
-    first = 0;
   }
   KernelTimer tm_fin(SCE_K_DW_FINAL, st);
-  bwd_dw_long_kernel<<<(int)V, 256, 0, st>>>(segoff, perm, hcoef, xq, S.dp, S.dq, S.Vp, xi, dwacc);
+  bwd_dw_long_kernel<<<dim3((unsigned)V, (unsigned)(S.dq / 256)), 256, 0, st>>>(segoff, perm, hcoef, xq, S.dp, S.Vp, xi, dwacc);
   {
     dim3 g((unsigned)((V + 63) / 64), (unsigned)((d + 63) / 64));
     if (a->dw_dtype == SCE_F32)
