@@ -194,41 +194,56 @@ __global__ __launch_bounds__(256) void transpose_bytes_kernel(const uint8_t* __r
 struct FwdParams {
   const uint8_t* xq;       // [Np][dp]
   const uint8_t* wqt;      // [Vp][dp]
-  const int64_t* targets;  // [N]
-  float4* partials;        // [S][Np]: sum exp(z - cap), max u, argmax u (bits), z at target (-inf if not seen)
+  float4* partials;        // [S][Np]: sum exp(z - cap), max u, argmax u (bits), unused
   int64_t dp;
   int N, V, Np, RT, CT, S;
   float sc;                // x_s * w_s
-  float c1;                // 2 log2(e) / cap
+  float k1;                // x_s * w_s * 2 log2(e) / cap : exp2(acc * k1) = e^{2u/cap}
   float c2;                // -2 cap log2(e)
-  float cap;
 };
 
+// Per 256 x 256 tile and per row a lane owns: add up e^{z - cap} over its 64 columns and keep the
+// largest raw accumulator.  z is bounded by +-cap, so no running maximum is needed for the sum:
+//   t = tanh(u/cap) = 1 - 2/(E + 1), E = e^{2u/cap};   e^{z - cap} = exp2(c2 / (E + 1)).
+// The column of the maximum is looked up only on the (rare, after the first tiles) occasion that
+// a tile raises a row's running maximum.
 template <bool EDGE>
-__device__ __forceinline__ void fwd_epilogue(const v16f (&acc)[4][4], const FwdParams& p, int vbase, const int (&dy)[4],
-                                             float (&sum)[4], float (&umax)[4], int (&uarg)[4], float (&zy)[4]) {
+__device__ __forceinline__ void fwd_epilogue(const v16f (&acc)[4][4], const FwdParams& p, int vbase,
+                                             float (&sum)[4], float (&amax)[4], int (&uarg)[4]) {
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
-    float tmax = -INFINITY, rry = 2.0f;     // best u of this tile and its offset; 1/(E+1) at the target (2 = not here)
-    int targ = 0;
+    float tmax = -INFINITY, s = 0.f;
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int vo = a * 32 + 8 * (r >> 2) + (r & 3);
-        float u = acc[a][b][r] * p.sc;
-        const float rr = fast_rcp(fast_exp2(u * p.c1) + 1.0f);   // 1 / (e^{2u/cap} + 1), so tanh = 1 - 2 rr
-        float pt = fast_exp2(p.c2 * rr);                          // e^{z - cap}
+        float x = acc[a][b][r];
+        const float rr = fast_rcp(fast_exp2(x * p.k1) + 1.0f);
+        float pt = fast_exp2(p.c2 * rr);
         if (EDGE) {
-          if (vo >= p.V - vbase) { pt = 0.f; u = -INFINITY; }
+          if (vo >= p.V - vbase) { pt = 0.f; x = -INFINITY; }
         }
-        sum[b] += pt;
-        if (u > tmax) { tmax = u; targ = vo; }
-        if (dy[b] == vo) rry = rr;
+        s += pt;
+        tmax = fmaxf(tmax, x);
       }
     }
-    if (tmax > umax[b]) { umax[b] = tmax; uarg[b] = vbase + targ; }
-    if (rry < 2.0f) zy[b] = p.cap - 2.0f * p.cap * rry;
+    sum[b] += s;
+    if (__builtin_amdgcn_ballot_w64(tmax > amax[b]) != 0) {
+      if (tmax > amax[b]) {
+        int targ = 0x7fffffff;
+#pragma unroll
+        for (int a = 3; a >= 0; --a) {
+#pragma unroll
+          for (int r = 15; r >= 0; --r) {
+            const int vo = a * 32 + 8 * (r >> 2) + (r & 3);
+            if (acc[a][b][r] == tmax && (!EDGE || vo < p.V - vbase)) targ = vo;   // descending scan: lowest column wins
+          }
+        }
+        amax[b] = tmax;
+        uarg[b] = vbase + targ;
+      }
+    }
   }
 }
 
@@ -240,42 +255,32 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p) {
   const int ct0 = (int)((int64_t)p.CT * s / p.S), ct1 = (int)((int64_t)p.CT * (s + 1) / p.S);
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
 
-  int y[4];
-  float sum[4], umax[4], zy[4];
+  float sum[4], amax[4];
   int uarg[4];
 #pragma unroll
-  for (int b = 0; b < 4; ++b) {
-    const int i = rt * 256 + wb * 128 + b * 32 + (lane & 31);
-    int64_t yy = (i < p.N) ? p.targets[i] : -1;
-    y[b] = (yy >= 0 && yy < p.V) ? (int)yy : -0x40000000;
-    sum[b] = 0.f; umax[b] = -INFINITY; uarg[b] = 0x7fffffff; zy[b] = -INFINITY;
-  }
+  for (int b = 0; b < 4; ++b) { sum[b] = 0.f; amax[b] = -INFINITY; uarg[b] = 0x7fffffff; }
   v16f acc[4][4];
   const uint8_t* Bg = p.xq + (int64_t)rt * 256 * p.dp;
   const int KT = (int)(p.dp / BK);
   for (int ct = ct0; ct < ct1; ++ct) {
     mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.dp, p.dp, Bg, p.dp, KT, smem, acc);
     const int vbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
-    int dy[4];
-#pragma unroll
-    for (int b = 0; b < 4; ++b) dy[b] = y[b] - vbase;
-    if (ct * 256 + 256 > p.V) fwd_epilogue<true>(acc, p, vbase, dy, sum, umax, uarg, zy);
-    else fwd_epilogue<false>(acc, p, vbase, dy, sum, umax, uarg, zy);
+    if (ct * 256 + 256 > p.V) fwd_epilogue<true>(acc, p, vbase, sum, amax, uarg);
+    else fwd_epilogue<false>(acc, p, vbase, sum, amax, uarg);
   }
   // the two half-waves hold different columns of the same rows
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
-    const float s2 = __shfl_xor(sum[b], 32), um2 = __shfl_xor(umax[b], 32), zy2 = __shfl_xor(zy[b], 32);
+    const float s2 = __shfl_xor(sum[b], 32), um2 = __shfl_xor(amax[b], 32);
     const int ua2 = __shfl_xor(uarg[b], 32);
     sum[b] += s2;
-    if (um2 > umax[b] || (um2 == umax[b] && ua2 < uarg[b])) { umax[b] = um2; uarg[b] = ua2; }
-    zy[b] = fmaxf(zy[b], zy2);
+    if (um2 > amax[b] || (um2 == amax[b] && ua2 < uarg[b])) { amax[b] = um2; uarg[b] = ua2; }
   }
   // waves wa = 0 and wa = 1 hold different columns of the same rows
   float4* red = reinterpret_cast<float4*>(smem);
   if (wa == 1 && lane < 32) {
 #pragma unroll
-    for (int b = 0; b < 4; ++b) red[wb * 128 + b * 32 + lane] = make_float4(sum[b], umax[b], __int_as_float(uarg[b]), zy[b]);
+    for (int b = 0; b < 4; ++b) red[wb * 128 + b * 32 + lane] = make_float4(sum[b], amax[b], __int_as_float(uarg[b]), 0.f);
   }
   __syncthreads();
   if (wa == 0 && lane < 32) {
@@ -284,37 +289,68 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p) {
       const float4 o = red[wb * 128 + b * 32 + lane];
       const int ua2 = __float_as_int(o.z);
       sum[b] += o.x;
-      if (o.y > umax[b] || (o.y == umax[b] && ua2 < uarg[b])) { umax[b] = o.y; uarg[b] = ua2; }
-      zy[b] = fmaxf(zy[b], o.w);
+      if (o.y > amax[b] || (o.y == amax[b] && ua2 < uarg[b])) { amax[b] = o.y; uarg[b] = ua2; }
       p.partials[(int64_t)s * p.Np + rt * 256 + wb * 128 + b * 32 + lane] =
-          make_float4(sum[b], umax[b], __int_as_float(uarg[b]), zy[b]);
+          make_float4(sum[b], amax[b] * p.sc, __int_as_float(uarg[b]), 0.f);
     }
   }
+}
+
+// z at the target: one wavefront per row takes the dot product of X_q[i, :] with W_q^T[y_i, :]
+// (both contiguous) and applies the softcap.  Rows that take no part get 0.
+__global__ __launch_bounds__(256) void fwd_target_logit_kernel(const uint8_t* __restrict__ xq, const uint8_t* __restrict__ wqt,
+                                                              int64_t dp, const int64_t* __restrict__ targets,
+                                                              int64_t ignore_index, int N, int V, float sc, float cap,
+                                                              float* __restrict__ s_zy) {
+  const int lane = threadIdx.x & 63;
+  const int i = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (i >= N) return;
+  const int64_t y = targets[i];
+  const bool valid = (y != ignore_index) && y >= 0 && y < V;
+  float acc = 0.f;
+  if (valid) {
+    const uint8_t* xr = xq + (int64_t)i * dp;
+    const uint8_t* wr = wqt + y * dp;
+    for (int64_t c = lane * 16; c < dp; c += 64 * 16) {
+      const v4i xa = *reinterpret_cast<const v4i*>(xr + c);
+      const v4i wa = *reinterpret_cast<const v4i*>(wr + c);
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const uint32_t xw = (uint32_t)xa[m], ww = (uint32_t)wa[m];
+        acc = fmaf(e4m3_to_float<0>(xw), e4m3_to_float<0>(ww), acc);
+        acc = fmaf(e4m3_to_float<1>(xw), e4m3_to_float<1>(ww), acc);
+        acc = fmaf(e4m3_to_float<2>(xw), e4m3_to_float<2>(ww), acc);
+        acc = fmaf(e4m3_to_float<3>(xw), e4m3_to_float<3>(ww), acc);
+      }
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+  if (lane == 0) s_zy[i] = valid ? cap * tanhf(acc * sc / cap) : 0.f;
 }
 
 // one thread per row: fold the V-splits, write lse / loss / argmax and the saved row statistics
 __global__ __launch_bounds__(256) void fwd_combine_kernel(const float4* __restrict__ partials, int S, int N, int Np, int V,
                                                          const int64_t* __restrict__ targets, int64_t ignore_index, float cap,
                                                          float* __restrict__ s_lse, float* __restrict__ s_umax,
-                                                         float* __restrict__ s_zy, float* __restrict__ losses,
+                                                         const float* __restrict__ s_zy, float* __restrict__ losses,
                                                          float* __restrict__ lse_out, int32_t* __restrict__ argmax_out) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= Np) return;
-  if (i >= N) { s_lse[i] = 0.f; s_umax[i] = 0.f; s_zy[i] = 0.f; return; }
-  float sum = 0.f, umax = -INFINITY, zy = -INFINITY;
+  if (i >= N) { s_lse[i] = 0.f; s_umax[i] = 0.f; return; }
+  float sum = 0.f, umax = -INFINITY;
   int uarg = 0x7fffffff;
   for (int s = 0; s < S; ++s) {
     const float4 o = partials[(int64_t)s * Np + i];
     const int ua = __float_as_int(o.z);
     sum += o.x;
     if (o.y > umax || (o.y == umax && ua < uarg)) { umax = o.y; uarg = ua; }
-    zy = fmaxf(zy, o.w);
   }
   const float lse = cap + logf(sum);
   const int64_t y = targets[i];
   const bool valid = (y != ignore_index) && y >= 0 && y < V;
-  s_lse[i] = lse; s_umax[i] = umax; s_zy[i] = valid ? zy : 0.f;
-  if (losses) losses[i] = valid ? (lse - zy) : 0.f;
+  s_lse[i] = lse; s_umax[i] = umax;
+  if (losses) losses[i] = valid ? (lse - s_zy[i]) : 0.f;
   if (lse_out) lse_out[i] = lse;
   if (argmax_out) argmax_out[i] = (uarg == 0x7fffffff) ? 0 : uarg;
 }
@@ -440,11 +476,18 @@ struct RecomputeParams {
   uint8_t* ghat_t;       // [Vp][Pw], already offset to this panel's first column
   int64_t dp, Vp, Pw;
   int RT, CT, V;
-  float sc, c1, c2;
+  float k1, c2;          // as in FwdParams
 };
 
 // Recompute a 256 x 256 logit tile and leave G = 256 (1 - t^2) e^{z - zmax_row} in e4m3, once
-// row-major (operand of dX) and once transposed (operand of dW).
+// row-major (operand of dX) and once transposed (operand of dW).  Both copies are assembled in LDS
+// (free once the main loop is done) and leave the chip as fully coalesced 16-byte stores.  The
+// transposed copy is formed in registers first: the four lanes of a quad hold four consecutive
+// rows of the same four columns, and two quad-permute + byte-permute steps turn that 4 x 4 byte
+// block around.
+constexpr int STG_PITCH = 272;                               // 256 + 16: 16-byte aligned, rows shifted by 4 banks
+constexpr int SMEM_RECOMPUTE = 2 * 256 * STG_PITCH;          // 139264 B >= the main loop's 131072 B
+
 __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   int rt, ct;
@@ -452,12 +495,18 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
   mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.dp, p.dp, p.xq + (int64_t)rt * 256 * p.dp, p.dp, (int)(p.dp / BK), smem, acc);
-  const int vbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
+  uint8_t* T = smem;                         // [256 rows i][STG_PITCH]: columns v contiguous
+  uint8_t* TT = smem + 256 * STG_PITCH;      // [256 columns v][STG_PITCH]: rows i contiguous
+  const int vloc0 = wa * 128 + 4 * (lane >> 5);
   const bool edge = ct * 256 + 256 > p.V;
+  const int vlim = p.V - ct * 256;           // columns >= vlim of this tile do not exist
+  const int k = lane & 3;
+  const uint32_t sel1 = (k & 1) ? 0x03070105u : 0x06020400u;
+  const uint32_t sel2 = (k & 2) ? 0x03020706u : 0x05040100u;
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
-    const int il = rt * 256 + wb * 128 + b * 32 + (lane & 31);      // row within the panel
-    const float c = p.crow[il];
+    const int iloc = wb * 128 + b * 32 + (lane & 31);        // row within the tile
+    const float c = p.crow[rt * 256 + iloc];
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
 #pragma unroll
@@ -465,21 +514,33 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
         float g[4];
 #pragma unroll
         for (int m = 0; m < 4; ++m) {
-          const float u = acc[a][b][4 * q + m] * p.sc;
-          const float rr = fast_rcp(fast_exp2(u * p.c1) + 1.0f);
+          const float rr = fast_rcp(fast_exp2(acc[a][b][4 * q + m] * p.k1) + 1.0f);
           g[m] = fast_exp2(fmaf(p.c2, rr, c)) * (rr - rr * rr);
         }
-        const int v = vbase + a * 32 + 8 * q;
+        const int vloc = vloc0 + a * 32 + 8 * q;
         if (edge) {
 #pragma unroll
-          for (int m = 0; m < 4; ++m) if (v + m >= p.V) g[m] = 0.f;
+          for (int m = 0; m < 4; ++m) if (vloc + m >= vlim) g[m] = 0.f;
         }
         const uint32_t w = cvt4_e4m3(g[0], g[1], g[2], g[3]);
-        *reinterpret_cast<uint32_t*>(p.ghat + (int64_t)il * p.Vp + v) = w;
-#pragma unroll
-        for (int m = 0; m < 4; ++m) p.ghat_t[(int64_t)(v + m) * p.Pw + il] = (uint8_t)(w >> (8 * m));
+        *reinterpret_cast<uint32_t*>(T + iloc * STG_PITCH + vloc) = w;
+        // 4 x 4 byte transpose inside the quad: lane k ends up with column vloc + k, rows (iloc & ~3) .. +3
+        const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xB1, 0xF, 0xF, false);    // lane ^ 1
+        const uint32_t x = __builtin_amdgcn_perm(p1, w, sel1);
+        const uint32_t p2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, false);    // lane ^ 2
+        const uint32_t yv = __builtin_amdgcn_perm(p2, x, sel2);
+        *reinterpret_cast<uint32_t*>(TT + (vloc + k) * STG_PITCH + (iloc & ~3)) = yv;
       }
     }
+  }
+  __syncthreads();
+  uint8_t* grow = p.ghat + (int64_t)rt * 256 * p.Vp + (int64_t)ct * 256;
+  uint8_t* gcol = p.ghat_t + (int64_t)ct * 256 * p.Pw + (int64_t)rt * 256;
+#pragma unroll
+  for (int n = 0; n < 16; ++n) {
+    const int cidx = t + 256 * n, row = cidx >> 4, col = (cidx & 15) * 16;
+    *reinterpret_cast<v4i*>(grow + (int64_t)row * p.Vp + col) = *reinterpret_cast<const v4i*>(T + row * STG_PITCH + col);
+    *reinterpret_cast<v4i*>(gcol + (int64_t)row * p.Pw + col) = *reinterpret_cast<const v4i*>(TT + row * STG_PITCH + col);
   }
 }
 
@@ -627,10 +688,10 @@ __global__ __launch_bounds__(256) void bwd_dw_long_kernel(const int32_t* __restr
   *dst -= sfold / xi[0];
 }
 
-// dW = x_s * ( xi * dwacc - sum over the (short) target segment of h_i X_q[i, :] ), cast to the
+// dW = x_s * ( xi * (sum of the dW partials) - sum over the (short) target segment of h_i X_q[i, :] ), cast to the
 // output type.  A thread owns one column v and 16 consecutive rows j.
 template <typename T>
-__global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restrict__ dwacc, int64_t Vp, const int32_t* __restrict__ segoff,
+__global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restrict__ dwacc, int nparts, int64_t part_stride, int64_t Vp, const int32_t* __restrict__ segoff,
                                                           const int32_t* __restrict__ perm, const float* __restrict__ hcoef,
                                                           const uint8_t* __restrict__ xq, int64_t dp, const float* __restrict__ xi,
                                                           float x_s, int d, int V, T* __restrict__ dw, int64_t dw_ld) {
@@ -641,7 +702,11 @@ __global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restri
   const float scale = x_s * xi[0];
   float o[16];
 #pragma unroll
-  for (int m = 0; m < 16; ++m) o[m] = dwacc[(int64_t)(j0 + m) * Vp + v] * scale;
+  for (int m = 0; m < 16; ++m) {
+    float sum = dwacc[(int64_t)(j0 + m) * Vp + v];
+    for (int q = 1; q < nparts; ++q) sum += dwacc[q * part_stride + (int64_t)(j0 + m) * Vp + v];   // fixed order
+    o[m] = sum * scale;
+  }
   const int s0 = segoff[v], L = segoff[v + 1] - s0;
   if (L > 0 && L < LONG_SEG) {
     for (int n = 0; n < L; ++n) {
@@ -752,7 +817,7 @@ static int check_device(int dev) {
     if (g_arch_ok[dev] == 1) {
       // the MFMA kernels hold two 64 KB K-slots in LDS
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
-      HIP_TRY(hipFuncSetAttribute((const void*)bwd_recompute_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_recompute_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_RECOMPUTE));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
@@ -781,9 +846,9 @@ static size_t sort_tmp_bytes(int64_t N, int64_t V) {
   return bytes;
 }
 
-static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw) {
+static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int nparts) {
   BwdLayout B;
-  B.P = P; B.Pw = Pw;
+  B.P = P; B.Pw = Pw; B.nparts = nparts;
   size_t o = 0;
   auto take = [&](size_t bytes) { size_t r = o; o += (bytes + 255) / 256 * 256; return r; };
   B.off_crow = take((size_t)S.Np * 4);
@@ -792,7 +857,6 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw) {
   B.off_blockmax = take((size_t)(S.Np / 256) * 4);
   B.off_xi = take(256);
   B.off_xt = take((size_t)S.dq * S.Np);
-  B.off_dwacc = take((size_t)S.dq * S.Vp * 4);
   B.off_perm = take((size_t)S.N * 4 * 2);      // sorted values + unsorted values
   B.off_keys = take((size_t)S.N * 4 * 2);      // sorted keys + unsorted keys
   B.off_segoff = take((size_t)(S.V + 2) * 4);
@@ -801,6 +865,8 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw) {
   B.fixed = o;
   B.off_ghat = take((size_t)P * S.Vp);
   B.off_ghat_t = take((size_t)S.Vp * Pw);
+  B.part_stride = ((size_t)S.dq * S.Vp * 4 + 255) / 256 * 256;
+  B.off_dwacc = take(B.part_stride * (size_t)nparts);     // fp32 dW partials, one per dW launch
   B.total = o;
   return B;
 }
@@ -822,6 +888,13 @@ static int64_t default_dw_panel(const SavedLayout& S, int64_t P) {
   int64_t Pw = m * P;
   const int64_t cap = round_up(S.Np, P);
   return Pw < cap ? Pw : cap;
+}
+
+// One fp32 dW partial per dW launch (plain stores, summed once at the end) as long as there are
+// at most 8; beyond that the last buffer is read, added to and rewritten.
+static int dw_launches(const SavedLayout& S, int64_t Pw) {
+  const int64_t n = (S.Np + Pw - 1) / Pw;
+  return (int)(n < 8 ? n : 8);
 }
 
 extern "C" int sce_version(void) { return SCE_VERSION; }
@@ -863,9 +936,12 @@ extern "C" int sce_sizes_for(const sce_shape* shape, sce_sizes* out) {
   const SavedLayout S = saved_layout(shape->N, shape->d, shape->V, shape->n_predict);
   out->saved_bytes = S.total;
   out->fwd_workspace_bytes = (size_t)8 * S.Np * 16 + 256;
-  out->bwd_workspace_min_bytes = bwd_layout(S, 256, 256).total;
+  out->bwd_workspace_min_bytes = bwd_layout(S, 256, 256, 1).total;
   out->bwd_panel_rows = default_panel(S);
-  out->bwd_workspace_bytes = bwd_layout(S, out->bwd_panel_rows, default_dw_panel(S, out->bwd_panel_rows)).total;
+  {
+    const int64_t Pw = default_dw_panel(S, out->bwd_panel_rows);
+    out->bwd_workspace_bytes = bwd_layout(S, out->bwd_panel_rows, Pw, dw_launches(S, Pw)).total;
+  }
   return SCE_OK;
 }
 
@@ -956,9 +1032,9 @@ extern "C" int sce_forward(const sce_args* a) {
     else return fail(SCE_EINVAL, "unsupported w dtype %d", a->w_dtype);
   }
   FwdParams p;
-  p.xq = xq; p.wqt = wqt; p.targets = a->targets; p.partials = (float4*)a->workspace;
+  p.xq = xq; p.wqt = wqt; p.partials = (float4*)a->workspace;
   p.dp = S.dp; p.N = (int)N; p.V = (int)V; p.Np = (int)S.Np; p.RT = RT; p.CT = CT; p.S = nsplit;
-  p.sc = a->x_s * a->w_s; p.c1 = 2.0f * LOG2E / a->cap; p.c2 = -2.0f * a->cap * LOG2E; p.cap = a->cap;
+  p.sc = a->x_s * a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.c2 = -2.0f * a->cap * LOG2E;
   const int grid = 8 * nsplit * ((RT + 7) / 8);
   {
     KernelTimer tm(SCE_K_FWD, st);
@@ -968,6 +1044,8 @@ extern "C" int sce_forward(const sce_args* a) {
   float* s_lse = (float*)(sv + S.off_lse);
   float* s_umax = (float*)(sv + S.off_umax);
   float* s_zy = (float*)(sv + S.off_zy);
+  fwd_target_logit_kernel<<<(int)((N + 3) / 4), 256, 0, st>>>(xq, wqt, S.dp, a->targets, a->ignore_index, (int)N, (int)V,
+                                                           a->x_s * a->w_s, a->cap, s_zy);
   fwd_combine_kernel<<<(int)(S.Np / 256), 256, 0, st>>>(p.partials, nsplit, (int)N, (int)S.Np, (int)V, a->targets, a->ignore_index,
                                                        a->cap, s_lse, s_umax, s_zy, a->losses, a->lse, a->argmax);
   fwd_reduce_kernel<<<1, 1024, 0, st>>>(s_lse, s_zy, a->targets, a->ignore_index, (int)N, (int)V, (int32_t*)(sv + S.off_hdr),
@@ -987,10 +1065,10 @@ extern "C" int sce_backward(const sce_args* a) {
   const SavedLayout S = saved_layout(N, d, V, a->shape.n_predict);
   if (a->saved_bytes < S.total) return fail(SCE_EINVAL, "saved buffer too small: %zu < %zu", a->saved_bytes, S.total);
   if (!a->workspace) return fail(SCE_EINVAL, "workspace is NULL");
-  const BwdLayout Bmin = bwd_layout(S, 256, 256);
+  const BwdLayout Bmin = bwd_layout(S, 256, 256, 1);
   if (a->workspace_bytes < Bmin.total) return fail(SCE_EINVAL, "backward workspace too small: %zu < %zu", a->workspace_bytes, Bmin.total);
   // panel sizes from what the caller gave: P rows per recompute/dX panel, Pw = m * P rows per dW launch
-  const size_t room = (a->workspace_bytes - Bmin.fixed) / (size_t)S.Vp;     // rows of e4m3 scratch available
+  const size_t room = (a->workspace_bytes - Bmin.fixed - Bmin.part_stride) / (size_t)S.Vp;     // rows of e4m3 scratch available
   int64_t P = default_panel(S);
   if (a->panel_rows > 0) {
     if (a->panel_rows % 256) return fail(SCE_EINVAL, "panel_rows must be a multiple of 256");
@@ -1001,7 +1079,9 @@ extern "C" int sce_backward(const sce_args* a) {
   int64_t Pw = default_dw_panel(S, P);
   if ((int64_t)room - P < Pw) Pw = ((int64_t)room - P) / P * P;
   if (Pw < P) return fail(SCE_EINVAL, "internal: dW panel smaller than the dX panel");
-  const BwdLayout B = bwd_layout(S, P, Pw);
+  int nparts = dw_launches(S, Pw);
+  while (nparts > 1 && bwd_layout(S, P, Pw, nparts).total > a->workspace_bytes) --nparts;
+  const BwdLayout B = bwd_layout(S, P, Pw, nparts);
   if (B.total > a->workspace_bytes) return fail(SCE_EINVAL, "internal: panel layout exceeds workspace");
   DeviceGuard guard(a->device);
   if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", a->device);
@@ -1051,19 +1131,19 @@ extern "C" int sce_backward(const sce_args* a) {
     bwd_segoff_kernel<<<(int)((N + 256) / 256), 256, 0, st>>>(skeys, (int)N, (int)V, segoff);
   }
   delete tm_prep;
-  const float sc = a->x_s * a->w_s, c1 = 2.0f * LOG2E / a->cap, c2 = -2.0f * a->cap * LOG2E;
+  const float k1 = a->x_s * a->w_s * 2.0f * LOG2E / a->cap, c2 = -2.0f * a->cap * LOG2E;
   const int CTv = (int)(S.Vp / 256), CTd = (int)(S.dq / 256);
-  int first = 1;
+  int launch = 0;
   int64_t w0 = 0;                      // first row of the rows gathered for the next dW launch
   for (int64_t p0 = 0; p0 < S.Np; p0 += P) {
     const int64_t prow = (S.Np - p0 < P) ? (S.Np - p0) : P;     // multiple of 256
     const int RTp = (int)(prow / 256);
     RecomputeParams rp;
     rp.xq = xq + p0 * S.dp; rp.wqt = wqt; rp.crow = crow + p0; rp.ghat = ghat; rp.ghat_t = ghat_t + (p0 - w0);
-    rp.dp = S.dp; rp.Vp = S.Vp; rp.Pw = Pw; rp.RT = RTp; rp.CT = CTv; rp.V = (int)V; rp.sc = sc; rp.c1 = c1; rp.c2 = c2;
+    rp.dp = S.dp; rp.Vp = S.Vp; rp.Pw = Pw; rp.RT = RTp; rp.CT = CTv; rp.V = (int)V; rp.k1 = k1; rp.c2 = c2;
     {
       KernelTimer tm(SCE_K_RECOMPUTE, st);
-      bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_BYTES, st>>>(rp);
+      bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_RECOMPUTE, st>>>(rp);
     }
 
     DxParams dp_;
@@ -1084,13 +1164,15 @@ extern "C" int sce_backward(const sce_args* a) {
     const int64_t gathered = p0 + prow - w0;
     if (gathered + P > Pw || p0 + prow >= S.Np) {      // the transposed scratch is full, or this was the last panel
       DwParams wp;
-      wp.xt = xt + w0; wp.ghat_t = ghat_t; wp.dwacc = dwacc; wp.Np = S.Np; wp.Pw = Pw; wp.Vp = S.Vp;
-      wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(gathered / BK); wp.accumulate = first ? 0 : 1;
+      const int part = launch < nparts ? launch : nparts - 1;
+      wp.xt = xt + w0; wp.ghat_t = ghat_t; wp.dwacc = (float*)((uint8_t*)dwacc + (size_t)part * B.part_stride);
+      wp.Np = S.Np; wp.Pw = Pw; wp.Vp = S.Vp;
+      wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(gathered / BK); wp.accumulate = launch >= nparts ? 1 : 0;
       {
         KernelTimer tm(SCE_K_DW, st);
         bwd_dw_kernel<<<map_tile_grid(CTd, CTv), NTHREADS, SMEM_BYTES, st>>>(wp);
       }
-      first = 0;
+      ++launch;
       w0 = p0 + prow;
     }
   }
@@ -1099,10 +1181,10 @@ extern "C" int sce_backward(const sce_args* a) {
   {
     dim3 g((unsigned)((V + 63) / 64), (unsigned)((d + 63) / 64));
     if (a->dw_dtype == SCE_F32)
-      bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, S.Vp, segoff, perm, hcoef, xq, S.dp, xi, a->x_s, (int)d, (int)V,
+      bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.dp, xi, a->x_s, (int)d, (int)V,
                                                    (float*)a->dw, a->dw_ld);
     else
-      bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, S.Vp, segoff, perm, hcoef, xq, S.dp, xi, a->x_s, (int)d, (int)V,
+      bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.dp, xi, a->x_s, (int)d, (int)V,
                                                     (bf16_t*)a->dw, a->dw_ld);
   }
   HIP_TRY(hipGetLastError());
