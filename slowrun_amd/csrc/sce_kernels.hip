@@ -296,16 +296,18 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p) {
   }
 }
 
-// z at the target: one wavefront per row takes the dot product of X_q[i, :] with W_q^T[y_i, :]
-// (both contiguous) and applies the softcap.  Rows that take no part get 0.
+// z at the targets: one wavefront per (row i, offset k) takes the dot product of X_q[i, :] with
+// W_q^T[y_{i+k}, :] (both contiguous) and applies the softcap.  Offsets index the flattened target
+// vector, as in the reference kernel (tiny/cuda_kernels.py:229).  Pairs that take no part get 0.
 __global__ __launch_bounds__(256) void fwd_target_logit_kernel(const uint8_t* __restrict__ xq, const uint8_t* __restrict__ wqt,
                                                               int64_t dp, const int64_t* __restrict__ targets,
-                                                              int64_t ignore_index, int N, int V, float sc, float cap,
+                                                              int64_t ignore_index, int N, int Np, int V, float sc, float cap,
                                                               float* __restrict__ s_zy) {
   const int lane = threadIdx.x & 63;
   const int i = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int k = blockIdx.y;
   if (i >= N) return;
-  const int64_t y = targets[i];
+  const int64_t y = (i + k < N) ? targets[i + k] : ignore_index;
   const bool valid = (y != ignore_index) && y >= 0 && y < V;
   float acc = 0.f;
   if (valid) {
@@ -326,12 +328,19 @@ __global__ __launch_bounds__(256) void fwd_target_logit_kernel(const uint8_t* __
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
-  if (lane == 0) s_zy[i] = valid ? cap * tanhf(acc * sc / cap) : 0.f;
+  if (lane == 0) s_zy[(int64_t)k * Np + i] = valid ? cap * tanhf(acc * sc / cap) : 0.f;
+}
+
+__device__ __forceinline__ bool target_valid(const int64_t* __restrict__ targets, int64_t ignore_index, int i, int N, int V) {
+  if (i >= N) return false;
+  const int64_t y = targets[i];
+  return (y != ignore_index) && y >= 0 && y < V;
 }
 
 // one thread per row: fold the V-splits, write lse / loss / argmax and the saved row statistics
 __global__ __launch_bounds__(256) void fwd_combine_kernel(const float4* __restrict__ partials, int S, int N, int Np, int V,
                                                          const int64_t* __restrict__ targets, int64_t ignore_index, float cap,
+                                                         const float* __restrict__ mtp_weights, int n_predict,
                                                          float* __restrict__ s_lse, float* __restrict__ s_umax,
                                                          const float* __restrict__ s_zy, float* __restrict__ losses,
                                                          float* __restrict__ lse_out, int32_t* __restrict__ argmax_out) {
@@ -347,10 +356,15 @@ __global__ __launch_bounds__(256) void fwd_combine_kernel(const float4* __restri
     if (o.y > umax || (o.y == umax && ua < uarg)) { umax = o.y; uarg = ua; }
   }
   const float lse = cap + logf(sum);
-  const int64_t y = targets[i];
-  const bool valid = (y != ignore_index) && y >= 0 && y < V;
   s_lse[i] = lse; s_umax[i] = umax;
-  if (losses) losses[i] = valid ? (lse - s_zy[i]) : 0.f;
+  if (losses) {
+    // loss_i = sum_k w_k (lse_i - z[i, y_{i+k}]) over the offsets that take part (tiny/cuda_kernels.py:226-240)
+    float l = 0.f;
+    for (int k = 0; k < n_predict; ++k)
+      if (target_valid(targets, ignore_index, i + k, N, V))
+        l += (mtp_weights ? mtp_weights[k] : 1.0f) * (lse - s_zy[(int64_t)k * Np + i]);
+    losses[i] = l;
+  }
   if (lse_out) lse_out[i] = lse;
   if (argmax_out) argmax_out[i] = (uarg == 0x7fffffff) ? 0 : uarg;
 }
@@ -390,30 +404,42 @@ __global__ __launch_bounds__(1024) void fwd_reduce_kernel(const float* __restric
 // ------------------------------------------------------------------------------------------
 // backward
 // ------------------------------------------------------------------------------------------
-// per row: c_row (exponent offset of G), rho (row scale of G), h (one-hot coefficient)
+// per row: c_row (exponent offset of G), rho (row scale of G), h_k (one-hot coefficients).
+//   dz_iv = g_i ( S_i p_iv - sum_k w_k [v = y_{i+k}] ),  S_i = sum of w_k over the offsets that take part.
 __global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__ s_lse, const float* __restrict__ s_umax,
                                                       const float* __restrict__ s_zy, const int64_t* __restrict__ targets,
                                                       int64_t ignore_index, const int32_t* __restrict__ hdr,
                                                       const float* __restrict__ grad_output, int per_row, float grad_scale,
+                                                      const float* __restrict__ mtp_weights, int n_predict,
                                                       float cap, int N, int Np, int V, float* __restrict__ crow,
                                                       float* __restrict__ rho, float* __restrict__ hcoef,
                                                       float* __restrict__ blockmax) {
   __shared__ float smax[256];
   const int i = blockIdx.x * 256 + threadIdx.x;
-  float c = -INFINITY, r = 0.f, h = 0.f;
+  float c = -INFINITY, r = 0.f;
+  float h[4] = {0.f, 0.f, 0.f, 0.f};
   if (i < N) {
-    const int64_t y = targets[i];
-    const bool valid = (y != ignore_index) && y >= 0 && y < V;
-    if (valid) {
-      const float g = (per_row ? grad_output[i] : grad_output[0] / (float)hdr[0]) * grad_scale;
+    const float g = (per_row ? grad_output[i] : grad_output[0] / (float)hdr[0]) * grad_scale;
+    float sw = 0.f;
+    bool any = false;
+    for (int k = 0; k < n_predict; ++k) {
+      if (!target_valid(targets, ignore_index, i + k, N, V)) continue;
+      const float wk = mtp_weights ? mtp_weights[k] : 1.0f;
+      const float ty = s_zy[(int64_t)k * Np + i] / cap;
+      h[k] = g * wk * (1.0f - ty * ty);
+      sw += wk;
+      any = true;
+    }
+    if (any) {
       const float zmax = cap * tanhf(s_umax[i] / cap);
       c = (cap - zmax) * LOG2E + 10.0f;        // G = 2^c * r(1-r) * e^{z-cap} = 256 (1-t^2) e^{z-zmax}
-      r = g * expf(zmax - s_lse[i]) * (1.0f / 256.0f);
-      const float ty = s_zy[i] / cap;
-      h = g * (1.0f - ty * ty);
+      r = g * sw * expf(zmax - s_lse[i]) * (1.0f / 256.0f);
     }
   }
-  if (i < Np) { crow[i] = c; rho[i] = r; hcoef[i] = h; }
+  if (i < Np) {
+    crow[i] = c; rho[i] = r;
+    for (int k = 0; k < n_predict; ++k) hcoef[(int64_t)k * Np + i] = h[k];
+  }
   smax[threadIdx.x] = fabsf(r);
   __syncthreads();
   for (int w = 128; w > 0; w >>= 1) {
@@ -549,11 +575,12 @@ struct DxParams {
   const uint8_t* ghat;    // [P][Vp]    B side (rows i of the panel)
   const uint8_t* wqt;     // [Vp][dp]   for the one-hot gather
   const float* rho;       // offset to the panel
-  const float* hcoef;     // offset to the panel
+  const float* hcoef;     // [n_predict][Np], offset to the panel
   const int64_t* targets; // offset to the panel
   void* dx;               // offset to the panel's first row
-  int64_t dx_ld, Vp, dp;
+  int64_t dx_ld, Vp, dp, Np;
   int RT, CT, rows, d, V;  // rows: valid rows in this panel
+  int n_predict, rows_left; // rows_left: N - (first row of the panel), bounds the target look-ahead
   float w_s;
 };
 
@@ -572,20 +599,33 @@ __global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p) {
     const int il = rt * 256 + wb * 128 + b * 32 + (lane & 31);
     if (il >= p.rows) continue;
     const float rs = p.rho[il] * p.w_s;
-    const float hs = p.hcoef[il] * p.w_s;
-    const int64_t y = p.targets[il];
-    const uint8_t* wrow = p.wqt + ((hs != 0.f && y >= 0 && y < p.V) ? y : 0) * p.dp;
+    float hs[4];
+    const uint8_t* wrow[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      hs[k] = 0.f; wrow[k] = p.wqt;
+      if (k < p.n_predict && il + k < p.rows_left) {
+        const float hk = p.hcoef[(int64_t)k * p.Np + il] * p.w_s;
+        const int64_t y = p.targets[il + k];
+        if (hk != 0.f && y >= 0 && y < p.V) { hs[k] = hk; wrow[k] = p.wqt + y * p.dp; }
+      }
+    }
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int j = jbase + a * 32 + 8 * q;
         if (j >= p.d) continue;                       // d is a multiple of 4, so j..j+3 are in range together
-        const uint32_t w = *reinterpret_cast<const uint32_t*>(wrow + j);
-        const float o0 = acc[a][b][4 * q + 0] * rs - hs * e4m3_to_float<0>(w);
-        const float o1 = acc[a][b][4 * q + 1] * rs - hs * e4m3_to_float<1>(w);
-        const float o2 = acc[a][b][4 * q + 2] * rs - hs * e4m3_to_float<2>(w);
-        const float o3 = acc[a][b][4 * q + 3] * rs - hs * e4m3_to_float<3>(w);
+        float o0 = acc[a][b][4 * q + 0] * rs, o1 = acc[a][b][4 * q + 1] * rs;
+        float o2 = acc[a][b][4 * q + 2] * rs, o3 = acc[a][b][4 * q + 3] * rs;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          if (k < p.n_predict) {
+            const uint32_t w = *reinterpret_cast<const uint32_t*>(wrow[k] + j);
+            o0 -= hs[k] * e4m3_to_float<0>(w); o1 -= hs[k] * e4m3_to_float<1>(w);
+            o2 -= hs[k] * e4m3_to_float<2>(w); o3 -= hs[k] * e4m3_to_float<3>(w);
+          }
+        }
         T* dst = dx + (int64_t)il * p.dx_ld + j;
         Elem<T>::store(dst + 0, o0); Elem<T>::store(dst + 1, o1);
         Elem<T>::store(dst + 2, o2); Elem<T>::store(dst + 3, o3);
@@ -625,14 +665,17 @@ __global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
   }
 }
 
-// sort keys: target (V for rows that take no part), value = row
-__global__ __launch_bounds__(256) void bwd_keys_kernel(const int64_t* __restrict__ targets, int64_t ignore_index, int N, int V,
-                                                      int32_t* __restrict__ keys, int32_t* __restrict__ vals) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= N) return;
-  const int64_t y = targets[i];
-  keys[i] = ((y != ignore_index) && y >= 0 && y < V) ? (int32_t)y : V;
-  vals[i] = i;
+// sort keys: one entry per (offset k, row i): key = target y_{i+k} (V if the pair takes no part),
+// value = entry id k * Np + i
+__global__ __launch_bounds__(256) void bwd_keys_kernel(const int64_t* __restrict__ targets, int64_t ignore_index, int N, int Np, int V,
+                                                      int n_predict, int32_t* __restrict__ keys, int32_t* __restrict__ vals,
+                                                      int32_t* __restrict__ longlist) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e == 0) longlist[0] = 0;        // counter of the long-column list, filled later on the same stream
+  if (e >= N * n_predict) return;
+  const int k = e / N, i = e - k * N;
+  keys[e] = target_valid(targets, ignore_index, i + k, N, V) ? (int32_t)targets[i + k] : V;
+  vals[e] = k * Np + i;
 }
 
 // segoff[v] = first sorted position whose key >= v, v = 0..V+1
@@ -645,36 +688,54 @@ __global__ __launch_bounds__(256) void bwd_segoff_kernel(const int32_t* __restri
   for (int v = kprev + 1; v <= k; ++v) segoff[v] = pos;
 }
 
-constexpr int LONG_SEG = 64;
+
+// List of the columns that are the target of at least LONG_SEG rows (order irrelevant: each
+// column is handled on its own).  longlist[0] is the count.
+__global__ __launch_bounds__(256) void bwd_longlist_kernel(const int32_t* __restrict__ segoff, int V, int32_t* __restrict__ longlist) {
+  const int v = blockIdx.x * 256 + threadIdx.x;
+  if (v >= V) return;
+  if (segoff[v + 1] - segoff[v] >= LONG_SEG) longlist[1 + atomicAdd(&longlist[0], 1)] = v;
+}
 
 // Columns that are the target of many rows: dwacc[:, v] -= sum_i h_i X_q[i, :] / xi.  One
-// workgroup per (column, block of 256 rows of dW); the rows of the segment are split over 16
-// row-lanes and folded in a fixed order, so the result does not depend on scheduling.
-__global__ __launch_bounds__(256) void bwd_dw_long_kernel(const int32_t* __restrict__ segoff, const int32_t* __restrict__ perm,
-                                                         const float* __restrict__ hcoef, const uint8_t* __restrict__ xq,
-                                                         int64_t dp, int64_t Vp, const float* __restrict__ xi,
-                                                         float* __restrict__ dwacc) {
+// workgroup per (long column, block of 256 rows of dW); the rows of the segment are split over
+// 16 row-lanes (8 independent loads in flight each) and folded in a fixed order, so the result
+// does not depend on scheduling.
+__global__ __launch_bounds__(256) void bwd_dw_long_kernel(const int32_t* __restrict__ longlist, const int32_t* __restrict__ segoff,
+                                                         const int32_t* __restrict__ perm, const float* __restrict__ hcoef,
+                                                         const uint8_t* __restrict__ xq, int64_t dp, int64_t Vp, int Np,
+                                                         const float* __restrict__ xi, float* __restrict__ dwacc) {
   __shared__ float red[16][256];
-  const int v = blockIdx.x;
+  if ((int)blockIdx.x >= longlist[0]) return;
+  const int v = longlist[1 + blockIdx.x];
   const int s0 = segoff[v], L = segoff[v + 1] - s0;
-  if (L < LONG_SEG) return;
   const int t = threadIdx.x, c = t & 15, rl = t >> 4;
   const int64_t jb = (int64_t)blockIdx.y * 256;
   float a[16];
 #pragma unroll
   for (int m = 0; m < 16; ++m) a[m] = 0.f;
   if (jb + c * 16 < dp) {
-    for (int n = rl; n < L; n += 16) {
-      const int i = perm[s0 + n];
-      const float h = hcoef[i];
-      const v4i raw = *reinterpret_cast<const v4i*>(xq + (int64_t)i * dp + jb + c * 16);
+    const uint8_t* xcol = xq + jb + c * 16;
+    for (int n0 = rl; n0 < L; n0 += 16 * 8) {
+      v4i raw[8];
+      float h[8];
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        const uint32_t w = (uint32_t)raw[m];
-        a[4 * m + 0] = fmaf(h, e4m3_to_float<0>(w), a[4 * m + 0]);
-        a[4 * m + 1] = fmaf(h, e4m3_to_float<1>(w), a[4 * m + 1]);
-        a[4 * m + 2] = fmaf(h, e4m3_to_float<2>(w), a[4 * m + 2]);
-        a[4 * m + 3] = fmaf(h, e4m3_to_float<3>(w), a[4 * m + 3]);
+      for (int u = 0; u < 8; ++u) {
+        const int n = n0 + 16 * u;
+        const int e = n < L ? perm[s0 + n] : -1;          // entry id k * Np + i
+        h[u] = e >= 0 ? hcoef[e] : 0.f;
+        raw[u] = *reinterpret_cast<const v4i*>(xcol + (int64_t)(e >= 0 ? e % Np : 0) * dp);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {        // rows in ascending order within a row-lane
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          const uint32_t w = (uint32_t)raw[u][m];
+          a[4 * m + 0] = fmaf(h[u], e4m3_to_float<0>(w), a[4 * m + 0]);
+          a[4 * m + 1] = fmaf(h[u], e4m3_to_float<1>(w), a[4 * m + 1]);
+          a[4 * m + 2] = fmaf(h[u], e4m3_to_float<2>(w), a[4 * m + 2]);
+          a[4 * m + 3] = fmaf(h[u], e4m3_to_float<3>(w), a[4 * m + 3]);
+        }
       }
     }
   }
@@ -693,7 +754,7 @@ __global__ __launch_bounds__(256) void bwd_dw_long_kernel(const int32_t* __restr
 template <typename T>
 __global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restrict__ dwacc, int nparts, int64_t part_stride, int64_t Vp, const int32_t* __restrict__ segoff,
                                                           const int32_t* __restrict__ perm, const float* __restrict__ hcoef,
-                                                          const uint8_t* __restrict__ xq, int64_t dp, const float* __restrict__ xi,
+                                                          const uint8_t* __restrict__ xq, int64_t dp, int Np, const float* __restrict__ xi,
                                                           float x_s, int d, int V, T* __restrict__ dw, int64_t dw_ld) {
   const int t = threadIdx.x;
   const int v = blockIdx.x * 64 + (t & 63);
@@ -710,9 +771,9 @@ __global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restri
   const int s0 = segoff[v], L = segoff[v + 1] - s0;
   if (L > 0 && L < LONG_SEG) {
     for (int n = 0; n < L; ++n) {
-      const int i = perm[s0 + n];
-      const float h = hcoef[i] * x_s;
-      const v4i raw = *reinterpret_cast<const v4i*>(xq + (int64_t)i * dp + j0);
+      const int e = perm[s0 + n];                         // entry id k * Np + i
+      const float h = hcoef[e] * x_s;
+      const v4i raw = *reinterpret_cast<const v4i*>(xq + (int64_t)(e % Np) * dp + j0);
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
         const uint32_t w = (uint32_t)raw[m];
@@ -834,7 +895,7 @@ static int check_shape(const sce_shape* s) {
   if (s->d % 16 != 0) return fail(SCE_EINVAL, "d = %lld must be a multiple of 16", (long long)s->d);
   if (s->N > (1ll << 24) - 256 || s->V > (1ll << 24) - 256 || s->d > (1ll << 24) - 256)
     return fail(SCE_EINVAL, "N, d and V must be below 2^24 (32-bit tile offsets)");
-  if (s->n_predict != 1) return fail(SCE_EINVAL, "n_predict = %d: only a single offset is built into the kernels", s->n_predict);
+  if (s->n_predict < 1 || s->n_predict > 4) return fail(SCE_EINVAL, "n_predict = %d must be between 1 and 4", s->n_predict);
   return SCE_OK;
 }
 
@@ -846,21 +907,22 @@ static size_t sort_tmp_bytes(int64_t N, int64_t V) {
   return bytes;
 }
 
-static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int nparts) {
+static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int nparts, int K) {
   BwdLayout B;
   B.P = P; B.Pw = Pw; B.nparts = nparts;
   size_t o = 0;
   auto take = [&](size_t bytes) { size_t r = o; o += (bytes + 255) / 256 * 256; return r; };
   B.off_crow = take((size_t)S.Np * 4);
   B.off_rho = take((size_t)S.Np * 4);
-  B.off_hcoef = take((size_t)S.Np * 4);
+  B.off_hcoef = take((size_t)S.Np * 4 * K);
   B.off_blockmax = take((size_t)(S.Np / 256) * 4);
   B.off_xi = take(256);
   B.off_xt = take((size_t)S.dq * S.Np);
-  B.off_perm = take((size_t)S.N * 4 * 2);      // sorted values + unsorted values
-  B.off_keys = take((size_t)S.N * 4 * 2);      // sorted keys + unsorted keys
+  B.off_perm = take((size_t)S.N * K * 4 * 2);  // sorted values + unsorted values, one entry per (offset, row)
+  B.off_keys = take((size_t)S.N * K * 4 * 2);  // sorted keys + unsorted keys
   B.off_segoff = take((size_t)(S.V + 2) * 4);
-  B.sorttmp_bytes = sort_tmp_bytes(S.N, S.V);
+  B.off_longlist = take((size_t)(S.N * K / LONG_SEG + 2) * 4);
+  B.sorttmp_bytes = sort_tmp_bytes(S.N * K, S.V);
   B.off_sorttmp = take(B.sorttmp_bytes);
   B.fixed = o;
   B.off_ghat = take((size_t)P * S.Vp);
@@ -936,11 +998,11 @@ extern "C" int sce_sizes_for(const sce_shape* shape, sce_sizes* out) {
   const SavedLayout S = saved_layout(shape->N, shape->d, shape->V, shape->n_predict);
   out->saved_bytes = S.total;
   out->fwd_workspace_bytes = (size_t)8 * S.Np * 16 + 256;
-  out->bwd_workspace_min_bytes = bwd_layout(S, 256, 256, 1).total;
+  out->bwd_workspace_min_bytes = bwd_layout(S, 256, 256, 1, shape->n_predict).total;
   out->bwd_panel_rows = default_panel(S);
   {
     const int64_t Pw = default_dw_panel(S, out->bwd_panel_rows);
-    out->bwd_workspace_bytes = bwd_layout(S, out->bwd_panel_rows, Pw, dw_launches(S, Pw)).total;
+    out->bwd_workspace_bytes = bwd_layout(S, out->bwd_panel_rows, Pw, dw_launches(S, Pw), shape->n_predict).total;
   }
   return SCE_OK;
 }
@@ -1002,6 +1064,8 @@ extern "C" int sce_forward(const sce_args* a) {
   if (a->x_ld < d || a->w_ld < V) return fail(SCE_EINVAL, "row strides smaller than the row length");
   if (a->reduction == SCE_REDUCE_NONE && !a->losses) return fail(SCE_EINVAL, "losses is NULL with reduction = none");
   if (a->reduction == SCE_REDUCE_MEAN && !a->loss) return fail(SCE_EINVAL, "loss is NULL with reduction = mean");
+  if (a->reduction == SCE_REDUCE_MEAN && a->shape.n_predict != 1)
+    return fail(SCE_EINVAL, "reduction = mean is defined for a single offset only; use reduction = none with n_predict > 1");
   const SavedLayout S = saved_layout(N, d, V, a->shape.n_predict);
   if (a->saved_bytes < S.total) return fail(SCE_EINVAL, "saved buffer too small: %zu < %zu", a->saved_bytes, S.total);
   const int RT = (int)(S.Np / 256), CT = (int)(S.Vp / 256);
@@ -1044,10 +1108,11 @@ extern "C" int sce_forward(const sce_args* a) {
   float* s_lse = (float*)(sv + S.off_lse);
   float* s_umax = (float*)(sv + S.off_umax);
   float* s_zy = (float*)(sv + S.off_zy);
-  fwd_target_logit_kernel<<<(int)((N + 3) / 4), 256, 0, st>>>(xq, wqt, S.dp, a->targets, a->ignore_index, (int)N, (int)V,
-                                                           a->x_s * a->w_s, a->cap, s_zy);
+  fwd_target_logit_kernel<<<dim3((unsigned)((N + 3) / 4), (unsigned)a->shape.n_predict), 256, 0, st>>>(
+      xq, wqt, S.dp, a->targets, a->ignore_index, (int)N, (int)S.Np, (int)V, a->x_s * a->w_s, a->cap, s_zy);
   fwd_combine_kernel<<<(int)(S.Np / 256), 256, 0, st>>>(p.partials, nsplit, (int)N, (int)S.Np, (int)V, a->targets, a->ignore_index,
-                                                       a->cap, s_lse, s_umax, s_zy, a->losses, a->lse, a->argmax);
+                                                       a->cap, a->mtp_weights, a->shape.n_predict, s_lse, s_umax, s_zy, a->losses, a->lse,
+                                                       a->argmax);
   fwd_reduce_kernel<<<1, 1024, 0, st>>>(s_lse, s_zy, a->targets, a->ignore_index, (int)N, (int)V, (int32_t*)(sv + S.off_hdr),
                                         a->reduction == SCE_REDUCE_MEAN ? a->loss : nullptr, a->n_valid);
   HIP_TRY(hipGetLastError());
@@ -1065,7 +1130,8 @@ extern "C" int sce_backward(const sce_args* a) {
   const SavedLayout S = saved_layout(N, d, V, a->shape.n_predict);
   if (a->saved_bytes < S.total) return fail(SCE_EINVAL, "saved buffer too small: %zu < %zu", a->saved_bytes, S.total);
   if (!a->workspace) return fail(SCE_EINVAL, "workspace is NULL");
-  const BwdLayout Bmin = bwd_layout(S, 256, 256, 1);
+  const int K = a->shape.n_predict;
+  const BwdLayout Bmin = bwd_layout(S, 256, 256, 1, K);
   if (a->workspace_bytes < Bmin.total) return fail(SCE_EINVAL, "backward workspace too small: %zu < %zu", a->workspace_bytes, Bmin.total);
   // panel sizes from what the caller gave: P rows per recompute/dX panel, Pw = m * P rows per dW launch
   const size_t room = (a->workspace_bytes - Bmin.fixed - Bmin.part_stride) / (size_t)S.Vp;     // rows of e4m3 scratch available
@@ -1080,8 +1146,8 @@ extern "C" int sce_backward(const sce_args* a) {
   if ((int64_t)room - P < Pw) Pw = ((int64_t)room - P) / P * P;
   if (Pw < P) return fail(SCE_EINVAL, "internal: dW panel smaller than the dX panel");
   int nparts = dw_launches(S, Pw);
-  while (nparts > 1 && bwd_layout(S, P, Pw, nparts).total > a->workspace_bytes) --nparts;
-  const BwdLayout B = bwd_layout(S, P, Pw, nparts);
+  while (nparts > 1 && bwd_layout(S, P, Pw, nparts, K).total > a->workspace_bytes) --nparts;
+  const BwdLayout B = bwd_layout(S, P, Pw, nparts, K);
   if (B.total > a->workspace_bytes) return fail(SCE_EINVAL, "internal: panel layout exceeds workspace");
   DeviceGuard guard(a->device);
   if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", a->device);
@@ -1103,18 +1169,20 @@ extern "C" int sce_backward(const sce_args* a) {
   uint8_t* xt = ws + B.off_xt;
   float* dwacc = (float*)(ws + B.off_dwacc);
   int32_t* perm = (int32_t*)(ws + B.off_perm);
-  int32_t* vals_in = perm + N;
+  const int64_t NE = N * K;            // one-hot entries: one per (offset, row)
+  int32_t* vals_in = perm + NE;
   int32_t* skeys = (int32_t*)(ws + B.off_keys);
-  int32_t* keys_in = skeys + N;
+  int32_t* keys_in = skeys + NE;
   int32_t* segoff = (int32_t*)(ws + B.off_segoff);
+  int32_t* longlist = (int32_t*)(ws + B.off_longlist);
   uint8_t* ghat = ws + B.off_ghat;
   uint8_t* ghat_t = ws + B.off_ghat_t;
 
   const int nblk = (int)(S.Np / 256);
   KernelTimer* tm_prep = new KernelTimer(SCE_K_BWD_PREP, st);
   bwd_prep_kernel<<<nblk, 256, 0, st>>>(s_lse, s_umax, s_zy, a->targets, a->ignore_index, hdr, a->grad_output,
-                                        a->reduction == SCE_REDUCE_NONE ? 1 : 0, a->grad_scale, a->cap, (int)N, (int)S.Np, (int)V,
-                                        crow, rho, hcoef, blockmax);
+                                        a->reduction == SCE_REDUCE_NONE ? 1 : 0, a->grad_scale, a->mtp_weights, K, a->cap, (int)N,
+                                        (int)S.Np, (int)V, crow, rho, hcoef, blockmax);
   bwd_xi_kernel<<<1, 1024, 0, st>>>(blockmax, nblk, xi);
   {
     dim3 g((unsigned)(S.Np / 64), (unsigned)(S.dq / 64));
@@ -1122,13 +1190,14 @@ extern "C" int sce_backward(const sce_args* a) {
   }
   // rows grouped by target, for the one-hot part of dW
   {
-    bwd_keys_kernel<<<(int)((N + 255) / 256), 256, 0, st>>>(a->targets, a->ignore_index, (int)N, (int)V, keys_in, vals_in);
+    bwd_keys_kernel<<<(int)((NE + 255) / 256), 256, 0, st>>>(a->targets, a->ignore_index, (int)N, (int)S.Np, (int)V, K, keys_in, vals_in, longlist);
     int bits = 1;
     while ((1ll << bits) <= V) ++bits;
     size_t tmp = B.sorttmp_bytes;
-    if (sce::sort_pairs(ws + B.off_sorttmp, &tmp, keys_in, skeys, vals_in, perm, (size_t)N, bits, st) != 0)
+    if (sce::sort_pairs(ws + B.off_sorttmp, &tmp, keys_in, skeys, vals_in, perm, (size_t)NE, bits, st) != 0)
     { delete tm_prep; return fail(SCE_EHIP, "radix sort of the targets failed"); }
-    bwd_segoff_kernel<<<(int)((N + 256) / 256), 256, 0, st>>>(skeys, (int)N, (int)V, segoff);
+    bwd_segoff_kernel<<<(int)((NE + 256) / 256), 256, 0, st>>>(skeys, (int)NE, (int)V, segoff);
+    bwd_longlist_kernel<<<(int)((V + 255) / 256), 256, 0, st>>>(segoff, (int)V, longlist);
   }
   delete tm_prep;
   const float k1 = a->x_s * a->w_s * 2.0f * LOG2E / a->cap, c2 = -2.0f * a->cap * LOG2E;
@@ -1148,7 +1217,8 @@ extern "C" int sce_backward(const sce_args* a) {
 
     DxParams dp_;
     dp_.wq = wq; dp_.ghat = ghat; dp_.wqt = wqt; dp_.rho = rho + p0; dp_.hcoef = hcoef + p0; dp_.targets = a->targets + p0;
-    dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.dp = S.dp; dp_.RT = RTp; dp_.CT = CTd;
+    dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.dp = S.dp; dp_.Np = S.Np; dp_.RT = RTp; dp_.CT = CTd;
+    dp_.n_predict = K; dp_.rows_left = (int)(N - p0 > 0 ? N - p0 : 0);
     dp_.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); dp_.d = (int)d; dp_.V = (int)V; dp_.w_s = a->w_s;
     {
       KernelTimer tm(SCE_K_DX, st);
@@ -1177,14 +1247,14 @@ extern "C" int sce_backward(const sce_args* a) {
     }
   }
   KernelTimer tm_fin(SCE_K_DW_FINAL, st);
-  bwd_dw_long_kernel<<<dim3((unsigned)V, (unsigned)(S.dq / 256)), 256, 0, st>>>(segoff, perm, hcoef, xq, S.dp, S.Vp, xi, dwacc);
+  bwd_dw_long_kernel<<<dim3((unsigned)(NE / LONG_SEG + 1), (unsigned)(S.dq / 256)), 256, 0, st>>>(longlist, segoff, perm, hcoef, xq, S.dp, S.Vp, (int)S.Np, xi, dwacc);
   {
     dim3 g((unsigned)((V + 63) / 64), (unsigned)((d + 63) / 64));
     if (a->dw_dtype == SCE_F32)
-      bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.dp, xi, a->x_s, (int)d, (int)V,
+      bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.dp, (int)S.Np, xi, a->x_s, (int)d, (int)V,
                                                    (float*)a->dw, a->dw_ld);
     else
-      bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.dp, xi, a->x_s, (int)d, (int)V,
+      bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.dp, (int)S.Np, xi, a->x_s, (int)d, (int)V,
                                                     (bf16_t*)a->dw, a->dw_ld);
   }
   HIP_TRY(hipGetLastError());

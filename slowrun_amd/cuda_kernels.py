@@ -16,6 +16,9 @@ Differences from the reference that a caller can see:
   * ``reduction='mean'`` is available (mean over rows whose target is not -1, like
     F.cross_entropy(ignore_index=-1) in the eager head, tiny/train.py:743);
   * rows with target -1 give loss 0 and zero gradient;
+  * up to 4 multi-token-prediction offsets (``mtp_weights``), with the offsets that run past
+    the end of the target vector or hit a -1 target left out of both the loss and the gradient
+    (the reference kernel leaves them out of the loss only, tiny/cuda_kernels.py:233,242-246);
   * ``grad_s`` is accepted and unused: the reference needs it to fit dlogits into
     e5m2 (tiny/cuda_kernels.py:265); here each row of the on-chip dlogits carries its
     own scale;
@@ -54,14 +57,24 @@ def _stream_ptr(device):
     return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
-def _base_args(x_like, N, d, V, x_s, w_s, cap, grad_scale, reduction, targets):
+def _mtp(mtp_weights, device):
+    """(n_predict, float32 device tensor or None).  None means a single offset of weight 1."""
+    if mtp_weights is None:
+        return 1, None
+    w = mtp_weights.detach().to(device=device, dtype=torch.float32).contiguous().reshape(-1)
+    if not 1 <= w.numel() <= 4:
+        raise ValueError(f"mtp_weights must hold 1 to 4 offsets, got {w.numel()}")
+    return w.numel(), w
+
+
+def _base_args(x_like, N, d, V, x_s, w_s, cap, grad_scale, reduction, targets, n_predict=1, mtp_w=None):
     a = SceArgs()
     a.struct_size = C.sizeof(SceArgs)
     a.device = x_like.device.index if x_like.device.index is not None else torch.cuda.current_device()
     a.stream = _stream_ptr(x_like.device)
-    a.shape = SceShape(N, d, V, 1, 0)
+    a.shape = SceShape(N, d, V, n_predict, 0)
     a.targets = targets.data_ptr()
-    a.mtp_weights = None
+    a.mtp_weights = mtp_w.data_ptr() if mtp_w is not None else None
     a.x_s, a.w_s, a.cap, a.grad_scale = x_s, w_s, cap, grad_scale
     a.ignore_index = IGNORE_INDEX
     a.reduction = _lib.SCE_REDUCE_MEAN if reduction == "mean" else _lib.SCE_REDUCE_NONE
@@ -77,16 +90,19 @@ def _check_inputs(x, w, targets):
         raise ValueError("targets must be int64 of shape (N,)")
 
 
-def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False):
+def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_weights=None):
     """One call of sce_forward.  Returns (out, saved, lse, argmax, n_valid)."""
     _check_inputs(x, w, targets)
+    n_predict, mtp_w = _mtp(mtp_weights, x.device)
+    if n_predict > 1 and reduction != "none":
+        raise ValueError("multi-token prediction returns per-row losses: use reduction='none'")
     x = x if x.stride(1) == 1 else x.contiguous()
     w = w if w.stride(1) == 1 else w.contiguous()
     targets = targets.contiguous()
     N, d = x.shape
     V = w.shape[1]
     dev = x.device
-    sz = _lib.sizes_for(N, d, V)
+    sz = _lib.sizes_for(N, d, V, n_predict)
     saved = torch.empty(sz.saved_bytes, dtype=torch.uint8, device=dev)
     ws = torch.empty(sz.fwd_workspace_bytes, dtype=torch.uint8, device=dev)
     losses = torch.empty(N, dtype=torch.float32, device=dev)
@@ -94,7 +110,7 @@ def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False):
     loss = torch.empty(1, dtype=torch.float32, device=dev)
     n_valid = torch.empty(2, dtype=torch.int32, device=dev)
     argmax = torch.empty(N, dtype=torch.int32, device=dev) if want_argmax else None
-    a = _base_args(x, N, d, V, x_s, w_s, cap, 1.0, reduction, targets)
+    a = _base_args(x, N, d, V, x_s, w_s, cap, 1.0, reduction, targets, n_predict, mtp_w)
     a.x, a.x_dtype, a.x_ld = x.data_ptr(), _dtype_code(x, "x"), x.stride(0)
     a.w, a.w_dtype, a.w_ld = w.data_ptr(), _dtype_code(w, "lm_head_weight"), w.stride(0)
     a.loss, a.losses, a.lse, a.n_valid = loss.data_ptr(), losses.data_ptr(), lse.data_ptr(), n_valid.data_ptr()
@@ -107,10 +123,11 @@ def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False):
 
 
 def ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale, reduction, x_dtype, w_dtype,
-                panel_rows=0, workspace_bytes=None):
+                panel_rows=0, workspace_bytes=None, mtp_weights=None):
     """One call of sce_backward.  Returns (dx (N,d) in x_dtype, dw (d,V) in w_dtype)."""
     dev = saved.device
-    sz = _lib.sizes_for(N, d, V)
+    n_predict, mtp_w = _mtp(mtp_weights, dev)
+    sz = _lib.sizes_for(N, d, V, n_predict)
     nbytes = sz.bwd_workspace_bytes if workspace_bytes is None else workspace_bytes
     ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     dx = torch.empty(N, d, dtype=x_dtype, device=dev)
@@ -121,7 +138,7 @@ def ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale,
             raise ValueError("grad_output must be a scalar for reduction='mean'")
     elif go.numel() != N:
         raise ValueError("grad_output must have one element per row for reduction='none'")
-    a = _base_args(saved, N, d, V, x_s, w_s, cap, grad_scale, reduction, targets)
+    a = _base_args(saved, N, d, V, x_s, w_s, cap, grad_scale, reduction, targets, n_predict, mtp_w)
     a.saved, a.saved_bytes = saved.data_ptr(), saved.numel()
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
     a.grad_output = go.data_ptr()
@@ -137,23 +154,22 @@ class FusedSoftcappedCrossEntropy(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, targets, mtp_weights, lm_head_weight, x_s, w_s, grad_s, grad_scale, cap=15.0, reduction="none"):
-        if mtp_weights is not None and mtp_weights.numel() != 1:
-            raise NotImplementedError("multi-token prediction (more than one offset) is not built into the kernels yet")
         if reduction not in ("none", "mean"):
             raise ValueError("reduction must be 'none' or 'mean'")
-        w0 = 1.0 if mtp_weights is None else float(mtp_weights.reshape(-1)[0])
         xs, ws_ = _scale_value(x_s, x), _scale_value(w_s, lm_head_weight)
-        out, saved, _lse, _am, _nv = ce_forward(x.detach(), lm_head_weight.detach(), targets, xs, ws_, float(cap), reduction)
-        ctx.save_for_backward(saved, targets)
-        ctx.params = (x.shape[0], x.shape[1], lm_head_weight.shape[1], xs, ws_, float(cap), float(grad_scale) * w0,
-                      reduction, x.dtype, lm_head_weight.dtype)
-        return out * w0 if w0 != 1.0 else out
+        out, saved, _lse, _am, _nv = ce_forward(x.detach(), lm_head_weight.detach(), targets, xs, ws_, float(cap), reduction,
+                                                mtp_weights=mtp_weights)
+        ctx.save_for_backward(saved, targets, mtp_weights if mtp_weights is not None else torch.empty(0, device=x.device))
+        ctx.params = (x.shape[0], x.shape[1], lm_head_weight.shape[1], xs, ws_, float(cap), float(grad_scale),
+                      reduction, x.dtype, lm_head_weight.dtype, mtp_weights is not None)
+        return out
 
     @staticmethod
     def backward(ctx, grad_output):
-        saved, targets = ctx.saved_tensors
-        N, d, V, xs, ws_, cap, gscale, reduction, x_dtype, w_dtype = ctx.params
-        dx, dw = ce_backward(saved, targets, grad_output, N, d, V, xs, ws_, cap, gscale, reduction, x_dtype, w_dtype)
+        saved, targets, mtp_w = ctx.saved_tensors
+        N, d, V, xs, ws_, cap, gscale, reduction, x_dtype, w_dtype, has_mtp = ctx.params
+        dx, dw = ce_backward(saved, targets, grad_output, N, d, V, xs, ws_, cap, gscale, reduction, x_dtype, w_dtype,
+                             mtp_weights=mtp_w if has_mtp else None)
         return dx, None, None, dw, None, None, None, None, None, None
 
 

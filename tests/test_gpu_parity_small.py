@@ -97,3 +97,26 @@ def test_autograd_function_signature():
     ref = eager.softcapped_ce(x.detach(), w.detach(), y, inp.x_s, inp.w_s, cap=15.0, reduction="none")
     assert float((losses.detach() - ref["loss"]).abs().max() / ref["loss"].abs().max()) < 1e-3
     assert pu.cosine(x.grad.float(), ref["dx"]) > pu.GRAD_COS and pu.cosine(w.grad.float(), ref["dw"]) > pu.GRAD_COS
+
+
+@pytest.mark.parametrize("weights", [[1.0], [1.0, 0.5, 0.25], [1.0, 0.5, 0.25, 0.125], [1.0, 0.0, 0.0]])
+def test_multi_token_prediction(weights):
+    """Per-row MTP losses and gradients against the oracle (tiny/cuda_kernels.py:226-301 semantics with the
+    offsets that take no part left out of the gradient as well)."""
+    from oracle import eager
+    from slowrun_amd.cuda_kernels import FusedSoftcappedCrossEntropy
+    inp = _small("irregular", 777, 128, 1300)        # has -1 targets, so some offsets drop out
+    x = inp.x.cuda().bfloat16().requires_grad_(True)
+    w = inp.w.cuda().bfloat16().requires_grad_(True)
+    y = inp.targets.cuda()
+    mw = torch.tensor(weights, device="cuda")
+    go = torch.rand(777, generator=torch.Generator().manual_seed(3)).cuda() / 777
+    losses = FusedSoftcappedCrossEntropy.apply(x, y, mw, w, inp.x_s, inp.w_s, 0.75 / 448, 1.0, inp.cap)   # trainer call
+    (losses * go).sum().backward()
+    ref = eager.softcapped_ce_mtp(x.detach(), w.detach(), y, weights, inp.x_s, inp.w_s, cap=inp.cap, grad_output=go)
+    assert float((losses.detach() - ref["loss"]).abs().max() / ref["loss"].abs().max()) < pu.LOSS_RTOL
+    for got, want in ((x.grad, ref["dx"]), (w.grad, ref["dw"])):
+        assert pu.maxrel(got.float(), want) <= pu.GRAD_MAXREL and pu.cosine(got.float(), want) > pu.GRAD_COS
+    if weights == [1.0, 0.0, 0.0]:
+        plain = FusedSoftcappedCrossEntropy.apply(x.detach(), y, None, w.detach(), inp.x_s, inp.w_s, 0.75 / 448, 1.0, inp.cap)
+        assert torch.equal(plain, losses.detach())
