@@ -26,6 +26,7 @@ Differences from the reference that a caller can see:
     not its mean (tiny/cuda_kernels.py:412 assumes it is uniform).
 """
 import ctypes as C
+from typing import Optional, Tuple
 
 import torch
 
@@ -149,6 +150,43 @@ def ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale,
     return dx, dw
 
 
+# ---------------------------------------------------------------------------------------------
+# torch.library custom ops, so that a torch.compile'd model (tiny/train.py:1254) traces the loss head
+# as two opaque calls instead of breaking the graph; the reference wraps its kernel the same way
+# (tiny/cuda_kernels.py:314).  The fake implementations only describe shapes and dtypes.
+# ---------------------------------------------------------------------------------------------
+@torch.library.custom_op("slowrun_amd::ce_forward", mutates_args=())
+def ce_forward_op(x: torch.Tensor, w: torch.Tensor, targets: torch.Tensor, mtp_weights: Optional[torch.Tensor],
+                  x_s: float, w_s: float, cap: float, mean: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    out, saved, _lse, _am, _nv = ce_forward(x, w, targets, x_s, w_s, cap, "mean" if mean else "none", mtp_weights=mtp_weights)
+    return out, saved
+
+
+@ce_forward_op.register_fake
+def _ce_forward_fake(x, w, targets, mtp_weights, x_s, w_s, cap, mean):
+    N, d = x.shape
+    V = w.shape[1]
+    n_predict = 1 if mtp_weights is None else mtp_weights.numel()
+    sz = _lib.sizes_for(N, d, V, n_predict)
+    out = x.new_empty((), dtype=torch.float32) if mean else x.new_empty((N,), dtype=torch.float32)
+    return out, x.new_empty((sz.saved_bytes,), dtype=torch.uint8)
+
+
+@torch.library.custom_op("slowrun_amd::ce_backward", mutates_args=())
+def ce_backward_op(saved: torch.Tensor, targets: torch.Tensor, grad_output: torch.Tensor, mtp_weights: Optional[torch.Tensor],
+                   N: int, d: int, V: int, x_s: float, w_s: float, cap: float, grad_scale: float, mean: bool,
+                   x_bf16: bool, w_bf16: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    return ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale, "mean" if mean else "none",
+                       torch.bfloat16 if x_bf16 else torch.float32, torch.bfloat16 if w_bf16 else torch.float32,
+                       mtp_weights=mtp_weights)
+
+
+@ce_backward_op.register_fake
+def _ce_backward_fake(saved, targets, grad_output, mtp_weights, N, d, V, x_s, w_s, cap, grad_scale, mean, x_bf16, w_bf16):
+    return (saved.new_empty((N, d), dtype=torch.bfloat16 if x_bf16 else torch.float32),
+            saved.new_empty((d, V), dtype=torch.bfloat16 if w_bf16 else torch.float32))
+
+
 class FusedSoftcappedCrossEntropy(torch.autograd.Function):
     """Same call as tiny/cuda_kernels.py:336-414; see the module docstring."""
 
@@ -156,20 +194,23 @@ class FusedSoftcappedCrossEntropy(torch.autograd.Function):
     def forward(ctx, x, targets, mtp_weights, lm_head_weight, x_s, w_s, grad_s, grad_scale, cap=15.0, reduction="none"):
         if reduction not in ("none", "mean"):
             raise ValueError("reduction must be 'none' or 'mean'")
+        _dtype_code(x, "x")
+        _dtype_code(lm_head_weight, "lm_head_weight")
         xs, ws_ = _scale_value(x_s, x), _scale_value(w_s, lm_head_weight)
-        out, saved, _lse, _am, _nv = ce_forward(x.detach(), lm_head_weight.detach(), targets, xs, ws_, float(cap), reduction,
-                                                mtp_weights=mtp_weights)
+        out, saved = ce_forward_op(x.detach(), lm_head_weight.detach(), targets, mtp_weights, xs, ws_, float(cap),
+                                   reduction == "mean")
         ctx.save_for_backward(saved, targets, mtp_weights if mtp_weights is not None else torch.empty(0, device=x.device))
         ctx.params = (x.shape[0], x.shape[1], lm_head_weight.shape[1], xs, ws_, float(cap), float(grad_scale),
-                      reduction, x.dtype, lm_head_weight.dtype, mtp_weights is not None)
+                      reduction == "mean", x.dtype == torch.bfloat16, lm_head_weight.dtype == torch.bfloat16,
+                      mtp_weights is not None)
         return out
 
     @staticmethod
     def backward(ctx, grad_output):
         saved, targets, mtp_w = ctx.saved_tensors
-        N, d, V, xs, ws_, cap, gscale, reduction, x_dtype, w_dtype, has_mtp = ctx.params
-        dx, dw = ce_backward(saved, targets, grad_output, N, d, V, xs, ws_, cap, gscale, reduction, x_dtype, w_dtype,
-                             mtp_weights=mtp_w if has_mtp else None)
+        N, d, V, xs, ws_, cap, gscale, mean, x_bf16, w_bf16, has_mtp = ctx.params
+        dx, dw = ce_backward_op(saved, targets, grad_output.contiguous(), mtp_w if has_mtp else None, N, d, V, xs, ws_, cap,
+                                gscale, mean, x_bf16, w_bf16)
         return dx, None, None, dw, None, None, None, None, None, None
 
 

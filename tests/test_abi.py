@@ -63,7 +63,7 @@ def test_sizes_for_and_shape_errors(lib):
     for bad in [(0, 128, 100), (10, 100, 100), (10, 128, 0), (1 << 25, 128, 100)]:
         with pytest.raises(RuntimeError):
             _lib.sizes_for(*bad)
-    shape = _lib.SceShape(10, 128, 100, 3, 0)
+    shape = _lib.SceShape(10, 128, 100, 5, 0)          # at most 4 multi-token-prediction offsets
     out = _lib.SceSizes()
     assert lib.sce_sizes_for(C.byref(shape), C.byref(out)) == 1
     assert b"n_predict" in lib.sce_last_error()
@@ -97,3 +97,21 @@ def test_python_wrapper_refuses_cpu_tensors():
     y = torch.randint(0, 32, (8,))
     with pytest.raises(RuntimeError, match="GPU"):
         FusedSoftcappedCrossEntropy.apply(x, y, None, w, 1.0, 1.0, 1.0, 1.0)
+
+
+def test_custom_ops_have_fake_implementations():
+    """torch.compile traces the loss head through slowrun_amd::ce_forward / ce_backward; their fake
+    implementations must give the shapes and dtypes of the real ones (checked here on meta tensors)."""
+    import torch
+    from slowrun_amd import cuda_kernels as ck
+    x = torch.empty(512, 128, dtype=torch.bfloat16, device="meta")
+    w = torch.empty(128, 1024, dtype=torch.bfloat16, device="meta")
+    y = torch.empty(512, dtype=torch.int64, device="meta")
+    mw = torch.empty(3, dtype=torch.float32, device="meta")
+    out, saved = ck.ce_forward_op(x, w, y, mw, 0.1, 0.1, 15.0, False)
+    assert out.shape == (512,) and out.dtype == torch.float32
+    assert saved.dtype == torch.uint8 and saved.numel() == _lib.sizes_for(512, 128, 1024, 3).saved_bytes
+    out2, _ = ck.ce_forward_op(x, w, y, None, 0.1, 0.1, 15.0, True)
+    assert out2.shape == ()
+    dx, dw = ck.ce_backward_op(saved, y, out, mw, 512, 128, 1024, 0.1, 0.1, 15.0, 1.0, False, True, False)
+    assert dx.shape == (512, 128) and dx.dtype == torch.bfloat16 and dw.shape == (128, 1024) and dw.dtype == torch.float32

@@ -120,3 +120,27 @@ def test_multi_token_prediction(weights):
     if weights == [1.0, 0.0, 0.0]:
         plain = FusedSoftcappedCrossEntropy.apply(x.detach(), y, None, w.detach(), inp.x_s, inp.w_s, 0.75 / 448, 1.0, inp.cap)
         assert torch.equal(plain, losses.detach())
+
+
+def test_traced_by_torch_compile():
+    """The trainer wraps its model in torch.compile (tiny/train.py:1254): the loss head must trace without
+    a graph break and give the eager result."""
+    from slowrun_amd.cuda_kernels import FusedSoftcappedCrossEntropy
+    inp = _small("tiny_track", 512, 128, 1024)
+    x0 = inp.x.cuda().bfloat16()
+    w0 = inp.w.cuda().bfloat16()
+    y = inp.targets.cuda()
+    mw = torch.tensor([1.0, 0.5], device="cuda")
+
+    def head(x, w):
+        h = x * 1.0
+        return FusedSoftcappedCrossEntropy.apply(h, y, mw, w, inp.x_s, inp.w_s, 0.75 / 448, 1.0).mean()
+
+    res = []
+    for fn in (head, torch.compile(head, fullgraph=True, dynamic=False)):
+        x = x0.clone().requires_grad_(True)
+        w = w0.clone().requires_grad_(True)
+        loss = fn(x, w)
+        loss.backward()
+        res.append((loss.detach(), x.grad, w.grad))
+    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1]) and torch.equal(res[0][2], res[1][2])
