@@ -17,6 +17,11 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP8_TFLOPS = 5000.0        # MI355X dense fp8 MFMA, published
 
+# HBM-side bytes per launch (fetched + written) of the MFMA kernels at the full limited_2p7b shape, from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB device copy (factors 2.0 / 1.0); the
+# summary is profiles/bench_limited_2p7b_pmc.txt.  None for any other workload.
+MEASURED_TRAFFIC_GIB = {"fwd": 29.62 + 0.50, "recompute": 1.556 + 0.560, "dx": 1.280 + 0.029, "dw": 3.727 + 0.612}
+
 
 def cpu_baseline(inp, rows, threads):
     """The eager reference path (oracle/eager.py) on the host cores, forward + backward,
@@ -43,6 +48,9 @@ def main():
     ap.add_argument("--panel-rows", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=16384)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="after the timed region, copy 1 GiB device to device once (a kernel of known traffic, "
+                         "to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (one process, one MI355X); run with --gpus 1", file=sys.stderr)
@@ -89,6 +97,12 @@ def main():
     _lib.timing_enable(False)
     ms_per_step = ms_total / args.steps
     loss = float(out[0])
+    if args.copy_calibration:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)      # 1 GiB read + 1 GiB written
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     flops_step = 6.0 * N * d * V                      # algorithmic: logits + dX + dW, no recompute
     tokens_per_s = N / (ms_per_step * 1e-3)
@@ -106,7 +120,9 @@ def main():
     dom = max((k for k in kernels if k in algo), key=lambda k: kernels[k]["ms_per_step"])
     roofline = {
         "bound": "mfma", "kernel": dom, "achieved": kernels[dom]["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-        "frac": round(kernels[dom]["tflops"] / PEAK_FP8_TFLOPS, 4), "traffic": None,
+        "frac": round(kernels[dom]["tflops"] / PEAK_FP8_TFLOPS, 4),
+        "traffic": (round(MEASURED_TRAFFIC_GIB[dom] * 2 ** 30) if (args.workload == "limited_2p7b" and args.rows is None
+                                                                   and args.panel_rows == 0) else None),
         "avg_launch_ms": kernels[dom]["avg_launch_ms"],
     }
     result = {
