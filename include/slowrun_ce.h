@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SCE_VERSION 1
+#define SCE_VERSION 2
 
 enum { SCE_F32 = 0, SCE_BF16 = 1 };               /* element types of X, W, dX, dW          */
 enum { SCE_REDUCE_NONE = 0, SCE_REDUCE_MEAN = 1 }; /* F.cross_entropy(reduction=...)         */
@@ -53,6 +53,8 @@ typedef struct sce_shape {
 
 typedef struct sce_sizes {
   size_t saved_bytes;        /* state written by sce_forward and read by sce_backward        */
+  size_t saved_x_bytes;      /* the same when the quantised W lives in a weight cache        */
+  size_t wcache_bytes;       /* size of that weight cache                                    */
   size_t fwd_workspace_bytes;
   size_t bwd_workspace_min_bytes;   /* backward with the smallest row panel (256 rows)       */
   size_t bwd_workspace_bytes;       /* backward with the default row panel                   */
@@ -93,6 +95,15 @@ typedef struct sce_args {
   void* dx;  int32_t dx_dtype;  int32_t pad3;  int64_t dx_ld;      /* (N,d)                  */
   void* dw;  int32_t dw_dtype;  int32_t pad4;  int64_t dw_ld;      /* (d,V)                  */
   int64_t panel_rows;        /* 0 = as many rows per panel as the workspace allows           */
+
+  /* ---- optional ---- */
+  int64_t vocab_limit;       /* columns >= vocab_limit take no part in the softmax (the eager head
+                                slices the padded vocabulary, tiny/train.py:741); 0 = all V       */
+  void* wcache;              /* NULL, or wcache_bytes of device memory holding the quantised W:
+                                forward fills it unless wcache_valid, backward reads it          */
+  size_t wcache_bytes;
+  int32_t wcache_valid;      /* non-zero: wcache already holds e4m3(W / w_s) of this very W      */
+  int32_t pad5;
 } sce_args;
 
 /* Library / ABI version (SCE_VERSION of the build). */

@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(HERE, "libslowrun_ce.so")
 
 SCE_F32, SCE_BF16 = 0, 1
 SCE_REDUCE_NONE, SCE_REDUCE_MEAN = 0, 1
-SCE_VERSION = 1
+SCE_VERSION = 2
 
 EXPORTS = ("sce_version", "sce_last_error", "sce_sizes_for", "sce_quantize_e4m3", "sce_transpose_bytes",
            "sce_forward", "sce_backward", "sce_timing_enable", "sce_timing_read")
@@ -24,7 +24,8 @@ class SceShape(C.Structure):
 
 
 class SceSizes(C.Structure):
-    _fields_ = [("saved_bytes", C.c_size_t), ("fwd_workspace_bytes", C.c_size_t),
+    _fields_ = [("saved_bytes", C.c_size_t), ("saved_x_bytes", C.c_size_t), ("wcache_bytes", C.c_size_t),
+                ("fwd_workspace_bytes", C.c_size_t),
                 ("bwd_workspace_min_bytes", C.c_size_t), ("bwd_workspace_bytes", C.c_size_t),
                 ("bwd_panel_rows", C.c_int64)]
 
@@ -43,6 +44,8 @@ class SceArgs(C.Structure):
         ("dx", C.c_void_p), ("dx_dtype", C.c_int32), ("pad3", C.c_int32), ("dx_ld", C.c_int64),
         ("dw", C.c_void_p), ("dw_dtype", C.c_int32), ("pad4", C.c_int32), ("dw_ld", C.c_int64),
         ("panel_rows", C.c_int64),
+        ("vocab_limit", C.c_int64), ("wcache", C.c_void_p), ("wcache_bytes", C.c_size_t),
+        ("wcache_valid", C.c_int32), ("pad5", C.c_int32),
     ]
 
 

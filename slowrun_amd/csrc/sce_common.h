@@ -27,12 +27,16 @@ constexpr int LONG_SEG = 64;     // target columns hit by at least this many row
 
 static inline int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 
-// Layout of the state sce_forward saves for sce_backward (byte offsets into `saved`).
+// Layout of the state sce_forward saves for sce_backward (byte offsets into `saved`).  The two
+// quantised copies of W come last; with a caller-provided weight cache they live there instead
+// (same relative offsets) and `saved` ends at x_total.
 struct SavedLayout {
   int64_t N, d, V, Np, dp, dq, Vp;   // Np, Vp: multiples of 256; dp: of 128, at least 256; dq: of 256
-  size_t off_hdr, off_xq, off_wqt, off_wq, off_lse, off_umax, off_zy, total;
+  size_t off_hdr, off_xq, off_lse, off_umax, off_zy, x_total;
+  size_t rel_wqt, rel_wq, w_total;   // relative to the start of the W region
+  size_t total;                      // x_total + w_total
 };
-// hdr: int32 n_valid, int32 n_bad_targets, float loss_sum, float pad
+// hdr: int32 n_valid, int32 n_bad_targets, float mean loss, float pad
 
 static inline SavedLayout saved_layout(int64_t N, int64_t d, int64_t V, int n_predict) {
   SavedLayout L;
@@ -42,12 +46,15 @@ static inline SavedLayout saved_layout(int64_t N, int64_t d, int64_t V, int n_pr
   auto take = [&](size_t bytes) { size_t r = o; o += (bytes + 255) / 256 * 256; return r; };
   L.off_hdr = take(256);
   L.off_xq = take((size_t)L.Np * L.dp);        // X_q   [Np][dp]  e4m3, zero padded
-  L.off_wqt = take((size_t)L.Vp * L.dp);       // W_q^T [Vp][dp]
-  L.off_wq = take((size_t)L.dq * L.Vp);        // W_q   [dq][Vp]
   L.off_lse = take((size_t)L.Np * 4);
   L.off_umax = take((size_t)L.Np * 4);
   L.off_zy = take((size_t)L.Np * 4 * n_predict);
-  L.total = o;
+  L.x_total = o;
+  o = 0;
+  L.rel_wqt = take((size_t)L.Vp * L.dp);       // W_q^T [Vp][dp]
+  L.rel_wq = take((size_t)L.dq * L.Vp);        // W_q   [dq][Vp]
+  L.w_total = o;
+  L.total = L.x_total + L.w_total;
   return L;
 }
 

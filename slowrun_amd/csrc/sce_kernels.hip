@@ -665,16 +665,17 @@ __global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
   }
 }
 
-// sort keys: one entry per (offset k, row i): key = target y_{i+k} (V if the pair takes no part),
+// sort keys: one entry per (offset k, row i): key = target y_{i+k} (V if the pair takes no part; targets at or
+// beyond the vocabulary limit Vl take no part),
 // value = entry id k * Np + i
-__global__ __launch_bounds__(256) void bwd_keys_kernel(const int64_t* __restrict__ targets, int64_t ignore_index, int N, int Np, int V,
-                                                      int n_predict, int32_t* __restrict__ keys, int32_t* __restrict__ vals,
+__global__ __launch_bounds__(256) void bwd_keys_kernel(const int64_t* __restrict__ targets, int64_t ignore_index, int N, int Np, int Vl,
+                                                      int V, int n_predict, int32_t* __restrict__ keys, int32_t* __restrict__ vals,
                                                       int32_t* __restrict__ longlist) {
   const int e = blockIdx.x * 256 + threadIdx.x;
   if (e == 0) longlist[0] = 0;        // counter of the long-column list, filled later on the same stream
   if (e >= N * n_predict) return;
   const int k = e / N, i = e - k * N;
-  keys[e] = target_valid(targets, ignore_index, i + k, N, V) ? (int32_t)targets[i + k] : V;
+  keys[e] = target_valid(targets, ignore_index, i + k, N, Vl) ? (int32_t)targets[i + k] : V;
   vals[e] = k * Np + i;
 }
 
@@ -997,6 +998,8 @@ extern "C" int sce_sizes_for(const sce_shape* shape, sce_sizes* out) {
   if (!out) return fail(SCE_EINVAL, "out is NULL");
   const SavedLayout S = saved_layout(shape->N, shape->d, shape->V, shape->n_predict);
   out->saved_bytes = S.total;
+  out->saved_x_bytes = S.x_total;
+  out->wcache_bytes = S.w_total;
   out->fwd_workspace_bytes = (size_t)8 * S.Np * 16 + 256;
   out->bwd_workspace_min_bytes = bwd_layout(S, 256, 256, 1, shape->n_predict).total;
   out->bwd_panel_rows = default_panel(S);
@@ -1053,7 +1056,9 @@ static int check_common(const sce_args* a) {
   if (!(a->x_s > 0.f) || !(a->w_s > 0.f)) return fail(SCE_EINVAL, "x_s and w_s must be positive");
   if (a->reduction != SCE_REDUCE_NONE && a->reduction != SCE_REDUCE_MEAN) return fail(SCE_EINVAL, "bad reduction %d", a->reduction);
   if (!a->saved) return fail(SCE_EINVAL, "saved is NULL");
-  if (((uintptr_t)a->saved & 255) || ((uintptr_t)a->workspace & 255)) return fail(SCE_EINVAL, "saved and workspace must be 256-byte aligned");
+  if (((uintptr_t)a->saved & 255) || ((uintptr_t)a->workspace & 255) || ((uintptr_t)a->wcache & 255))
+    return fail(SCE_EINVAL, "saved, workspace and wcache must be 256-byte aligned");
+  if (a->vocab_limit < 0 || a->vocab_limit > a->shape.V) return fail(SCE_EINVAL, "vocab_limit must be in [0, V]");
   return check_device(a->device);
 }
 
@@ -1067,8 +1072,11 @@ extern "C" int sce_forward(const sce_args* a) {
   if (a->reduction == SCE_REDUCE_MEAN && a->shape.n_predict != 1)
     return fail(SCE_EINVAL, "reduction = mean is defined for a single offset only; use reduction = none with n_predict > 1");
   const SavedLayout S = saved_layout(N, d, V, a->shape.n_predict);
-  if (a->saved_bytes < S.total) return fail(SCE_EINVAL, "saved buffer too small: %zu < %zu", a->saved_bytes, S.total);
-  const int RT = (int)(S.Np / 256), CT = (int)(S.Vp / 256);
+  const size_t need_saved = a->wcache ? S.x_total : S.total;
+  if (a->saved_bytes < need_saved) return fail(SCE_EINVAL, "saved buffer too small: %zu < %zu", a->saved_bytes, need_saved);
+  if (a->wcache && a->wcache_bytes < S.w_total) return fail(SCE_EINVAL, "weight cache too small: %zu < %zu", a->wcache_bytes, S.w_total);
+  const int64_t Vl = a->vocab_limit > 0 ? a->vocab_limit : V;       // columns that take part
+  const int RT = (int)(S.Np / 256), CT = (int)((Vl + 255) / 256);
   const int nsplit = CT < 8 ? CT : 8;
   const size_t need_ws = (size_t)nsplit * S.Np * 16;
   if (!a->workspace || a->workspace_bytes < need_ws) return fail(SCE_EINVAL, "forward workspace too small: %zu < %zu", a->workspace_bytes, need_ws);
@@ -1077,8 +1085,9 @@ extern "C" int sce_forward(const sce_args* a) {
   hipStream_t st = (hipStream_t)a->stream;
   uint8_t* sv = (uint8_t*)a->saved;
   uint8_t* xq = sv + S.off_xq;
-  uint8_t* wqt = sv + S.off_wqt;
-  uint8_t* wq = sv + S.off_wq;
+  uint8_t* wbase = a->wcache ? (uint8_t*)a->wcache : sv + S.x_total;
+  uint8_t* wqt = wbase + S.rel_wqt;
+  uint8_t* wq = wbase + S.rel_wq;
 
   {
     KernelTimer tm(SCE_K_QUANT, st);
@@ -1089,7 +1098,9 @@ extern "C" int sce_forward(const sce_args* a) {
       quantize_pad_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, a->x_s);
     else return fail(SCE_EINVAL, "unsupported x dtype %d", a->x_dtype);
     dim3 gw((unsigned)(S.Vp / 64), (unsigned)(S.dq / 64));
-    if (a->w_dtype == SCE_F32)
+    if (a->wcache && a->wcache_valid) {
+      // the caller vouches that the cache holds e4m3(W / w_s) of this W (unchanged since an earlier call)
+    } else if (a->w_dtype == SCE_F32)
       quantize_w_kernel<float><<<gw, 256, 0, st>>>((const float*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.Vp, a->w_s);
     else if (a->w_dtype == SCE_BF16)
       quantize_w_kernel<bf16_t><<<gw, 256, 0, st>>>((const bf16_t*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.Vp, a->w_s);
@@ -1097,7 +1108,7 @@ extern "C" int sce_forward(const sce_args* a) {
   }
   FwdParams p;
   p.xq = xq; p.wqt = wqt; p.partials = (float4*)a->workspace;
-  p.dp = S.dp; p.N = (int)N; p.V = (int)V; p.Np = (int)S.Np; p.RT = RT; p.CT = CT; p.S = nsplit;
+  p.dp = S.dp; p.N = (int)N; p.V = (int)Vl; p.Np = (int)S.Np; p.RT = RT; p.CT = CT; p.S = nsplit;
   p.sc = a->x_s * a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.c2 = -2.0f * a->cap * LOG2E;
   const int grid = 8 * nsplit * ((RT + 7) / 8);
   {
@@ -1109,11 +1120,11 @@ extern "C" int sce_forward(const sce_args* a) {
   float* s_umax = (float*)(sv + S.off_umax);
   float* s_zy = (float*)(sv + S.off_zy);
   fwd_target_logit_kernel<<<dim3((unsigned)((N + 3) / 4), (unsigned)a->shape.n_predict), 256, 0, st>>>(
-      xq, wqt, S.dp, a->targets, a->ignore_index, (int)N, (int)S.Np, (int)V, a->x_s * a->w_s, a->cap, s_zy);
-  fwd_combine_kernel<<<(int)(S.Np / 256), 256, 0, st>>>(p.partials, nsplit, (int)N, (int)S.Np, (int)V, a->targets, a->ignore_index,
+      xq, wqt, S.dp, a->targets, a->ignore_index, (int)N, (int)S.Np, (int)Vl, a->x_s * a->w_s, a->cap, s_zy);
+  fwd_combine_kernel<<<(int)(S.Np / 256), 256, 0, st>>>(p.partials, nsplit, (int)N, (int)S.Np, (int)Vl, a->targets, a->ignore_index,
                                                        a->cap, a->mtp_weights, a->shape.n_predict, s_lse, s_umax, s_zy, a->losses, a->lse,
                                                        a->argmax);
-  fwd_reduce_kernel<<<1, 1024, 0, st>>>(s_lse, s_zy, a->targets, a->ignore_index, (int)N, (int)V, (int32_t*)(sv + S.off_hdr),
+  fwd_reduce_kernel<<<1, 1024, 0, st>>>(s_lse, s_zy, a->targets, a->ignore_index, (int)N, (int)Vl, (int32_t*)(sv + S.off_hdr),
                                         a->reduction == SCE_REDUCE_MEAN ? a->loss : nullptr, a->n_valid);
   HIP_TRY(hipGetLastError());
   return SCE_OK;
@@ -1128,7 +1139,10 @@ extern "C" int sce_backward(const sce_args* a) {
   if ((a->dx_dtype != SCE_F32 && a->dx_dtype != SCE_BF16) || (a->dw_dtype != SCE_F32 && a->dw_dtype != SCE_BF16))
     return fail(SCE_EINVAL, "unsupported gradient dtype");
   const SavedLayout S = saved_layout(N, d, V, a->shape.n_predict);
-  if (a->saved_bytes < S.total) return fail(SCE_EINVAL, "saved buffer too small: %zu < %zu", a->saved_bytes, S.total);
+  const size_t need_saved = a->wcache ? S.x_total : S.total;
+  if (a->saved_bytes < need_saved) return fail(SCE_EINVAL, "saved buffer too small: %zu < %zu", a->saved_bytes, need_saved);
+  if (a->wcache && a->wcache_bytes < S.w_total) return fail(SCE_EINVAL, "weight cache too small: %zu < %zu", a->wcache_bytes, S.w_total);
+  const int64_t Vl = a->vocab_limit > 0 ? a->vocab_limit : V;       // columns that take part
   if (!a->workspace) return fail(SCE_EINVAL, "workspace is NULL");
   const int K = a->shape.n_predict;
   const BwdLayout Bmin = bwd_layout(S, 256, 256, 1, K);
@@ -1155,8 +1169,9 @@ extern "C" int sce_backward(const sce_args* a) {
   uint8_t* sv = (uint8_t*)a->saved;
   uint8_t* ws = (uint8_t*)a->workspace;
   const uint8_t* xq = sv + S.off_xq;
-  const uint8_t* wqt = sv + S.off_wqt;
-  const uint8_t* wq = sv + S.off_wq;
+  const uint8_t* wbase = a->wcache ? (const uint8_t*)a->wcache : sv + S.x_total;
+  const uint8_t* wqt = wbase + S.rel_wqt;
+  const uint8_t* wq = wbase + S.rel_wq;
   const float* s_lse = (const float*)(sv + S.off_lse);
   const float* s_umax = (const float*)(sv + S.off_umax);
   const float* s_zy = (const float*)(sv + S.off_zy);
@@ -1182,7 +1197,7 @@ extern "C" int sce_backward(const sce_args* a) {
   KernelTimer* tm_prep = new KernelTimer(SCE_K_BWD_PREP, st);
   bwd_prep_kernel<<<nblk, 256, 0, st>>>(s_lse, s_umax, s_zy, a->targets, a->ignore_index, hdr, a->grad_output,
                                         a->reduction == SCE_REDUCE_NONE ? 1 : 0, a->grad_scale, a->mtp_weights, K, a->cap, (int)N,
-                                        (int)S.Np, (int)V, crow, rho, hcoef, blockmax);
+                                        (int)S.Np, (int)Vl, crow, rho, hcoef, blockmax);
   bwd_xi_kernel<<<1, 1024, 0, st>>>(blockmax, nblk, xi);
   {
     dim3 g((unsigned)(S.Np / 64), (unsigned)(S.dq / 64));
@@ -1190,7 +1205,7 @@ extern "C" int sce_backward(const sce_args* a) {
   }
   // rows grouped by target, for the one-hot part of dW
   {
-    bwd_keys_kernel<<<(int)((NE + 255) / 256), 256, 0, st>>>(a->targets, a->ignore_index, (int)N, (int)S.Np, (int)V, K, keys_in, vals_in, longlist);
+    bwd_keys_kernel<<<(int)((NE + 255) / 256), 256, 0, st>>>(a->targets, a->ignore_index, (int)N, (int)S.Np, (int)Vl, (int)V, K, keys_in, vals_in, longlist);
     int bits = 1;
     while ((1ll << bits) <= V) ++bits;
     size_t tmp = B.sorttmp_bytes;
@@ -1209,7 +1224,7 @@ extern "C" int sce_backward(const sce_args* a) {
     const int RTp = (int)(prow / 256);
     RecomputeParams rp;
     rp.xq = xq + p0 * S.dp; rp.wqt = wqt; rp.crow = crow + p0; rp.ghat = ghat; rp.ghat_t = ghat_t + (p0 - w0);
-    rp.dp = S.dp; rp.Vp = S.Vp; rp.Pw = Pw; rp.RT = RTp; rp.CT = CTv; rp.V = (int)V; rp.k1 = k1; rp.c2 = c2;
+    rp.dp = S.dp; rp.Vp = S.Vp; rp.Pw = Pw; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2;
     {
       KernelTimer tm(SCE_K_RECOMPUTE, st);
       bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_RECOMPUTE, st>>>(rp);
@@ -1219,7 +1234,7 @@ extern "C" int sce_backward(const sce_args* a) {
     dp_.wq = wq; dp_.ghat = ghat; dp_.wqt = wqt; dp_.rho = rho + p0; dp_.hcoef = hcoef + p0; dp_.targets = a->targets + p0;
     dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.dp = S.dp; dp_.Np = S.Np; dp_.RT = RTp; dp_.CT = CTd;
     dp_.n_predict = K; dp_.rows_left = (int)(N - p0 > 0 ? N - p0 : 0);
-    dp_.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); dp_.d = (int)d; dp_.V = (int)V; dp_.w_s = a->w_s;
+    dp_.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); dp_.d = (int)d; dp_.V = (int)Vl; dp_.w_s = a->w_s;
     {
       KernelTimer tm(SCE_K_DX, st);
       if (a->dx_dtype == SCE_F32) {

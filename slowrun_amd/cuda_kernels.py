@@ -91,7 +91,31 @@ def _check_inputs(x, w, targets):
         raise ValueError("targets must be int64 of shape (N,)")
 
 
-def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_weights=None):
+class WeightCache:
+    """The two e4m3 copies of the LM-head weight, kept across calls.
+
+    The reference re-quantises and re-lays-out W on every micro-step (tiny/cuda_kernels.py:341-343) although W
+    only changes at optimizer.step().  With a WeightCache the forward quantises W only when the tensor (storage,
+    version counter, scale) differs from the one the cache was filled from.
+    """
+
+    def __init__(self):
+        self.buf = None
+        self.key = None
+
+    def prepare(self, w, w_s, nbytes):
+        """Returns (buffer, valid)."""
+        key = (w.data_ptr(), w._version, tuple(w.shape), w.dtype, float(w_s), w.device)
+        if self.buf is None or self.buf.numel() < nbytes or self.buf.device != w.device:
+            self.buf = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+            self.key = None
+        valid = self.key == key
+        self.key = key
+        return self.buf, valid
+
+
+def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_weights=None, vocab_size=None,
+               weight_cache=None):
     """One call of sce_forward.  Returns (out, saved, lse, argmax, n_valid)."""
     _check_inputs(x, w, targets)
     n_predict, mtp_w = _mtp(mtp_weights, x.device)
@@ -104,7 +128,7 @@ def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_w
     V = w.shape[1]
     dev = x.device
     sz = _lib.sizes_for(N, d, V, n_predict)
-    saved = torch.empty(sz.saved_bytes, dtype=torch.uint8, device=dev)
+    saved = torch.empty(sz.saved_x_bytes if weight_cache is not None else sz.saved_bytes, dtype=torch.uint8, device=dev)
     ws = torch.empty(sz.fwd_workspace_bytes, dtype=torch.uint8, device=dev)
     losses = torch.empty(N, dtype=torch.float32, device=dev)
     lse = torch.empty(N, dtype=torch.float32, device=dev)
@@ -118,13 +142,17 @@ def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_w
     a.argmax = argmax.data_ptr() if want_argmax else None
     a.saved, a.saved_bytes = saved.data_ptr(), saved.numel()
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    a.vocab_limit = 0 if vocab_size is None else int(vocab_size)
+    if weight_cache is not None:
+        wbuf, valid = weight_cache.prepare(w, w_s, sz.wcache_bytes)
+        a.wcache, a.wcache_bytes, a.wcache_valid = wbuf.data_ptr(), wbuf.numel(), int(valid)
     _lib.check(_lib.lib().sce_forward(C.byref(a)), "sce_forward")
     out = loss.reshape(()) if reduction == "mean" else losses
     return out, saved, lse, argmax, n_valid
 
 
 def ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale, reduction, x_dtype, w_dtype,
-                panel_rows=0, workspace_bytes=None, mtp_weights=None):
+                panel_rows=0, workspace_bytes=None, mtp_weights=None, vocab_size=None, weight_cache=None):
     """One call of sce_backward.  Returns (dx (N,d) in x_dtype, dw (d,V) in w_dtype)."""
     dev = saved.device
     n_predict, mtp_w = _mtp(mtp_weights, dev)
@@ -146,6 +174,9 @@ def ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale,
     a.dx, a.dx_dtype, a.dx_ld = dx.data_ptr(), _DTYPES[x_dtype], d
     a.dw, a.dw_dtype, a.dw_ld = dw.data_ptr(), _DTYPES[w_dtype], V
     a.panel_rows = panel_rows
+    a.vocab_limit = 0 if vocab_size is None else int(vocab_size)
+    if weight_cache is not None:
+        a.wcache, a.wcache_bytes, a.wcache_valid = weight_cache.buf.data_ptr(), weight_cache.buf.numel(), 1
     _lib.check(_lib.lib().sce_backward(C.byref(a)), "sce_backward")
     return dx, dw
 
@@ -212,6 +243,18 @@ class FusedSoftcappedCrossEntropy(torch.autograd.Function):
         dx, dw = ce_backward_op(saved, targets, grad_output.contiguous(), mtp_w if has_mtp else None, N, d, V, xs, ws_, cap,
                                 gscale, mean, x_bf16, w_bf16)
         return dx, None, None, dw, None, None, None, None, None, None
+
+
+def softcapped_cross_entropy(x, lm_head_weight, targets, x_s, w_s, cap=15.0, vocab_size=None, reduction="mean"):
+    """Forward-only loss of the eager head (tiny/train.py:741-743) on the fused kernel:
+    ``F.cross_entropy(cap * tanh((x @ W)[..., :vocab_size] / cap), targets, ignore_index=-1, reduction=...)`` with
+    fp8 operands; the N x V logits are never stored.  ``x`` may have leading batch dimensions."""
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, x.shape[-1])
+    out, _saved, _lse, _am, _nv = ce_forward(x2.detach(), lm_head_weight.detach(), targets.reshape(-1),
+                                             _scale_value(x_s, x2), _scale_value(w_s, lm_head_weight), float(cap),
+                                             reduction, vocab_size=vocab_size)
+    return out if reduction == "mean" else out.reshape(lead)
 
 
 def quantize_e4m3(t, scale):

@@ -144,3 +144,62 @@ def test_traced_by_torch_compile():
         loss.backward()
         res.append((loss.detach(), x.grad, w.grad))
     assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1]) and torch.equal(res[0][2], res[1][2])
+
+
+def test_eval_head_with_vocabulary_slice():
+    """tiny/train.py:741-743: logits sliced to the real vocabulary before softcap and cross entropy."""
+    import torch.nn.functional as F
+    from oracle import eager
+    from slowrun_amd.cuda_kernels import softcapped_cross_entropy
+    inp = _small("irregular", 600, 128, 1024)
+    vocab = 1000
+    inp.targets[inp.targets >= vocab] = 3
+    x = inp.x.cuda().bfloat16().reshape(3, 200, 128)
+    w = inp.w.cuda().bfloat16()
+    y = inp.targets.cuda().reshape(3, 200)
+    xq = eager.dequantize(eager.quantize_e4m3(x.reshape(-1, 128), inp.x_s), inp.x_s)
+    wq = eager.dequantize(eager.quantize_e4m3(w, inp.w_s), inp.w_s)
+    logits = (xq @ wq)[..., :vocab].float()
+    logits = inp.cap * torch.tanh(logits / inp.cap)
+    for red in ("mean", "none"):
+        ref = F.cross_entropy(logits, y.reshape(-1), ignore_index=-1, reduction=red)
+        got = softcapped_cross_entropy(x, w, y, inp.x_s, inp.w_s, cap=inp.cap, vocab_size=vocab, reduction=red)
+        assert got.shape == (() if red == "mean" else (3, 200))
+        assert float((got.reshape(-1) - ref.reshape(-1)).abs().max() / ref.abs().max()) < pu.LOSS_RTOL
+
+
+def test_vocabulary_slice_backward_and_weight_cache():
+    from oracle import eager
+    from slowrun_amd import cuda_kernels as ck
+    inp = _small("tiny_track", 520, 128, 1024)
+    vocab = 900
+    inp.targets[inp.targets >= vocab] = 7
+    x = inp.x.cuda().bfloat16()
+    w = inp.w.cuda().bfloat16()
+    y = inp.targets.cuda()
+    # oracle: zero weight columns do not reproduce a slice (they still enter the softmax), so slice W itself
+    ref = eager.softcapped_ce(x, w[:, :vocab].contiguous(), y, inp.x_s, inp.w_s, cap=inp.cap, reduction="mean")
+    cache = ck.WeightCache()
+    go = torch.ones((), device="cuda")
+    for rep in range(2):                      # second pass reuses the cached quantised W
+        loss, saved, _lse, _am, _nv = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, "mean", vocab_size=vocab,
+                                                    weight_cache=cache)
+        dx, dw = ck.ce_backward(saved, y, go, 520, 128, 1024, inp.x_s, inp.w_s, inp.cap, 1.0, "mean", torch.bfloat16,
+                                torch.bfloat16, vocab_size=vocab, weight_cache=cache)
+        assert abs(float(loss) - float(ref["loss"])) / float(ref["loss"]) < pu.LOSS_RTOL
+        assert pu.cosine(dx.float(), ref["dx"]) > pu.GRAD_COS and pu.maxrel(dx.float(), ref["dx"]) < pu.GRAD_MAXREL
+        assert pu.cosine(dw[:, :vocab].float(), ref["dw"]) > pu.GRAD_COS
+        assert float(dw[:, vocab:].float().abs().max()) == 0.0
+        if rep == 0:
+            first = (loss.clone(), dx.clone(), dw.clone())
+    assert torch.equal(first[0], loss) and torch.equal(first[1], dx) and torch.equal(first[2], dw)
+    # a changed weight invalidates the cache
+    w2 = w.clone()
+    w2[:, :10] *= 0.5
+    loss2, *_ = ck.ce_forward(x, w2, y, inp.x_s, inp.w_s, inp.cap, "mean", vocab_size=vocab, weight_cache=cache)
+    loss2_nocache, *_ = ck.ce_forward(x, w2, y, inp.x_s, inp.w_s, inp.cap, "mean", vocab_size=vocab)
+    assert torch.equal(loss2, loss2_nocache) and not torch.equal(loss2, loss)
+    w2.mul_(0.5)                                  # in-place update bumps the version counter
+    loss3, *_ = ck.ce_forward(x, w2, y, inp.x_s, inp.w_s, inp.cap, "mean", vocab_size=vocab, weight_cache=cache)
+    loss3_nocache, *_ = ck.ce_forward(x, w2, y, inp.x_s, inp.w_s, inp.cap, "mean", vocab_size=vocab)
+    assert torch.equal(loss3, loss3_nocache)
