@@ -203,3 +203,52 @@ def test_vocabulary_slice_backward_and_weight_cache():
     loss3, *_ = ck.ce_forward(x, w2, y, inp.x_s, inp.w_s, inp.cap, "mean", vocab_size=vocab, weight_cache=cache)
     loss3_nocache, *_ = ck.ce_forward(x, w2, y, inp.x_s, inp.w_s, inp.cap, "mean", vocab_size=vocab)
     assert torch.equal(loss3, loss3_nocache)
+
+
+def test_minimum_workspace_and_strided_rows():
+    """Smallest allowed backward workspace: 256-row panels, a single fp32 dW buffer that later launches read,
+    add to and rewrite.  Also feeds X and W as row-strided views (row stride > row length)."""
+    from slowrun_amd import _lib
+    from slowrun_amd import cuda_kernels as ck
+    inp = _small("limited_2p7b", 1300, 256, 2100)
+    xbig = torch.zeros(1300, 300, dtype=torch.bfloat16, device="cuda")
+    wbig = torch.zeros(256, 2200, dtype=torch.bfloat16, device="cuda")
+    xbig[:, :256] = inp.x.cuda().bfloat16()
+    wbig[:, :2100] = inp.w.cuda().bfloat16()
+    x, w = xbig[:, :256], wbig[:, :2100]              # stride(0) = 300 / 2200, stride(1) = 1
+    y = inp.targets.cuda()
+    sz = _lib.sizes_for(1300, 256, 2100)
+    loss, saved, lse, _am, _nv = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, "mean")
+    go = torch.ones((), device="cuda")
+    dx_min, dw_min = ck.ce_backward(saved, y, go, 1300, 256, 2100, inp.x_s, inp.w_s, inp.cap, 1.0, "mean", torch.bfloat16,
+                                    torch.float32, workspace_bytes=sz.bwd_workspace_min_bytes)
+    ours = dict(loss=loss, lse=lse, argmax=None, n_valid=_nv, dx=dx_min, dw=dw_min, x=x.contiguous(), w=w.contiguous(), y=y,
+                x_s=inp.x_s, w_s=inp.w_s)
+    ref = pu.run_oracle(inp, ours, "mean")
+    print(pu.check_parity(ours, ref, "mean", check_argmax=False))
+    dx_def, dw_def = ck.ce_backward(saved, y, go, 1300, 256, 2100, inp.x_s, inp.w_s, inp.cap, 1.0, "mean", torch.bfloat16,
+                                    torch.float32)
+    assert torch.equal(dx_def, dx_min)
+    assert pu.maxrel(dw_def, dw_min) < 1e-4          # same terms, different order of the fp32 sums
+    with pytest.raises(RuntimeError, match="workspace too small"):
+        ck.ce_backward(saved, y, go, 1300, 256, 2100, inp.x_s, inp.w_s, inp.cap, 1.0, "mean", torch.bfloat16, torch.float32,
+                       workspace_bytes=sz.bwd_workspace_min_bytes - 4096)
+
+
+def test_fixed_scales_of_the_trainer_and_overflow_to_nan():
+    """The trainer's fixed scales (tiny/train.py:188-189).  A value that overflows e4m3 becomes NaN in torch's
+    cast and poisons that row's loss in the eager path; the fused path must do the same, not saturate."""
+    from oracle import eager
+    inp = _small("tiny_track", 300, 128, 700)
+    x_s, w_s = 100 / 448, 1.6 / 448
+    inp.x_s, inp.w_s = x_s, w_s
+    ours = pu.run_ours(inp, "none")
+    ref = pu.run_oracle(inp, ours, "none")
+    print(pu.check_parity(ours, ref, "none"))
+    inp.x[17, 5] = 150.0                              # 150 / x_s = 672 > 464 -> NaN code
+    ours = pu.run_ours(inp, "none")
+    ref = eager.softcapped_ce(ours["x"], ours["w"], ours["y"], x_s, w_s, cap=inp.cap, reduction="none", want_grads=False)
+    assert torch.isnan(ref["loss"][17]) and torch.isnan(ours["loss"][17])
+    ok = torch.ones(300, dtype=torch.bool, device="cuda")
+    ok[17] = False
+    assert float((ours["loss"][ok] - ref["loss"][ok]).abs().max()) < 1e-3
