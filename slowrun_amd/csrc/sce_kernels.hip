@@ -95,6 +95,34 @@ static inline int map_tile_grid(int RT, int CT) { return 8 * ((RT * CT + 7) / 8)
 // ------------------------------------------------------------------------------------------
 // quantisation
 // ------------------------------------------------------------------------------------------
+// 16 consecutive elements starting at p as floats after the scaled division; elements at or beyond
+// `valid` are 0.  One or two 16/32-byte vector loads when the run is complete and 16-byte aligned.
+template <typename T>
+__device__ __forceinline__ void load16_scaled(const T* __restrict__ p, int64_t valid, float scale, float (&v)[16]) {
+  if (valid >= 16 && (((uintptr_t)p) & 15) == 0) {
+    if constexpr (sizeof(T) == 2) {
+      const v4i r0 = *reinterpret_cast<const v4i*>(p), r1 = *reinterpret_cast<const v4i*>(p + 8);
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        v[2 * m] = Elem<T>::div_round(__uint_as_float((uint32_t)r0[m] << 16), scale);
+        v[2 * m + 1] = Elem<T>::div_round(__uint_as_float((uint32_t)r0[m] & 0xffff0000u), scale);
+        v[8 + 2 * m] = Elem<T>::div_round(__uint_as_float((uint32_t)r1[m] << 16), scale);
+        v[8 + 2 * m + 1] = Elem<T>::div_round(__uint_as_float((uint32_t)r1[m] & 0xffff0000u), scale);
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const v4f r = *reinterpret_cast<const v4f*>(p + 4 * q);
+#pragma unroll
+        for (int m = 0; m < 4; ++m) v[4 * q + m] = Elem<T>::div_round(r[m], scale);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int m = 0; m < 16; ++m) v[m] = (m < valid) ? Elem<T>::div_round(Elem<T>::load(p + m), scale) : 0.f;
+  }
+}
+
 // dst [rows_p][cols_p] e4m3 = src [rows][cols] / scale, zero outside; 16 outputs per thread.
 template <typename T>
 __global__ __launch_bounds__(256) void quantize_pad_kernel(const T* __restrict__ src, int64_t ld, int64_t rows,
@@ -107,9 +135,7 @@ __global__ __launch_bounds__(256) void quantize_pad_kernel(const T* __restrict__
     uint32_t out[4] = {0, 0, 0, 0};
     if (r < rows && c0 < cols) {
       float v[16];
-#pragma unroll
-      for (int m = 0; m < 16; ++m)
-        v[m] = (c0 + m < cols) ? Elem<T>::div_round(Elem<T>::load(src + r * ld + c0 + m), scale) : 0.f;
+      load16_scaled<T>(src + r * ld + c0, cols - c0, scale, v);
 #pragma unroll
       for (int m = 0; m < 4; ++m) out[m] = cvt4_e4m3(v[4 * m], v[4 * m + 1], v[4 * m + 2], v[4 * m + 3]);
     }
@@ -131,9 +157,7 @@ __global__ __launch_bounds__(256) void quantize_w_kernel(const T* __restrict__ w
     uint32_t out[4] = {0, 0, 0, 0};
     if (j < d && v < V) {
       float x[16];
-#pragma unroll
-      for (int m = 0; m < 16; ++m)
-        x[m] = (v + m < V) ? Elem<T>::div_round(Elem<T>::load(w + j * ld + v + m), scale) : 0.f;
+      load16_scaled<T>(w + j * ld + v, V - v, scale, x);
 #pragma unroll
       for (int m = 0; m < 4; ++m) out[m] = cvt4_e4m3(x[4 * m], x[4 * m + 1], x[4 * m + 2], x[4 * m + 3]);
     }
