@@ -286,8 +286,10 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p) {
   v16f acc[4][4];
   const uint8_t* Bg = p.xq + (int64_t)rt * 256 * p.dp;
   const int KT = (int)(p.dp / BK);
+  // of the workgroups that start together on this XCD, those with the same split share the W tiles, those with the same rt the X rows
+  const int rot_a = 2 * ((slot / p.S) & 3), rot_b = s & 7;
   for (int ct = ct0; ct < ct1; ++ct) {
-    mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.dp, p.dp, Bg, p.dp, KT, smem, acc);
+    mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.dp, p.dp, Bg, p.dp, KT, smem, acc, rot_a, rot_b);
     const int vbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
     if (ct * 256 + 256 > p.V) fwd_epilogue<true>(acc, p, vbase, sum, amax, uarg);
     else fwd_epilogue<false>(acc, p, vbase, sum, amax, uarg);
@@ -544,7 +546,7 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
-  mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.dp, p.dp, p.xq + (int64_t)rt * 256 * p.dp, p.dp, (int)(p.dp / BK), smem, acc);
+  mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.dp, p.dp, p.xq + (int64_t)rt * 256 * p.dp, p.dp, (int)(p.dp / BK), smem, acc, 2 * (rt & 3), ct & 7);
   uint8_t* T = smem;                         // [256 rows i][STG_PITCH]: columns v contiguous
   uint8_t* TT = smem + 256 * STG_PITCH;      // [256 columns v][STG_PITCH]: rows i contiguous
   const int vloc0 = wa * 128 + 4 * (lane >> 5);
@@ -615,7 +617,7 @@ __global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p) {
   if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
-  mfma_mainloop(p.wq + (int64_t)ct * 256 * p.Vp, p.Vp, p.ghat + (int64_t)rt * 256 * p.Vp, p.Vp, (int)(p.Vp / BK), smem, acc);
+  mfma_mainloop(p.wq + (int64_t)ct * 256 * p.Vp, p.Vp, p.ghat + (int64_t)rt * 256 * p.Vp, p.Vp, (int)(p.Vp / BK), smem, acc, 2 * (rt & 3), ct & 7);
   const int jbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
   T* dx = reinterpret_cast<T*>(p.dx);
 #pragma unroll
@@ -672,7 +674,7 @@ __global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
   if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
-  mfma_mainloop(p.xt + (int64_t)rt * 256 * p.Np, p.Np, p.ghat_t + (int64_t)ct * 256 * p.Pw, p.Pw, p.KT, smem, acc);
+  mfma_mainloop(p.xt + (int64_t)rt * 256 * p.Np, p.Np, p.ghat_t + (int64_t)ct * 256 * p.Pw, p.Pw, p.KT, smem, acc, ct & 7, 2 * (rt & 3));
   const int jbase = rt * 256 + wa * 128 + 4 * (lane >> 5);
 #pragma unroll
   for (int b = 0; b < 4; ++b) {

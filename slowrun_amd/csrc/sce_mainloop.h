@@ -9,9 +9,15 @@
 // Two 64 KB LDS slots each hold K = 128 bytes of the 512 tile rows.  16-byte chunks are XOR
 // swizzled by row so that fragment reads are free of bank conflicts without padding (a wave-wide
 // direct load fills 1 KB of LDS contiguously, so padding rows is not possible).  Fragments are
-// double-buffered in registers one 64-byte sub-step ahead; there is one barrier per sub-step,
-// placed in its middle, and the instruction order (one MFMA, then its share of LDS reads and
-// global loads) is pinned with sched_barrier.
+// double-buffered in registers one 64-byte sub-step ahead; there is one barrier per K block,
+// placed in the middle of its second sub-step, and the instruction order (one MFMA, then its
+// share of LDS reads and global loads) is pinned with sched_barrier.
+//
+// Workgroups that run side by side on one XCD share tile rows through its L2.  Each of them
+// starts its loads of a K block at a different 8-row chunk (rot_a, rot_b: the workgroup's index
+// among the sharers of its A and B rows), so that together they touch every line of the block
+// at the start of the issue window: whichever line misses L2 is requested as early as possible,
+// and the others find it there (measured +7 to +13 % on operands that come from HBM).
 #pragma once
 #include "sce_common.h"
 
@@ -24,25 +30,27 @@ __device__ __forceinline__ void lds_direct_16(uint32_t lds_addr, uint32_t voff, 
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
 }
 
-// lda, ldb: row strides in bytes, multiples of 16, at most 2^24; KD = K / 128 >= 2.
+// lda, ldb: row strides in bytes, multiples of 16, at most 2^24; KD = K / 128 >= 2;
+// rot_a, rot_b in [0, 8), uniform over the workgroup.
 __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, int64_t lda,
                                               const uint8_t* __restrict__ Bg, int64_t ldb, int KD,
-                                              uint8_t* smem, v16f (&acc)[4][4]) {
+                                              uint8_t* smem, v16f (&acc)[4][4], int rot_a, int rot_b) {
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6), wa = wave >> 1, wb = wave & 1;
   const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
   // global -> LDS: one wave instruction covers 8 rows x 128 B; a wave fills rows [64 w, 64 w + 64) of A and of B
   const int lr = lane >> 3, pc = lane & 7;
-  uint32_t vo[16];   // even: A, odd: B
+  uint32_t vo[16];   // even: A, odd: B; load n of an operand covers the 8-row chunk (n + rot) % 8
 #pragma unroll
   for (int n = 0; n < 8; ++n) {
-    const int row = wave * 64 + n * 8 + lr;
-    const int sw = (row & 7) ^ ((row >> 3) & 1);
-    vo[2 * n] = (uint32_t)(row * lda + ((pc ^ sw) * 16));
-    vo[2 * n + 1] = (uint32_t)(row * ldb + ((pc ^ sw) * 16));
+    const int rowa = wave * 64 + ((n + rot_a) & 7) * 8 + lr, rowb = wave * 64 + ((n + rot_b) & 7) * 8 + lr;
+    const int swa = (rowa & 7) ^ ((rowa >> 3) & 1), swb = (rowb & 7) ^ ((rowb >> 3) & 1);
+    vo[2 * n] = (uint32_t)(rowa * lda + ((pc ^ swa) * 16));
+    vo[2 * n + 1] = (uint32_t)(rowb * ldb + ((pc ^ swb) * 16));
   }
   auto issue1 = [&](int kd, int n) {
-    const uint32_t base = lds0 + (kd & 1) * SLOT_BYTES + (n & 1) * TM * BK + wave * 64 * BK + (n >> 1) * 8 * BK;
+    const int chunk = ((n >> 1) + ((n & 1) ? rot_b : rot_a)) & 7;
+    const uint32_t base = lds0 + (kd & 1) * SLOT_BYTES + (n & 1) * TM * BK + wave * 64 * BK + chunk * 8 * BK;
     const uint8_t* g = ((n & 1) ? Bg : Ag) + (int64_t)kd * BK;
     lds_direct_16(base, vo[n], g);
   };
@@ -90,10 +98,7 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
       if (!odd && j > 0 && ((j + 2) >> 1) < KD) issue1((j + 2) >> 1, 8 + i);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (j + 1 < J) {
-      if (odd) asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-      else asm volatile("s_barrier" ::: "memory");
-    }
+    if (odd && j + 1 < J) asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     const int kd_new = (j + 3) >> 1;
 #pragma unroll
