@@ -31,7 +31,7 @@ static inline int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * 
 // quantised copies of W come last; with a caller-provided weight cache they live there instead
 // (same relative offsets) and `saved` ends at x_total.
 struct SavedLayout {
-  int64_t N, d, V, Np, dp, dq, Vp;   // Np, Vp: multiples of 256; dp: of 128, at least 256; dq: of 256
+  int64_t N, d, V, Np, dp, dq, Vp;   // all padded sizes are multiples of 256 (every K loop runs over an even number of 128-byte blocks); dp = dq
   size_t off_hdr, off_xq, off_lse, off_umax, off_zy, x_total;
   size_t rel_wqt, rel_wq, w_total;   // relative to the start of the W region
   size_t total;                      // x_total + w_total
@@ -41,7 +41,7 @@ struct SavedLayout {
 static inline SavedLayout saved_layout(int64_t N, int64_t d, int64_t V, int n_predict) {
   SavedLayout L;
   L.N = N; L.d = d; L.V = V;
-  L.Np = round_up(N, 256); L.dp = round_up(d, 128) < 256 ? 256 : round_up(d, 128); L.dq = round_up(d, 256); L.Vp = round_up(V, 256);
+  L.Np = round_up(N, 256); L.dp = round_up(d, 256); L.dq = round_up(d, 256); L.Vp = round_up(V, 256);
   size_t o = 0;
   auto take = [&](size_t bytes) { size_t r = o; o += (bytes + 255) / 256 * 256; return r; };
   L.off_hdr = take(256);

@@ -288,8 +288,11 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p) {
   const int KT = (int)(p.dp / BK);
   // of the workgroups that start together on this XCD, those with the same split share the W tiles, those with the same rt the X rows
   const int rot_a = 2 * ((slot / p.S) & 3), rot_b = s & 7;
+  // the first K blocks of the next tile travel while the epilogue of this one runs (it does not touch LDS)
+  if (ct0 < ct1) mfma_prefetch(p.wqt + (int64_t)ct0 * 256 * p.dp, p.dp, Bg, p.dp, smem, rot_a, rot_b);
   for (int ct = ct0; ct < ct1; ++ct) {
-    mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.dp, p.dp, Bg, p.dp, KT, smem, acc, rot_a, rot_b);
+    mfma_mainloop<true>(p.wqt + (int64_t)ct * 256 * p.dp, p.dp, Bg, p.dp, KT, smem, acc, rot_a, rot_b);
+    if (ct + 1 < ct1) mfma_prefetch(p.wqt + (int64_t)(ct + 1) * 256 * p.dp, p.dp, Bg, p.dp, smem, rot_a, rot_b);
     const int vbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
     if (ct * 256 + 256 > p.V) fwd_epilogue<true>(acc, p, vbase, sum, amax, uarg);
     else fwd_epilogue<false>(acc, p, vbase, sum, amax, uarg);

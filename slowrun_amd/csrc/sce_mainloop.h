@@ -25,42 +25,74 @@ namespace sce {
 
 // The compiler must not see these loads: it would serialise every later LDS read behind
 // vmcnt(0).  Completion is tracked by hand with s_waitcnt vmcnt before the barrier that
-// publishes the data.
+// publishes the data.  LDS_CONST is an immediate, so that the only scalar work per load is the one
+// addition that forms M0.  (The instruction's own offset field is of no use for stepping through
+// K: the hardware adds it to the LDS address as well as to the memory address.)
+template <int LDS_CONST>
 __device__ __forceinline__ void lds_direct_16(uint32_t lds_addr, uint32_t voff, const uint8_t* sbase) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+  asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
+               ::"s"(lds_addr), "n"(LDS_CONST), "v"(voff), "s"(sbase) : "memory", "scc");
 }
 
-// lda, ldb: row strides in bytes, multiples of 16, at most 2^24; KD = K / 128 >= 2;
+// Global -> LDS loads of one tile: per wave, 16 instructions per K block (8 for A, 8 for B).
+struct TileLoads {
+  uint32_t vo[16];    // per-lane byte offset of load n; even n: A, odd n: B
+  uint32_t lds[16];   // LDS address of load n in slot 0 (wave-uniform)
+  // load n of an operand covers the 8-row chunk (n / 2 + rot) % 8 of the wave's 64 rows
+  __device__ __forceinline__ TileLoads(int64_t lda, int64_t ldb, uint8_t* smem, int rot_a, int rot_b) {
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
+    // one wave instruction covers 8 rows x 128 B; a wave fills rows [64 w, 64 w + 64) of A and of B
+    const int lr = lane >> 3, pc = lane & 7;
+#pragma unroll
+    for (int n = 0; n < 8; ++n) {
+      const int ca = (n + rot_a) & 7, cb = (n + rot_b) & 7;
+      const int rowa = wave * 64 + ca * 8 + lr, rowb = wave * 64 + cb * 8 + lr;
+      const int swa = (rowa & 7) ^ ((rowa >> 3) & 1), swb = (rowb & 7) ^ ((rowb >> 3) & 1);
+      vo[2 * n] = (uint32_t)(rowa * lda + ((pc ^ swa) * 16));
+      vo[2 * n + 1] = (uint32_t)(rowb * ldb + ((pc ^ swb) * 16));
+      lds[2 * n] = lds0 + wave * 64 * BK + ca * 8 * BK;
+      lds[2 * n + 1] = lds0 + TM * BK + wave * 64 * BK + cb * 8 * BK;
+    }
+  }
+  // load n of the K block that starts at ga / gb, into LDS slot SLOT
+  template <int SLOT>
+  __device__ __forceinline__ void issue(int n, const uint8_t* ga, const uint8_t* gb) const {
+    lds_direct_16<SLOT * SLOT_BYTES>(lds[n], vo[n], (n & 1) ? gb : ga);
+  }
+};
+
+// Puts K block 0 and the first half of the loads of K block 1 of a tile in flight (24 loads per wave).
+// Both LDS slots must be free: every wave is past the closing barrier of the previous main loop.  A
+// main loop that follows with PREFETCHED = true expects exactly these 24 loads to be the wave's newest
+// vector memory operations.
+__device__ __forceinline__ void mfma_prefetch(const uint8_t* __restrict__ Ag, int64_t lda, const uint8_t* __restrict__ Bg,
+                                              int64_t ldb, uint8_t* smem, int rot_a, int rot_b) {
+  const TileLoads ld(lda, ldb, smem, rot_a, rot_b);
+#pragma unroll
+  for (int n = 0; n < 16; ++n) ld.issue<0>(n, Ag, Bg);
+#pragma unroll
+  for (int n = 0; n < 8; ++n) ld.issue<1>(n, Ag + BK, Bg + BK);
+}
+
+// lda, ldb: row strides in bytes, multiples of 16, at most 2^24; KD = K / 128, even, >= 2;
 // rot_a, rot_b in [0, 8), uniform over the workgroup.
+template <bool PREFETCHED = false>
 __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, int64_t lda,
                                               const uint8_t* __restrict__ Bg, int64_t ldb, int KD,
                                               uint8_t* smem, v16f (&acc)[4][4], int rot_a, int rot_b) {
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6), wa = wave >> 1, wb = wave & 1;
-  const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
-  // global -> LDS: one wave instruction covers 8 rows x 128 B; a wave fills rows [64 w, 64 w + 64) of A and of B
-  const int lr = lane >> 3, pc = lane & 7;
-  uint32_t vo[16];   // even: A, odd: B; load n of an operand covers the 8-row chunk (n + rot) % 8
-#pragma unroll
-  for (int n = 0; n < 8; ++n) {
-    const int rowa = wave * 64 + ((n + rot_a) & 7) * 8 + lr, rowb = wave * 64 + ((n + rot_b) & 7) * 8 + lr;
-    const int swa = (rowa & 7) ^ ((rowa >> 3) & 1), swb = (rowb & 7) ^ ((rowb >> 3) & 1);
-    vo[2 * n] = (uint32_t)(rowa * lda + ((pc ^ swa) * 16));
-    vo[2 * n + 1] = (uint32_t)(rowb * ldb + ((pc ^ swb) * 16));
-  }
-  auto issue1 = [&](int kd, int n) {
-    const int chunk = ((n >> 1) + ((n & 1) ? rot_b : rot_a)) & 7;
-    const uint32_t base = lds0 + (kd & 1) * SLOT_BYTES + (n & 1) * TM * BK + wave * 64 * BK + chunk * 8 * BK;
-    const uint8_t* g = ((n & 1) ? Bg : Ag) + (int64_t)kd * BK;
-    lds_direct_16(base, vo[n], g);
-  };
+  const TileLoads ld(lda, ldb, smem, rot_a, rot_b);
   // fragments: lane reads row l%32 of a 32-row block, 32 bytes of K at (l/32)*32 within the sub-step
   const int r = lane & 31, h = lane >> 5;
   const int sw = (r & 7) ^ ((r >> 3) & 1);
   const int abase = wa * 128 * BK + r * BK, bbase = TM * BK + wb * 128 * BK + r * BK;
-  auto rfrag1 = [&](int j, int n, v8i (&fa)[4], v8i (&fb)[4]) {   // sub-step j, fragment n (0-3: A, 4-7: B)
-    const int c0 = ((4 * (j & 1) + 2 * h) ^ sw) * 16;
-    const uint8_t* s = smem + ((j >> 1) & 1) * SLOT_BYTES + ((n < 4) ? abase + n * 32 * BK : bbase + (n - 4) * 32 * BK);
+  // fragment n (0-3: A, 4-7: B) of the sub-step with K half `half` in LDS slot `slot`
+  auto rfrag1 = [&](int slot, int half, int n, v8i (&fa)[4], v8i (&fb)[4]) {
+    const int c0 = ((4 * half + 2 * h) ^ sw) * 16;
+    const uint8_t* s = smem + slot * SLOT_BYTES + ((n < 4) ? abase + n * 32 * BK : bbase + (n - 4) * 32 * BK);
     const v4i lo = *reinterpret_cast<const v4i*>(s + c0);
     const v4i hi = *reinterpret_cast<const v4i*>(s + (c0 ^ 16));
     const v8i f = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
@@ -73,46 +105,97 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
 #pragma unroll
       for (int q = 0; q < 16; ++q) acc[a][b][q] = 0.f;
 
-  // prologue: K blocks 0 and 1 in flight, block 0 visible, fragments of sub-step 0 in registers
+  // prologue: K block 0 and half of block 1 in flight, block 0 visible, fragments of sub-step 0 in registers
+  if (!PREFETCHED) {
 #pragma unroll
-  for (int n = 0; n < 16; ++n) issue1(0, n);
+    for (int n = 0; n < 16; ++n) ld.issue<0>(n, Ag, Bg);
 #pragma unroll
-  for (int n = 0; n < 16; ++n) issue1(1, n);
-  asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");
+    for (int n = 0; n < 8; ++n) ld.issue<1>(n, Ag + BK, Bg + BK);
+  }
+  asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
   v8i fa[2][4], fb[2][4];
 #pragma unroll
-  for (int n = 0; n < 8; ++n) rfrag1(0, n, fa[0], fb[0]);
+  for (int n = 0; n < 8; ++n) rfrag1(0, 0, n, fa[0], fb[0]);
   auto mm = [&](int cur, int i) {
     const int a = i >> 2, b = i & 3;
     acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[cur][a], fb[cur][b], acc[a][b], 0, 0, 0, 0, 0, 0);
   };
-  const int J = 2 * KD;
-  // Sub-step j works from register set `cur`.  After the barrier of an odd sub-step every wave has
-  // its fragments of K block (j-1)/2 in registers, so that slot is refilled with block (j+3)/2:
-  // 8 loads in the second half of this sub-step, 8 in the first half of the next.  The barrier of
-  // the next odd sub-step waits for them (vmcnt(0)) and publishes the block.
-  auto substep = [&](int j, int cur, bool odd) {
+  // One K block = two sub-steps of 16 MFMAs; register set 0 feeds the first, set 1 the second.  The
+  // loop body handles the blocks in pairs (slot 0, then slot 1) so that every LDS address and every
+  // load offset is a constant.  While block k (slot s) is consumed:
+  //   first half of its first sub-step : loads 8..15 of block k+1 (other slot; its loads 0..7 went out before)
+  //   second half                      : fragments of the second sub-step from slot s
+  //   middle of the second sub-step    : every wave has the last fragments of block k in registers and waits
+  //                                      for its own loads of block k+1; the barrier then frees slot s
+  //                                      and publishes block k+1
+  //   second half                      : fragments of block k+1, loads 0..7 of block k+2 into slot s
+  // ga / gb point at the first block of the current pair; MORE tells whether a further pair follows.
+  const uint8_t* ga = Ag;
+  const uint8_t* gb = Bg;
+  auto pair = [&](bool more) {
+    // ---- block 2p (slot 0)
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      mm(cur, i);
-      if (!odd && j > 0 && ((j + 2) >> 1) < KD) issue1((j + 2) >> 1, 8 + i);
+      mm(0, i);
+      ld.issue<1>(8 + i, ga + BK, gb + BK);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (odd && j + 1 < J) asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-    const int kd_new = (j + 3) >> 1;
 #pragma unroll
     for (int i = 8; i < 16; ++i) {
-      mm(cur, i);
-      if (j + 1 < J) rfrag1(j + 1, i - 8, fa[cur ^ 1], fb[cur ^ 1]);
-      if (odd && kd_new < KD) issue1(kd_new, i - 8);
+      mm(0, i);
+      rfrag1(0, 1, i - 8, fa[1], fb[1]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      mm(1, i);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 8; i < 16; ++i) {
+      mm(1, i);
+      rfrag1(1, 0, i - 8, fa[0], fb[0]);
+      if (more) ld.issue<0>(i - 8, ga + 2 * BK, gb + 2 * BK);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // ---- block 2p + 1 (slot 1)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      mm(0, i);
+      if (more) ld.issue<0>(8 + i, ga + 2 * BK, gb + 2 * BK);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int i = 8; i < 16; ++i) {
+      mm(0, i);
+      rfrag1(1, 1, i - 8, fa[1], fb[1]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      mm(1, i);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (more) asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 8; i < 16; ++i) {
+      mm(1, i);
+      if (more) {
+        rfrag1(0, 0, i - 8, fa[0], fb[0]);
+        ld.issue<1>(i - 8, ga + 3 * BK, gb + 3 * BK);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  for (int j = 0; j < J; j += 2) {
-    substep(j, 0, false);
-    substep(j + 1, 1, true);
+  for (int p = 0; p < (KD >> 1) - 1; ++p) {
+    pair(true);
+    ga += 2 * BK;
+    gb += 2 * BK;
   }
+  pair(false);
   // all LDS reads of this tile are complete in every wave before the caller reuses the buffer
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
