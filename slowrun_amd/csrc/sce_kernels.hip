@@ -564,14 +564,22 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
     const float c = p.crow[rt * 256 + iloc];
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
+      // stage by stage over the 16 values of the block: the transcendental unit is pipelined, a chain
+      // of dependent exp2 / rcp / exp2 on one value at a time is not
+      float rr[16], gg[16];
+#pragma unroll
+      for (int m = 0; m < 16; ++m) rr[m] = fast_exp2(acc[a][b][m] * p.k1);
+#pragma unroll
+      for (int m = 0; m < 16; ++m) rr[m] = fast_rcp(rr[m] + 1.0f);
+#pragma unroll
+      for (int m = 0; m < 16; ++m) gg[m] = fast_exp2(fmaf(p.c2, rr[m], c));
+#pragma unroll
+      for (int m = 0; m < 16; ++m) gg[m] *= rr[m] - rr[m] * rr[m];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         float g[4];
 #pragma unroll
-        for (int m = 0; m < 4; ++m) {
-          const float rr = fast_rcp(fast_exp2(acc[a][b][4 * q + m] * p.k1) + 1.0f);
-          g[m] = fast_exp2(fmaf(p.c2, rr, c)) * (rr - rr * rr);
-        }
+        for (int m = 0; m < 4; ++m) g[m] = gg[4 * q + m];
         const int vloc = vloc0 + a * 32 + 8 * q;
         if (edge) {
 #pragma unroll

@@ -78,10 +78,14 @@ __device__ __forceinline__ void mfma_prefetch(const uint8_t* __restrict__ Ag, in
 
 // lda, ldb: row strides in bytes, multiples of 16, at most 2^24; KD = K / 128, even, >= 2;
 // rot_a, rot_b in [0, 8), uniform over the workgroup.
-template <bool PREFETCHED = false>
+struct NoHook { __device__ __forceinline__ void operator()(int) const {} };
+
+// `hook(i)` is called after MFMA i (0..63) of every pair of K blocks: a place for vector ALU work that
+// does not depend on the accumulators (it runs while the matrix pipe is busy).
+template <bool PREFETCHED = false, class Hook = NoHook>
 __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, int64_t lda,
                                               const uint8_t* __restrict__ Bg, int64_t ldb, int KD,
-                                              uint8_t* smem, v16f (&acc)[4][4], int rot_a, int rot_b) {
+                                              uint8_t* smem, v16f (&acc)[4][4], int rot_a, int rot_b, Hook&& hook = NoHook()) {
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6), wa = wave >> 1, wb = wave & 1;
   const TileLoads ld(lda, ldb, smem, rot_a, rot_b);
@@ -137,18 +141,21 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       mm(0, i);
+      hook(0 + (i & 7));
       ld.issue<1>(8 + i, ga + BK, gb + BK);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 8; i < 16; ++i) {
       mm(0, i);
+      hook(8 + (i & 7));
       rfrag1(0, 1, i - 8, fa[1], fb[1]);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       mm(1, i);
+      hook(16 + (i & 7));
       __builtin_amdgcn_sched_barrier(0);
     }
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
@@ -156,6 +163,7 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
 #pragma unroll
     for (int i = 8; i < 16; ++i) {
       mm(1, i);
+      hook(24 + (i & 7));
       rfrag1(1, 0, i - 8, fa[0], fb[0]);
       if (more) ld.issue<0>(i - 8, ga + 2 * BK, gb + 2 * BK);
       __builtin_amdgcn_sched_barrier(0);
@@ -164,18 +172,21 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       mm(0, i);
+      hook(32 + (i & 7));
       if (more) ld.issue<0>(8 + i, ga + 2 * BK, gb + 2 * BK);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 8; i < 16; ++i) {
       mm(0, i);
+      hook(40 + (i & 7));
       rfrag1(1, 1, i - 8, fa[1], fb[1]);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       mm(1, i);
+      hook(48 + (i & 7));
       __builtin_amdgcn_sched_barrier(0);
     }
     if (more) asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
@@ -183,6 +194,7 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
 #pragma unroll
     for (int i = 8; i < 16; ++i) {
       mm(1, i);
+      hook(56 + (i & 7));
       if (more) {
         rfrag1(0, 0, i - 8, fa[0], fb[0]);
         ld.issue<1>(i - 8, ga + 3 * BK, gb + 3 * BK);
