@@ -615,29 +615,22 @@ struct DxParams {
   const float* hcoef;     // [n_predict][Np], offset to the panel
   const int64_t* targets; // offset to the panel
   void* dx;               // offset to the panel's first row
-  int64_t dx_ld, Vp, dp, Np;
+  float* part;            // [ksplit][RT * 256][dq] fp32 partial sums (ksplit > 1 only)
+  int64_t dx_ld, Vp, dp, Np, dq;
   int RT, CT, rows, d, V;  // rows: valid rows in this panel
   int n_predict, rows_left; // rows_left: N - (first row of the panel), bounds the target look-ahead
+  int ksplit;              // the K loop (V) is cut into this many parts, one workgroup each
   float w_s;
 };
 
-template <typename T>
-__global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  int rt, ct;
-  if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
-  v16f acc[4][4];
-  mfma_mainloop(p.wq + (int64_t)ct * 256 * p.Vp, p.Vp, p.ghat + (int64_t)rt * 256 * p.Vp, p.Vp, (int)(p.Vp / BK), smem, acc, 2 * (rt & 3), ct & 7);
-  const int jbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
-  T* dx = reinterpret_cast<T*>(p.dx);
-#pragma unroll
-  for (int b = 0; b < 4; ++b) {
-    const int il = rt * 256 + wb * 128 + b * 32 + (lane & 31);
-    if (il >= p.rows) continue;
-    const float rs = p.rho[il] * p.w_s;
-    float hs[4];
-    const uint8_t* wrow[4];
+// Row scale and one-hot term of four consecutive dX columns j..j+3 of panel row il:
+//   dX = rho_i w_s (G W_q^T) - sum_k h_ik w_s W_q^T[y_{i+k}, :]
+struct DxRowTerms {
+  float rs;
+  float hs[4];
+  const uint8_t* wrow[4];
+  __device__ __forceinline__ DxRowTerms(const DxParams& p, int il) {
+    rs = p.rho[il] * p.w_s;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       hs[k] = 0.f; wrow[k] = p.wqt;
@@ -647,28 +640,84 @@ __global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p) {
         if (hk != 0.f && y >= 0 && y < p.V) { hs[k] = hk; wrow[k] = p.wqt + y * p.dp; }
       }
     }
+  }
+  template <typename T>
+  __device__ __forceinline__ void store4(const DxParams& p, T* dst, int j, float o0, float o1, float o2, float o3) const {
+    o0 *= rs; o1 *= rs; o2 *= rs; o3 *= rs;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (k < p.n_predict) {
+        const uint32_t w = *reinterpret_cast<const uint32_t*>(wrow[k] + j);
+        o0 -= hs[k] * e4m3_to_float<0>(w); o1 -= hs[k] * e4m3_to_float<1>(w);
+        o2 -= hs[k] * e4m3_to_float<2>(w); o3 -= hs[k] * e4m3_to_float<3>(w);
+      }
+    }
+    Elem<T>::store(dst + 0, o0); Elem<T>::store(dst + 1, o1);
+    Elem<T>::store(dst + 2, o2); Elem<T>::store(dst + 3, o3);
+  }
+};
+
+// SPLIT = false: one workgroup per 256 x 256 tile of dX, whole K loop, finished values stored.
+// SPLIT = true : a panel with too few tiles to fill the chip; each tile's K loop is shared by ksplit
+//                workgroups that store raw fp32 partial sums, and bwd_dx_finish_kernel adds them up.
+template <typename T, bool SPLIT>
+__global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  int rt, ct, ks = 0;
+  if (!map_tile(blockIdx.x, p.RT, SPLIT ? p.CT * p.ksplit : p.CT, rt, ct)) return;
+  int64_t k0 = 0;
+  int KD = (int)(p.Vp / BK);
+  if (SPLIT) {
+    ks = ct % p.ksplit; ct /= p.ksplit;
+    const int pairs = KD >> 1;
+    const int q0 = (int)((int64_t)pairs * ks / p.ksplit), q1 = (int)((int64_t)pairs * (ks + 1) / p.ksplit);
+    k0 = (int64_t)q0 * 2 * BK; KD = 2 * (q1 - q0);
+  }
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
+  v16f acc[4][4];
+  mfma_mainloop(p.wq + (int64_t)ct * 256 * p.Vp + k0, p.Vp, p.ghat + (int64_t)rt * 256 * p.Vp + k0, p.Vp, KD, smem, acc, 2 * (rt & 3), ct & 7);
+  const int jbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
+  T* dx = reinterpret_cast<T*>(p.dx);
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int il = rt * 256 + wb * 128 + b * 32 + (lane & 31);
+    if (SPLIT) {
+      float* dst = p.part + ((int64_t)ks * p.RT * 256 + il) * p.dq;
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          *reinterpret_cast<v4f*>(dst + jbase + a * 32 + 8 * q) =
+              (v4f){acc[a][b][4 * q + 0], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2], acc[a][b][4 * q + 3]};
+      continue;
+    }
+    if (il >= p.rows) continue;
+    const DxRowTerms row(p, il);
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int j = jbase + a * 32 + 8 * q;
         if (j >= p.d) continue;                       // d is a multiple of 4, so j..j+3 are in range together
-        float o0 = acc[a][b][4 * q + 0] * rs, o1 = acc[a][b][4 * q + 1] * rs;
-        float o2 = acc[a][b][4 * q + 2] * rs, o3 = acc[a][b][4 * q + 3] * rs;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          if (k < p.n_predict) {
-            const uint32_t w = *reinterpret_cast<const uint32_t*>(wrow[k] + j);
-            o0 -= hs[k] * e4m3_to_float<0>(w); o1 -= hs[k] * e4m3_to_float<1>(w);
-            o2 -= hs[k] * e4m3_to_float<2>(w); o3 -= hs[k] * e4m3_to_float<3>(w);
-          }
-        }
-        T* dst = dx + (int64_t)il * p.dx_ld + j;
-        Elem<T>::store(dst + 0, o0); Elem<T>::store(dst + 1, o1);
-        Elem<T>::store(dst + 2, o2); Elem<T>::store(dst + 3, o3);
+        row.store4<T>(p, dx + (int64_t)il * p.dx_ld + j, j, acc[a][b][4 * q + 0], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2],
+                      acc[a][b][4 * q + 3]);
       }
     }
   }
+}
+
+// sum of the K-split partials, row scale, one-hot term, cast: a thread per (row, four columns)
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_dx_finish_kernel(DxParams p) {
+  const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int per_row = p.d / 4;
+  const int il = (int)(q / per_row), j = (int)(q - (int64_t)il * per_row) * 4;
+  if (il >= p.rows) return;
+  v4f sum = (v4f){0.f, 0.f, 0.f, 0.f};
+  for (int ks = 0; ks < p.ksplit; ++ks)      // fixed order
+    sum += *reinterpret_cast<const v4f*>(p.part + ((int64_t)ks * p.RT * 256 + il) * p.dq + j);
+  const DxRowTerms row(p, il);
+  row.store4<T>(p, reinterpret_cast<T*>(p.dx) + (int64_t)il * p.dx_ld + j, j, sum[0], sum[1], sum[2], sum[3]);
 }
 
 struct DwParams {
@@ -917,8 +966,10 @@ static int check_device(int dev) {
       // the MFMA kernels hold two 64 KB K-slots in LDS
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_recompute_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_RECOMPUTE));
-      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
-      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
     }
   }
@@ -945,6 +996,9 @@ static size_t sort_tmp_bytes(int64_t N, int64_t V) {
   return bytes;
 }
 
+// fp32 partial sums of a K-split dX panel: at most 256 tiles of 256 x 256
+constexpr size_t DX_PART_BYTES = (size_t)256 * 256 * 256 * 4;
+
 static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int nparts, int K) {
   BwdLayout B;
   B.P = P; B.Pw = Pw; B.nparts = nparts;
@@ -962,6 +1016,7 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int npa
   B.off_longlist = take((size_t)(S.N * K / LONG_SEG + 2) * 4);
   B.sorttmp_bytes = sort_tmp_bytes(S.N * K, S.V);
   B.off_sorttmp = take(B.sorttmp_bytes);
+  B.off_dxpart = take(DX_PART_BYTES);
   B.fixed = o;
   B.off_ghat = take((size_t)P * S.Vp);
   B.off_ghat_t = take((size_t)S.Vp * Pw);
@@ -1269,17 +1324,32 @@ extern "C" int sce_backward(const sce_args* a) {
 
     DxParams dp_;
     dp_.wq = wq; dp_.ghat = ghat; dp_.wqt = wqt; dp_.rho = rho + p0; dp_.hcoef = hcoef + p0; dp_.targets = a->targets + p0;
-    dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.dp = S.dp; dp_.Np = S.Np; dp_.RT = RTp; dp_.CT = CTd;
+    dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.dp = S.dp; dp_.Np = S.Np; dp_.dq = S.dq; dp_.RT = RTp; dp_.CT = CTd;
     dp_.n_predict = K; dp_.rows_left = (int)(N - p0 > 0 ? N - p0 : 0);
     dp_.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); dp_.d = (int)d; dp_.V = (int)Vl; dp_.w_s = a->w_s;
+    dp_.part = (float*)(ws + B.off_dxpart);
+    // a panel with fewer than half as many tiles as there are CUs shares each tile's K loop among several workgroups
+    const int tiles = RTp * CTd, kpairs = (int)(S.Vp / BK / 2);
+    int ksplit = tiles * 2 <= 256 ? 256 / tiles : 1;
+    if (ksplit > 8) ksplit = 8;
+    if (ksplit > kpairs) ksplit = kpairs;
+    dp_.ksplit = ksplit;
     {
       KernelTimer tm(SCE_K_DX, st);
-      if (a->dx_dtype == SCE_F32) {
-        dp_.dx = (float*)a->dx + p0 * a->dx_ld;
-        bwd_dx_kernel<float><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_BYTES, st>>>(dp_);
-      } else {
-        dp_.dx = (bf16_t*)a->dx + p0 * a->dx_ld;
-        bwd_dx_kernel<bf16_t><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_BYTES, st>>>(dp_);
+      const bool f32 = a->dx_dtype == SCE_F32;
+      dp_.dx = f32 ? (void*)((float*)a->dx + p0 * a->dx_ld) : (void*)((bf16_t*)a->dx + p0 * a->dx_ld);
+      if (ksplit == 1) {
+        if (f32) bwd_dx_kernel<float, false><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_BYTES, st>>>(dp_);
+        else bwd_dx_kernel<bf16_t, false><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_BYTES, st>>>(dp_);
+      } else if (dp_.rows > 0) {
+        const int fgrid = (int)(((int64_t)dp_.rows * (d / 4) + 255) / 256);
+        if (f32) {
+          bwd_dx_kernel<float, true><<<map_tile_grid(RTp, CTd * ksplit), NTHREADS, SMEM_BYTES, st>>>(dp_);
+          bwd_dx_finish_kernel<float><<<fgrid, 256, 0, st>>>(dp_);
+        } else {
+          bwd_dx_kernel<bf16_t, true><<<map_tile_grid(RTp, CTd * ksplit), NTHREADS, SMEM_BYTES, st>>>(dp_);
+          bwd_dx_finish_kernel<bf16_t><<<fgrid, 256, 0, st>>>(dp_);
+        }
       }
     }
 
