@@ -24,6 +24,7 @@
 #include <stdio.h>
 #include <string.h>
 #include <mutex>
+#include <type_traits>
 #include <vector>
 
 namespace sce {
@@ -558,44 +559,45 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   const int k = lane & 3;
   const uint32_t sel1 = (k & 1) ? 0x03070105u : 0x06020400u;
   const uint32_t sel2 = (k & 2) ? 0x03020706u : 0x05040100u;
+  auto form_g = [&](auto edge_tag) {
+    constexpr bool EDGE = decltype(edge_tag)::value;
 #pragma unroll
-  for (int b = 0; b < 4; ++b) {
-    const int iloc = wb * 128 + b * 32 + (lane & 31);        // row within the tile
-    const float c = p.crow[rt * 256 + iloc];
+    for (int b = 0; b < 4; ++b) {
+      const int iloc = wb * 128 + b * 32 + (lane & 31);        // row within the tile
+      const float c = p.crow[rt * 256 + iloc];
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      // stage by stage over the 16 values of the block: the transcendental unit is pipelined, a chain
-      // of dependent exp2 / rcp / exp2 on one value at a time is not
-      float rr[16], gg[16];
+      for (int a = 0; a < 4; ++a) {
+        // stage by stage over the 16 values of the block: the transcendental unit is pipelined, a chain
+        // of dependent exp2 / rcp / exp2 on one value at a time is not
+        float rr[16], gg[16];
 #pragma unroll
-      for (int m = 0; m < 16; ++m) rr[m] = fast_exp2(acc[a][b][m] * p.k1);
+        for (int m = 0; m < 16; ++m) rr[m] = fast_exp2(acc[a][b][m] * p.k1);
 #pragma unroll
-      for (int m = 0; m < 16; ++m) rr[m] = fast_rcp(rr[m] + 1.0f);
+        for (int m = 0; m < 16; ++m) rr[m] = fast_rcp(rr[m] + 1.0f);
 #pragma unroll
-      for (int m = 0; m < 16; ++m) gg[m] = fast_exp2(fmaf(p.c2, rr[m], c));
+        for (int m = 0; m < 16; ++m) gg[m] = fast_exp2(fmaf(p.c2, rr[m], c));
 #pragma unroll
-      for (int m = 0; m < 16; ++m) gg[m] *= rr[m] - rr[m] * rr[m];
+        for (int m = 0; m < 16; ++m) gg[m] *= rr[m] - rr[m] * rr[m];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        float g[4];
+        for (int q = 0; q < 4; ++q) {
+          const int vloc = vloc0 + a * 32 + 8 * q;
+          if (EDGE) {
 #pragma unroll
-        for (int m = 0; m < 4; ++m) g[m] = gg[4 * q + m];
-        const int vloc = vloc0 + a * 32 + 8 * q;
-        if (edge) {
-#pragma unroll
-          for (int m = 0; m < 4; ++m) if (vloc + m >= vlim) g[m] = 0.f;
+            for (int m = 0; m < 4; ++m) gg[4 * q + m] = (vloc + m >= vlim) ? 0.f : gg[4 * q + m];
+          }
+          const uint32_t w = cvt4_e4m3(gg[4 * q], gg[4 * q + 1], gg[4 * q + 2], gg[4 * q + 3]);
+          *reinterpret_cast<uint32_t*>(T + iloc * STG_PITCH + vloc) = w;
+          // 4 x 4 byte transpose inside the quad: lane k ends up with column vloc + k, rows (iloc & ~3) .. +3
+          const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xB1, 0xF, 0xF, false);    // lane ^ 1
+          const uint32_t x = __builtin_amdgcn_perm(p1, w, sel1);
+          const uint32_t p2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, false);    // lane ^ 2
+          const uint32_t yv = __builtin_amdgcn_perm(p2, x, sel2);
+          *reinterpret_cast<uint32_t*>(TT + (vloc + k) * STG_PITCH + (iloc & ~3)) = yv;
         }
-        const uint32_t w = cvt4_e4m3(g[0], g[1], g[2], g[3]);
-        *reinterpret_cast<uint32_t*>(T + iloc * STG_PITCH + vloc) = w;
-        // 4 x 4 byte transpose inside the quad: lane k ends up with column vloc + k, rows (iloc & ~3) .. +3
-        const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xB1, 0xF, 0xF, false);    // lane ^ 1
-        const uint32_t x = __builtin_amdgcn_perm(p1, w, sel1);
-        const uint32_t p2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, false);    // lane ^ 2
-        const uint32_t yv = __builtin_amdgcn_perm(p2, x, sel2);
-        *reinterpret_cast<uint32_t*>(TT + (vloc + k) * STG_PITCH + (iloc & ~3)) = yv;
       }
     }
-  }
+  };
+  if (edge) form_g(std::true_type{}); else form_g(std::false_type{});
   __syncthreads();
   uint8_t* grow = p.ghat + (int64_t)rt * 256 * p.Vp + (int64_t)ct * 256;
   uint8_t* gcol = p.ghat_t + (int64_t)ct * 256 * p.Pw + (int64_t)rt * 256;
