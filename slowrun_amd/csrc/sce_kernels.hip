@@ -128,7 +128,7 @@ __device__ __forceinline__ void load16_scaled(const T* __restrict__ p, int64_t v
 template <typename T>
 __global__ __launch_bounds__(256) void quantize_pad_kernel(const T* __restrict__ src, int64_t ld, int64_t rows,
                                                           int64_t cols, uint8_t* __restrict__ dst,
-                                                          int64_t rows_p, int64_t cols_p, float scale) {
+                                                          int64_t rows_p, int64_t cols_p, int64_t dst_ld, float scale) {
   const int64_t chunks_per_row = cols_p / 16;
   const int64_t total = rows_p * chunks_per_row;
   for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < total; q += (int64_t)gridDim.x * blockDim.x) {
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(256) void quantize_pad_kernel(const T* __restrict__
 #pragma unroll
       for (int m = 0; m < 4; ++m) out[m] = cvt4_e4m3(v[4 * m], v[4 * m + 1], v[4 * m + 2], v[4 * m + 3]);
     }
-    *reinterpret_cast<v4i*>(dst + r * cols_p + c0) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
+    *reinterpret_cast<v4i*>(dst + r * dst_ld + c0) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
   }
 }
 
@@ -148,7 +148,7 @@ __global__ __launch_bounds__(256) void quantize_pad_kernel(const T* __restrict__
 template <typename T>
 __global__ __launch_bounds__(256) void quantize_w_kernel(const T* __restrict__ w, int64_t ld, int64_t d, int64_t V,
                                                         uint8_t* __restrict__ wq, uint8_t* __restrict__ wqt,
-                                                        int64_t dp, int64_t Vp, float scale) {
+                                                        int64_t dp, int64_t ldx, int64_t ldv, float scale) {
   __shared__ uint8_t tile[64][68];
   const int t = threadIdx.x;
   const int64_t j0 = (int64_t)blockIdx.y * 64, v0 = (int64_t)blockIdx.x * 64;
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(256) void quantize_w_kernel(const T* __restrict__ w
 #pragma unroll
       for (int m = 0; m < 4; ++m) out[m] = cvt4_e4m3(x[4 * m], x[4 * m + 1], x[4 * m + 2], x[4 * m + 3]);
     }
-    *reinterpret_cast<v4i*>(wq + j * Vp + v) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
+    *reinterpret_cast<v4i*>(wq + j * ldv + v) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
 #pragma unroll
     for (int m = 0; m < 4; ++m) *reinterpret_cast<uint32_t*>(&tile[r][c + 4 * m]) = out[m];
   }
@@ -175,7 +175,7 @@ __global__ __launch_bounds__(256) void quantize_w_kernel(const T* __restrict__ w
       out[m] = (uint32_t)tile[jc + 4 * m][vr] | ((uint32_t)tile[jc + 4 * m + 1][vr] << 8) |
                ((uint32_t)tile[jc + 4 * m + 2][vr] << 16) | ((uint32_t)tile[jc + 4 * m + 3][vr] << 24);
     }
-    *reinterpret_cast<v4i*>(wqt + (v0 + vr) * dp + j0 + jc) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
+    *reinterpret_cast<v4i*>(wqt + (v0 + vr) * ldx + j0 + jc) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
   }
 }
 
@@ -220,7 +220,7 @@ struct FwdParams {
   const uint8_t* xq;       // [Np][dp]
   const uint8_t* wqt;      // [Vp][dp]
   float4* partials;        // [S][Np]: sum exp(z - cap), max u, argmax u (bits), unused
-  int64_t dp;
+  int64_t dp, ldx;         // K extent and row stride of xq / wqt
   int N, V, Np, RT, CT, S;
   float sc;                // x_s * w_s
   float k1;                // x_s * w_s * 2 log2(e) / cap : exp2(acc * k1) = e^{2u/cap}
@@ -285,15 +285,15 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p) {
 #pragma unroll
   for (int b = 0; b < 4; ++b) { sum[b] = 0.f; amax[b] = -INFINITY; uarg[b] = 0x7fffffff; }
   v16f acc[4][4];
-  const uint8_t* Bg = p.xq + (int64_t)rt * 256 * p.dp;
+  const uint8_t* Bg = p.xq + (int64_t)rt * 256 * p.ldx;
   const int KT = (int)(p.dp / BK);
   // of the workgroups that start together on this XCD, those with the same split share the W tiles, those with the same rt the X rows
   const int rot_a = 2 * ((slot / p.S) & 3), rot_b = s & 7;
   // the first K blocks of the next tile travel while the epilogue of this one runs (it does not touch LDS)
-  if (ct0 < ct1) mfma_prefetch(p.wqt + (int64_t)ct0 * 256 * p.dp, p.dp, Bg, p.dp, smem, rot_a, rot_b);
+  if (ct0 < ct1) mfma_prefetch(p.wqt + (int64_t)ct0 * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b);
   for (int ct = ct0; ct < ct1; ++ct) {
-    mfma_mainloop<true>(p.wqt + (int64_t)ct * 256 * p.dp, p.dp, Bg, p.dp, KT, smem, acc, rot_a, rot_b);
-    if (ct + 1 < ct1) mfma_prefetch(p.wqt + (int64_t)(ct + 1) * 256 * p.dp, p.dp, Bg, p.dp, smem, rot_a, rot_b);
+    mfma_mainloop<true>(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, Bg, p.ldx, KT, smem, acc, rot_a, rot_b);
+    if (ct + 1 < ct1) mfma_prefetch(p.wqt + (int64_t)(ct + 1) * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b);
     const int vbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
     if (ct * 256 + 256 > p.V) fwd_epilogue<true>(acc, p, vbase, sum, amax, uarg);
     else fwd_epilogue<false>(acc, p, vbase, sum, amax, uarg);
@@ -330,7 +330,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p) {
 // W_q^T[y_{i+k}, :] (both contiguous) and applies the softcap.  Offsets index the flattened target
 // vector, as in the reference kernel (tiny/cuda_kernels.py:229).  Pairs that take no part get 0.
 __global__ __launch_bounds__(256) void fwd_target_logit_kernel(const uint8_t* __restrict__ xq, const uint8_t* __restrict__ wqt,
-                                                              int64_t dp, const int64_t* __restrict__ targets,
+                                                              int64_t dp, int64_t ldx, const int64_t* __restrict__ targets,
                                                               int64_t ignore_index, int N, int Np, int V, float sc, float cap,
                                                               float* __restrict__ s_zy) {
   const int lane = threadIdx.x & 63;
@@ -341,8 +341,8 @@ __global__ __launch_bounds__(256) void fwd_target_logit_kernel(const uint8_t* __
   const bool valid = (y != ignore_index) && y >= 0 && y < V;
   float acc = 0.f;
   if (valid) {
-    const uint8_t* xr = xq + (int64_t)i * dp;
-    const uint8_t* wr = wqt + y * dp;
+    const uint8_t* xr = xq + (int64_t)i * ldx;
+    const uint8_t* wr = wqt + y * ldx;
     for (int64_t c = lane * 16; c < dp; c += 64 * 16) {
       const v4i xa = *reinterpret_cast<const v4i*>(xr + c);
       const v4i wa = *reinterpret_cast<const v4i*>(wr + c);
@@ -493,7 +493,7 @@ __global__ __launch_bounds__(1024) void bwd_xi_kernel(const float* __restrict__ 
 }
 
 // Xt [dq][Np] = e4m3( X_q[i][j] * rho_i / xi ), transposed through LDS in 64 x 64 tiles.
-__global__ __launch_bounds__(256) void bwd_xt_kernel(const uint8_t* __restrict__ xq, int64_t dp, int64_t Np,
+__global__ __launch_bounds__(256) void bwd_xt_kernel(const uint8_t* __restrict__ xq, int64_t dp, int64_t ldx, int64_t ldn,
                                                     const float* __restrict__ rho, const float* __restrict__ xi,
                                                     uint8_t* __restrict__ xt) {
   __shared__ uint8_t tile[64][68];
@@ -501,7 +501,7 @@ __global__ __launch_bounds__(256) void bwd_xt_kernel(const uint8_t* __restrict__
   const int64_t i0 = (int64_t)blockIdx.x * 64, j0 = (int64_t)blockIdx.y * 64;
   if (j0 < dp) {
     const int r = t >> 2, c = (t & 3) * 16;
-    const v4i raw = *reinterpret_cast<const v4i*>(xq + (i0 + r) * dp + j0 + c);
+    const v4i raw = *reinterpret_cast<const v4i*>(xq + (i0 + r) * ldx + j0 + c);
     const float f = rho[i0 + r] / xi[0];
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
@@ -521,7 +521,7 @@ __global__ __launch_bounds__(256) void bwd_xt_kernel(const uint8_t* __restrict__
     out[m] = (uint32_t)tile[ic + 4 * m][jr] | ((uint32_t)tile[ic + 4 * m + 1][jr] << 8) |
              ((uint32_t)tile[ic + 4 * m + 2][jr] << 16) | ((uint32_t)tile[ic + 4 * m + 3][jr] << 24);
   }
-  *reinterpret_cast<v4i*>(xt + (j0 + jr) * Np + i0 + ic) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
+  *reinterpret_cast<v4i*>(xt + (j0 + jr) * ldn + i0 + ic) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
 }
 
 struct RecomputeParams {
@@ -530,7 +530,7 @@ struct RecomputeParams {
   const float* crow;     // offset to the panel's first row
   uint8_t* ghat;         // [P][Vp]
   uint8_t* ghat_t;       // [Vp][Pw], already offset to this panel's first column
-  int64_t dp, Vp, Pw;
+  int64_t dp, ldx, ldv, ldw;   // K extent; row strides of xq / wqt, of ghat and of ghat_t
   int RT, CT, V;
   float k1, c2;          // as in FwdParams
 };
@@ -550,7 +550,7 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
-  mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.dp, p.dp, p.xq + (int64_t)rt * 256 * p.dp, p.dp, (int)(p.dp / BK), smem, acc, 2 * (rt & 3), ct & 7);
+  mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 2 * (rt & 3), ct & 7);
   uint8_t* T = smem;                         // [256 rows i][STG_PITCH]: columns v contiguous
   uint8_t* TT = smem + 256 * STG_PITCH;      // [256 columns v][STG_PITCH]: rows i contiguous
   const int vloc0 = wa * 128 + 4 * (lane >> 5);
@@ -599,13 +599,13 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   };
   if (edge) form_g(std::true_type{}); else form_g(std::false_type{});
   __syncthreads();
-  uint8_t* grow = p.ghat + (int64_t)rt * 256 * p.Vp + (int64_t)ct * 256;
-  uint8_t* gcol = p.ghat_t + (int64_t)ct * 256 * p.Pw + (int64_t)rt * 256;
+  uint8_t* grow = p.ghat + (int64_t)rt * 256 * p.ldv + (int64_t)ct * 256;
+  uint8_t* gcol = p.ghat_t + (int64_t)ct * 256 * p.ldw + (int64_t)rt * 256;
 #pragma unroll
   for (int n = 0; n < 16; ++n) {
     const int cidx = t + 256 * n, row = cidx >> 4, col = (cidx & 15) * 16;
-    *reinterpret_cast<v4i*>(grow + (int64_t)row * p.Vp + col) = *reinterpret_cast<const v4i*>(T + row * STG_PITCH + col);
-    *reinterpret_cast<v4i*>(gcol + (int64_t)row * p.Pw + col) = *reinterpret_cast<const v4i*>(TT + row * STG_PITCH + col);
+    *reinterpret_cast<v4i*>(grow + (int64_t)row * p.ldv + col) = *reinterpret_cast<const v4i*>(T + row * STG_PITCH + col);
+    *reinterpret_cast<v4i*>(gcol + (int64_t)row * p.ldw + col) = *reinterpret_cast<const v4i*>(TT + row * STG_PITCH + col);
   }
 }
 
@@ -618,7 +618,7 @@ struct DxParams {
   const int64_t* targets; // offset to the panel
   void* dx;               // offset to the panel's first row
   float* part;            // [ksplit][RT * 256][dq] fp32 partial sums (ksplit > 1 only)
-  int64_t dx_ld, Vp, dp, Np, dq;
+  int64_t dx_ld, Vp, ldv, ldx, Np, dq;   // Vp: K extent; ldv: row stride of wq / ghat; ldx: of wqt
   int RT, CT, rows, d, V;  // rows: valid rows in this panel
   int n_predict, rows_left; // rows_left: N - (first row of the panel), bounds the target look-ahead
   int ksplit;              // the K loop (V) is cut into this many parts, one workgroup each
@@ -639,7 +639,7 @@ struct DxRowTerms {
       if (k < p.n_predict && il + k < p.rows_left) {
         const float hk = p.hcoef[(int64_t)k * p.Np + il] * p.w_s;
         const int64_t y = p.targets[il + k];
-        if (hk != 0.f && y >= 0 && y < p.V) { hs[k] = hk; wrow[k] = p.wqt + y * p.dp; }
+        if (hk != 0.f && y >= 0 && y < p.V) { hs[k] = hk; wrow[k] = p.wqt + y * p.ldx; }
       }
     }
   }
@@ -677,7 +677,7 @@ __global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p) {
   }
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
-  mfma_mainloop(p.wq + (int64_t)ct * 256 * p.Vp + k0, p.Vp, p.ghat + (int64_t)rt * 256 * p.Vp + k0, p.Vp, KD, smem, acc, 2 * (rt & 3), ct & 7);
+  mfma_mainloop(p.wq + (int64_t)ct * 256 * p.ldv + k0, p.ldv, p.ghat + (int64_t)rt * 256 * p.ldv + k0, p.ldv, KD, smem, acc, 2 * (rt & 3), ct & 7);
   const int jbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
   T* dx = reinterpret_cast<T*>(p.dx);
 #pragma unroll
@@ -726,7 +726,7 @@ struct DwParams {
   const uint8_t* xt;      // [dq][Np], offset to the first row of the dW panel   A side (rows j)
   const uint8_t* ghat_t;  // [Vp][Pw]                                             B side (rows v)
   float* dwacc;           // [dq][Vp] fp32
-  int64_t Np, Pw, Vp;
+  int64_t ldn, ldw, Vp;   // row strides of xt and of ghat_t; row length of dwacc
   int RT, CT, KT, accumulate;
 };
 
@@ -736,7 +736,7 @@ __global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
   if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
-  mfma_mainloop(p.xt + (int64_t)rt * 256 * p.Np, p.Np, p.ghat_t + (int64_t)ct * 256 * p.Pw, p.Pw, p.KT, smem, acc, ct & 7, 2 * (rt & 3));
+  mfma_mainloop(p.xt + (int64_t)rt * 256 * p.ldn, p.ldn, p.ghat_t + (int64_t)ct * 256 * p.ldw, p.ldw, p.KT, smem, acc, ct & 7, 2 * (rt & 3));
   const int jbase = rt * 256 + wa * 128 + 4 * (lane >> 5);
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
@@ -792,7 +792,7 @@ __global__ __launch_bounds__(256) void bwd_longlist_kernel(const int32_t* __rest
 // does not depend on scheduling.
 __global__ __launch_bounds__(256) void bwd_dw_long_kernel(const int32_t* __restrict__ longlist, const int32_t* __restrict__ segoff,
                                                          const int32_t* __restrict__ perm, const float* __restrict__ hcoef,
-                                                         const uint8_t* __restrict__ xq, int64_t dp, int64_t Vp, int Np,
+                                                         const uint8_t* __restrict__ xq, int64_t dp, int64_t ldx, int64_t Vp, int Np,
                                                          const float* __restrict__ xi, float* __restrict__ dwacc) {
   __shared__ float red[16][256];
   if ((int)blockIdx.x >= longlist[0]) return;
@@ -813,7 +813,7 @@ __global__ __launch_bounds__(256) void bwd_dw_long_kernel(const int32_t* __restr
         const int n = n0 + 16 * u;
         const int e = n < L ? perm[s0 + n] : -1;          // entry id k * Np + i
         h[u] = e >= 0 ? hcoef[e] : 0.f;
-        raw[u] = *reinterpret_cast<const v4i*>(xcol + (int64_t)(e >= 0 ? e % Np : 0) * dp);
+        raw[u] = *reinterpret_cast<const v4i*>(xcol + (int64_t)(e >= 0 ? e % Np : 0) * ldx);
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {        // rows in ascending order within a row-lane
@@ -843,7 +843,7 @@ __global__ __launch_bounds__(256) void bwd_dw_long_kernel(const int32_t* __restr
 template <typename T>
 __global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restrict__ dwacc, int nparts, int64_t part_stride, int64_t Vp, const int32_t* __restrict__ segoff,
                                                           const int32_t* __restrict__ perm, const float* __restrict__ hcoef,
-                                                          const uint8_t* __restrict__ xq, int64_t dp, int Np, const float* __restrict__ xi,
+                                                          const uint8_t* __restrict__ xq, int64_t ldx, int Np, const float* __restrict__ xi,
                                                           float x_s, int d, int V, T* __restrict__ dw, int64_t dw_ld) {
   const int t = threadIdx.x;
   const int v = blockIdx.x * 64 + (t & 63);
@@ -862,7 +862,7 @@ __global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restri
     for (int n = 0; n < L; ++n) {
       const int e = perm[s0 + n];                         // entry id k * Np + i
       const float h = hcoef[e] * x_s;
-      const v4i raw = *reinterpret_cast<const v4i*>(xq + (int64_t)(e % Np) * dp + j0);
+      const v4i raw = *reinterpret_cast<const v4i*>(xq + (int64_t)(e % Np) * ldx + j0);
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
         const uint32_t w = (uint32_t)raw[m];
@@ -1004,6 +1004,7 @@ constexpr size_t DX_PART_BYTES = (size_t)256 * 256 * 256 * 4;
 static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int nparts, int K) {
   BwdLayout B;
   B.P = P; B.Pw = Pw; B.nparts = nparts;
+  B.ldn = row_stride(S.Np); B.ldw = row_stride(Pw);
   size_t o = 0;
   auto take = [&](size_t bytes) { size_t r = o; o += (bytes + 255) / 256 * 256; return r; };
   B.off_crow = take((size_t)S.Np * 4);
@@ -1011,7 +1012,7 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int npa
   B.off_hcoef = take((size_t)S.Np * 4 * K);
   B.off_blockmax = take((size_t)(S.Np / 256) * 4);
   B.off_xi = take(256);
-  B.off_xt = take((size_t)S.dq * S.Np);
+  B.off_xt = take((size_t)S.dq * B.ldn);
   B.off_perm = take((size_t)S.N * K * 4 * 2);  // sorted values + unsorted values, one entry per (offset, row)
   B.off_keys = take((size_t)S.N * K * 4 * 2);  // sorted keys + unsorted keys
   B.off_segoff = take((size_t)(S.V + 2) * 4);
@@ -1020,8 +1021,8 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int npa
   B.off_sorttmp = take(B.sorttmp_bytes);
   B.off_dxpart = take(DX_PART_BYTES);
   B.fixed = o;
-  B.off_ghat = take((size_t)P * S.Vp);
-  B.off_ghat_t = take((size_t)S.Vp * Pw);
+  B.off_ghat = take((size_t)P * S.ldv);
+  B.off_ghat_t = take((size_t)S.Vp * B.ldw);
   B.part_stride = ((size_t)S.dq * S.Vp * 4 + 255) / 256 * 256;
   B.off_dwacc = take(B.part_stride * (size_t)nparts);     // fp32 dW partials, one per dW launch
   B.total = o;
@@ -1040,7 +1041,7 @@ static int64_t default_panel(const SavedLayout& S) {
 // Rows per dW launch: several dX panels are gathered (transposed) before dW runs, so that its
 // fp32 accumulator is read and rewritten less often and its K loop is long.
 static int64_t default_dw_panel(const SavedLayout& S, int64_t P) {
-  int64_t m = 24576 / P;
+  int64_t m = 40960 / P;
   if (m < 1) m = 1;
   int64_t Pw = m * P;
   const int64_t cap = round_up(S.Np, P);
@@ -1187,22 +1188,22 @@ extern "C" int sce_forward(const sce_args* a) {
     KernelTimer tm(SCE_K_QUANT, st);
     const int grid = grid_for((size_t)S.Np * (S.dp / 16), 256);
     if (a->x_dtype == SCE_F32)
-      quantize_pad_kernel<float><<<grid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, a->x_s);
+      quantize_pad_kernel<float><<<grid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, S.ldx, a->x_s);
     else if (a->x_dtype == SCE_BF16)
-      quantize_pad_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, a->x_s);
+      quantize_pad_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, S.ldx, a->x_s);
     else return fail(SCE_EINVAL, "unsupported x dtype %d", a->x_dtype);
     dim3 gw((unsigned)(S.Vp / 64), (unsigned)(S.dq / 64));
     if (a->wcache && a->wcache_valid) {
       // the caller vouches that the cache holds e4m3(W / w_s) of this W (unchanged since an earlier call)
     } else if (a->w_dtype == SCE_F32)
-      quantize_w_kernel<float><<<gw, 256, 0, st>>>((const float*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.Vp, a->w_s);
+      quantize_w_kernel<float><<<gw, 256, 0, st>>>((const float*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.ldv, a->w_s);
     else if (a->w_dtype == SCE_BF16)
-      quantize_w_kernel<bf16_t><<<gw, 256, 0, st>>>((const bf16_t*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.Vp, a->w_s);
+      quantize_w_kernel<bf16_t><<<gw, 256, 0, st>>>((const bf16_t*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.ldv, a->w_s);
     else return fail(SCE_EINVAL, "unsupported w dtype %d", a->w_dtype);
   }
   FwdParams p;
   p.xq = xq; p.wqt = wqt; p.partials = (float4*)a->workspace;
-  p.dp = S.dp; p.N = (int)N; p.V = (int)Vl; p.Np = (int)S.Np; p.RT = RT; p.CT = CT; p.S = nsplit;
+  p.dp = S.dp; p.ldx = S.ldx; p.N = (int)N; p.V = (int)Vl; p.Np = (int)S.Np; p.RT = RT; p.CT = CT; p.S = nsplit;
   p.sc = a->x_s * a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.c2 = -2.0f * a->cap * LOG2E;
   const int grid = 8 * nsplit * ((RT + 7) / 8);
   {
@@ -1214,7 +1215,7 @@ extern "C" int sce_forward(const sce_args* a) {
   float* s_umax = (float*)(sv + S.off_umax);
   float* s_zy = (float*)(sv + S.off_zy);
   fwd_target_logit_kernel<<<dim3((unsigned)((N + 3) / 4), (unsigned)a->shape.n_predict), 256, 0, st>>>(
-      xq, wqt, S.dp, a->targets, a->ignore_index, (int)N, (int)S.Np, (int)Vl, a->x_s * a->w_s, a->cap, s_zy);
+      xq, wqt, S.dp, S.ldx, a->targets, a->ignore_index, (int)N, (int)S.Np, (int)Vl, a->x_s * a->w_s, a->cap, s_zy);
   fwd_combine_kernel<<<(int)(S.Np / 256), 256, 0, st>>>(p.partials, nsplit, (int)N, (int)S.Np, (int)Vl, a->targets, a->ignore_index,
                                                        a->cap, a->mtp_weights, a->shape.n_predict, s_lse, s_umax, s_zy, a->losses, a->lse,
                                                        a->argmax);
@@ -1242,21 +1243,27 @@ extern "C" int sce_backward(const sce_args* a) {
   const BwdLayout Bmin = bwd_layout(S, 256, 256, 1, K);
   if (a->workspace_bytes < Bmin.total) return fail(SCE_EINVAL, "backward workspace too small: %zu < %zu", a->workspace_bytes, Bmin.total);
   // panel sizes from what the caller gave: P rows per recompute/dX panel, Pw = m * P rows per dW launch
-  const size_t room = (a->workspace_bytes - Bmin.fixed - Bmin.part_stride) / (size_t)S.Vp;     // rows of e4m3 scratch available
+  // bytes left for the two e4m3 copies of dlogits: P rows of ldv bytes and Vp rows of Pw + 128 bytes
+  const int64_t room = (int64_t)(a->workspace_bytes - Bmin.fixed - Bmin.part_stride) - 128 * S.Vp;
   int64_t P = default_panel(S);
   if (a->panel_rows > 0) {
     if (a->panel_rows % 256) return fail(SCE_EINVAL, "panel_rows must be a multiple of 256");
     P = a->panel_rows < S.Np ? a->panel_rows : S.Np;
   }
-  if ((int64_t)(room / 2) < P) P = (int64_t)(room / 2) / 256 * 256;
-  if (P < 256) return fail(SCE_EINVAL, "backward workspace too small for one 256-row panel");
+  if (P * (S.ldv + S.Vp) > room) P = room / (S.ldv + S.Vp) / 256 * 256;
+  if (P < 256) P = 256;                                  // Bmin fits, as checked above
   int64_t Pw = default_dw_panel(S, P);
-  if ((int64_t)room - P < Pw) Pw = ((int64_t)room - P) / P * P;
-  if (Pw < P) return fail(SCE_EINVAL, "internal: dW panel smaller than the dX panel");
+  if (P * S.ldv + Pw * S.Vp > room) Pw = (room - P * S.ldv) / S.Vp / P * P;
+  if (Pw < P) Pw = P;
   int nparts = dw_launches(S, Pw);
-  while (nparts > 1 && bwd_layout(S, P, Pw, nparts, K).total > a->workspace_bytes) --nparts;
+  // the estimate above ignores the 256-byte alignment of each region: settle on a layout that fits
+  while (bwd_layout(S, P, Pw, nparts, K).total > a->workspace_bytes) {
+    if (nparts > 1) --nparts;
+    else if (Pw > P) Pw -= P;
+    else if (P > 256) { P -= 256; Pw = P; }
+    else return fail(SCE_EINVAL, "internal: panel layout exceeds workspace");
+  }
   const BwdLayout B = bwd_layout(S, P, Pw, nparts, K);
-  if (B.total > a->workspace_bytes) return fail(SCE_EINVAL, "internal: panel layout exceeds workspace");
   DeviceGuard guard(a->device);
   if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", a->device);
   hipStream_t st = (hipStream_t)a->stream;
@@ -1295,7 +1302,7 @@ extern "C" int sce_backward(const sce_args* a) {
   bwd_xi_kernel<<<1, 1024, 0, st>>>(blockmax, nblk, xi);
   {
     dim3 g((unsigned)(S.Np / 64), (unsigned)(S.dq / 64));
-    bwd_xt_kernel<<<g, 256, 0, st>>>(xq, S.dp, S.Np, rho, xi, xt);
+    bwd_xt_kernel<<<g, 256, 0, st>>>(xq, S.dp, S.ldx, B.ldn, rho, xi, xt);
   }
   // rows grouped by target, for the one-hot part of dW
   {
@@ -1317,8 +1324,8 @@ extern "C" int sce_backward(const sce_args* a) {
     const int64_t prow = (S.Np - p0 < P) ? (S.Np - p0) : P;     // multiple of 256
     const int RTp = (int)(prow / 256);
     RecomputeParams rp;
-    rp.xq = xq + p0 * S.dp; rp.wqt = wqt; rp.crow = crow + p0; rp.ghat = ghat; rp.ghat_t = ghat_t + (p0 - w0);
-    rp.dp = S.dp; rp.Vp = S.Vp; rp.Pw = Pw; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2;
+    rp.xq = xq + p0 * S.ldx; rp.wqt = wqt; rp.crow = crow + p0; rp.ghat = ghat; rp.ghat_t = ghat_t + (p0 - w0);
+    rp.dp = S.dp; rp.ldx = S.ldx; rp.ldv = S.ldv; rp.ldw = B.ldw; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2;
     {
       KernelTimer tm(SCE_K_RECOMPUTE, st);
       bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_RECOMPUTE, st>>>(rp);
@@ -1326,7 +1333,7 @@ extern "C" int sce_backward(const sce_args* a) {
 
     DxParams dp_;
     dp_.wq = wq; dp_.ghat = ghat; dp_.wqt = wqt; dp_.rho = rho + p0; dp_.hcoef = hcoef + p0; dp_.targets = a->targets + p0;
-    dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.dp = S.dp; dp_.Np = S.Np; dp_.dq = S.dq; dp_.RT = RTp; dp_.CT = CTd;
+    dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.ldv = S.ldv; dp_.ldx = S.ldx; dp_.Np = S.Np; dp_.dq = S.dq; dp_.RT = RTp; dp_.CT = CTd;
     dp_.n_predict = K; dp_.rows_left = (int)(N - p0 > 0 ? N - p0 : 0);
     dp_.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); dp_.d = (int)d; dp_.V = (int)Vl; dp_.w_s = a->w_s;
     dp_.part = (float*)(ws + B.off_dxpart);
@@ -1360,7 +1367,7 @@ extern "C" int sce_backward(const sce_args* a) {
       DwParams wp;
       const int part = launch < nparts ? launch : nparts - 1;
       wp.xt = xt + w0; wp.ghat_t = ghat_t; wp.dwacc = (float*)((uint8_t*)dwacc + (size_t)part * B.part_stride);
-      wp.Np = S.Np; wp.Pw = Pw; wp.Vp = S.Vp;
+      wp.ldn = B.ldn; wp.ldw = B.ldw; wp.Vp = S.Vp;
       wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(gathered / BK); wp.accumulate = launch >= nparts ? 1 : 0;
       {
         KernelTimer tm(SCE_K_DW, st);
@@ -1371,14 +1378,14 @@ extern "C" int sce_backward(const sce_args* a) {
     }
   }
   KernelTimer tm_fin(SCE_K_DW_FINAL, st);
-  bwd_dw_long_kernel<<<dim3((unsigned)(NE / LONG_SEG + 1), (unsigned)(S.dq / 256)), 256, 0, st>>>(longlist, segoff, perm, hcoef, xq, S.dp, S.Vp, (int)S.Np, xi, dwacc);
+  bwd_dw_long_kernel<<<dim3((unsigned)(NE / LONG_SEG + 1), (unsigned)(S.dq / 256)), 256, 0, st>>>(longlist, segoff, perm, hcoef, xq, S.dp, S.ldx, S.Vp, (int)S.Np, xi, dwacc);
   {
     dim3 g((unsigned)((V + 63) / 64), (unsigned)((d + 63) / 64));
     if (a->dw_dtype == SCE_F32)
-      bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.dp, (int)S.Np, xi, a->x_s, (int)d, (int)V,
+      bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, a->x_s, (int)d, (int)V,
                                                    (float*)a->dw, a->dw_ld);
     else
-      bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.dp, (int)S.Np, xi, a->x_s, (int)d, (int)V,
+      bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, a->x_s, (int)d, (int)V,
                                                     (bf16_t*)a->dw, a->dw_ld);
   }
   HIP_TRY(hipGetLastError());
