@@ -24,6 +24,7 @@ constexpr int NTHREADS = 256;
 
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr int LONG_SEG = 64;     // target columns hit by at least this many rows get their own reduction kernel
+constexpr int LONG_CHUNK = 1024; // ... which handles at most about this many rows per workgroup
 
 static inline int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 // Row stride of an MFMA operand with K = k bytes (a multiple of 256): the next odd multiple of 128.
@@ -67,7 +68,7 @@ struct BwdLayout {
   int64_t P, Pw;                     // rows per recompute/dX panel and per dW launch (multiples of 256, Pw of P)
   int64_t ldn, ldw;                  // row strides of X~^T [dq][Np] and of G^T [Vp][Pw]
   size_t off_crow, off_rho, off_hcoef, off_blockmax, off_xi, off_xt, off_dwacc, off_perm, off_keys,
-      off_segoff, off_longlist, off_sorttmp, off_dxpart, off_ghat, off_ghat_t, fixed, total;
+      off_segoff, off_longlist, off_longsum, off_sorttmp, off_dxpart, off_ghat, off_ghat_t, fixed, total;
   size_t sorttmp_bytes, part_stride;   // part_stride: bytes between consecutive fp32 dW partials
   int nparts;
 };

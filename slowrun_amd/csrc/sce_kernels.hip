@@ -778,26 +778,43 @@ __global__ __launch_bounds__(256) void bwd_segoff_kernel(const int32_t* __restri
 }
 
 
-// List of the columns that are the target of at least LONG_SEG rows (order irrelevant: each
-// column is handled on its own).  longlist[0] is the count.
+// A column that is the target of at least LONG_SEG rows has its segment of the sorted list cut into
+// nch = ceil(L / LONG_CHUNK) equal chunks of at least LONG_SEG rows each; chunk c starts at sorted
+// position s0 + c * ceil(L / nch).  Distinct chunks start at least LONG_SEG positions apart, so
+// (start / LONG_SEG) is a slot of its own in the array of chunk sums.
+__device__ __forceinline__ void long_chunks(int L, int& nch, int& len) {
+  nch = (L + LONG_CHUNK - 1) / LONG_CHUNK;
+  len = (L + nch - 1) / nch;
+}
+
+// List of (column, chunk) pairs of the long columns (order irrelevant: each pair is handled on its
+// own).  longlist[0] is the count, then two ints per pair.
 __global__ __launch_bounds__(256) void bwd_longlist_kernel(const int32_t* __restrict__ segoff, int V, int32_t* __restrict__ longlist) {
   const int v = blockIdx.x * 256 + threadIdx.x;
   if (v >= V) return;
-  if (segoff[v + 1] - segoff[v] >= LONG_SEG) longlist[1 + atomicAdd(&longlist[0], 1)] = v;
+  const int L = segoff[v + 1] - segoff[v];
+  if (L < LONG_SEG) return;
+  int nch, len;
+  long_chunks(L, nch, len);
+  const int at = atomicAdd(&longlist[0], nch);
+  for (int c = 0; c < nch; ++c) { longlist[1 + 2 * (at + c)] = v; longlist[2 + 2 * (at + c)] = c; }
 }
 
-// Columns that are the target of many rows: dwacc[:, v] -= sum_i h_i X_q[i, :] / xi.  One
-// workgroup per (long column, block of 256 rows of dW); the rows of the segment are split over
-// 16 row-lanes (8 independent loads in flight each) and folded in a fixed order, so the result
-// does not depend on scheduling.
+// One-hot part of dW for the long columns: longsum[slot][:] = sum over the chunk's rows of h_i X_q[i, :].
+// One workgroup per (chunk, block of 256 rows of dW); the rows of the chunk are split over 16
+// row-lanes (8 independent loads in flight each) and folded in a fixed order, so the result does
+// not depend on scheduling.
 __global__ __launch_bounds__(256) void bwd_dw_long_kernel(const int32_t* __restrict__ longlist, const int32_t* __restrict__ segoff,
                                                          const int32_t* __restrict__ perm, const float* __restrict__ hcoef,
-                                                         const uint8_t* __restrict__ xq, int64_t dp, int64_t ldx, int64_t Vp, int Np,
-                                                         const float* __restrict__ xi, float* __restrict__ dwacc) {
+                                                         const uint8_t* __restrict__ xq, int64_t dp, int64_t ldx, int64_t dq, int Np,
+                                                         float* __restrict__ longsum) {
   __shared__ float red[16][256];
   if ((int)blockIdx.x >= longlist[0]) return;
-  const int v = longlist[1 + blockIdx.x];
-  const int s0 = segoff[v], L = segoff[v + 1] - s0;
+  const int v = longlist[1 + 2 * blockIdx.x], ch = longlist[2 + 2 * blockIdx.x];
+  int nch, len;
+  long_chunks(segoff[v + 1] - segoff[v], nch, len);
+  const int s0 = segoff[v] + ch * len;
+  const int L = (segoff[v + 1] - s0) < len ? (segoff[v + 1] - s0) : len;
   const int t = threadIdx.x, c = t & 15, rl = t >> 4;
   const int64_t jb = (int64_t)blockIdx.y * 256;
   float a[16];
@@ -834,16 +851,17 @@ __global__ __launch_bounds__(256) void bwd_dw_long_kernel(const int32_t* __restr
   float sfold = 0.f;
 #pragma unroll
   for (int k = 0; k < 16; ++k) sfold += red[k][t];
-  float* dst = dwacc + (jb + t) * Vp + v;
-  *dst -= sfold / xi[0];
+  longsum[(int64_t)(s0 / LONG_SEG) * dq + jb + t] = sfold;
 }
 
-// dW = x_s * ( xi * (sum of the dW partials) - sum over the (short) target segment of h_i X_q[i, :] ), cast to the
-// output type.  A thread owns one column v and 16 consecutive rows j.
+// dW = x_s * ( xi * (sum of the dW partials) - sum over the target segment of h_i X_q[i, :] ), cast to the output
+// type; the segment sum is formed here for short segments and read from the chunk sums for long ones.  A thread
+// owns one column v and 16 consecutive rows j.
 template <typename T>
 __global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restrict__ dwacc, int nparts, int64_t part_stride, int64_t Vp, const int32_t* __restrict__ segoff,
                                                           const int32_t* __restrict__ perm, const float* __restrict__ hcoef,
                                                           const uint8_t* __restrict__ xq, int64_t ldx, int Np, const float* __restrict__ xi,
+                                                          const float* __restrict__ longsum, int64_t dq,
                                                           float x_s, int d, int V, T* __restrict__ dw, int64_t dw_ld) {
   const int t = threadIdx.x;
   const int v = blockIdx.x * 64 + (t & 63);
@@ -858,7 +876,15 @@ __global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restri
     o[m] = sum * scale;
   }
   const int s0 = segoff[v], L = segoff[v + 1] - s0;
-  if (L > 0 && L < LONG_SEG) {
+  if (L >= LONG_SEG) {
+    int nch, len;
+    long_chunks(L, nch, len);
+    for (int c = 0; c < nch; ++c) {                       // fixed order
+      const float* ls = longsum + (int64_t)((s0 + c * len) / LONG_SEG) * dq + j0;
+#pragma unroll
+      for (int m = 0; m < 16; ++m) o[m] -= ls[m] * x_s;
+    }
+  } else if (L > 0) {
     for (int n = 0; n < L; ++n) {
       const int e = perm[s0 + n];                         // entry id k * Np + i
       const float h = hcoef[e] * x_s;
@@ -1016,7 +1042,8 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int npa
   B.off_perm = take((size_t)S.N * K * 4 * 2);  // sorted values + unsorted values, one entry per (offset, row)
   B.off_keys = take((size_t)S.N * K * 4 * 2);  // sorted keys + unsorted keys
   B.off_segoff = take((size_t)(S.V + 2) * 4);
-  B.off_longlist = take((size_t)(S.N * K / LONG_SEG + 2) * 4);
+  B.off_longlist = take((size_t)(2 * (S.N * K / LONG_SEG + 1) + 2) * 4);   // (column, chunk) pairs: at most one per LONG_SEG entries
+  B.off_longsum = take((size_t)(S.N * K / LONG_SEG + 1) * S.dq * 4);      // chunk sums, one slot per LONG_SEG sorted positions
   B.sorttmp_bytes = sort_tmp_bytes(S.N * K, S.V);
   B.off_sorttmp = take(B.sorttmp_bytes);
   B.off_dxpart = take(DX_PART_BYTES);
@@ -1291,6 +1318,7 @@ extern "C" int sce_backward(const sce_args* a) {
   int32_t* keys_in = skeys + NE;
   int32_t* segoff = (int32_t*)(ws + B.off_segoff);
   int32_t* longlist = (int32_t*)(ws + B.off_longlist);
+  float* longsum = (float*)(ws + B.off_longsum);
   uint8_t* ghat = ws + B.off_ghat;
   uint8_t* ghat_t = ws + B.off_ghat_t;
 
@@ -1378,14 +1406,14 @@ extern "C" int sce_backward(const sce_args* a) {
     }
   }
   KernelTimer tm_fin(SCE_K_DW_FINAL, st);
-  bwd_dw_long_kernel<<<dim3((unsigned)(NE / LONG_SEG + 1), (unsigned)(S.dq / 256)), 256, 0, st>>>(longlist, segoff, perm, hcoef, xq, S.dp, S.ldx, S.Vp, (int)S.Np, xi, dwacc);
+  bwd_dw_long_kernel<<<dim3((unsigned)(NE / LONG_SEG + 1), (unsigned)(S.dq / 256)), 256, 0, st>>>(longlist, segoff, perm, hcoef, xq, S.dp, S.ldx, S.dq, (int)S.Np, longsum);
   {
     dim3 g((unsigned)((V + 63) / 64), (unsigned)((d + 63) / 64));
     if (a->dw_dtype == SCE_F32)
-      bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, a->x_s, (int)d, (int)V,
+      bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, S.dq, a->x_s, (int)d, (int)V,
                                                    (float*)a->dw, a->dw_ld);
     else
-      bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, a->x_s, (int)d, (int)V,
+      bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, S.dq, a->x_s, (int)d, (int)V,
                                                     (bf16_t*)a->dw, a->dw_ld);
   }
   HIP_TRY(hipGetLastError());
