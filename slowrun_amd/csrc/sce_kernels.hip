@@ -492,8 +492,16 @@ __global__ __launch_bounds__(1024) void bwd_xi_kernel(const float* __restrict__ 
   if (threadIdx.x == 0) xi[0] = (smax[0] > 0.f && isfinite(smax[0])) ? smax[0] : 1.0f;
 }
 
-// Xt [dq][Np] = e4m3( X_q[i][j] * rho_i / xi ), transposed through LDS in 64 x 64 tiles.
-__global__ __launch_bounds__(256) void bwd_xt_kernel(const uint8_t* __restrict__ xq, int64_t dp, int64_t ldx, int64_t ldn,
+// The two operands of dW are stored tile by tile: for every 256 rows, K block after K block, 256 rows of
+// 128 bytes each.  A workgroup's load of one K block of one operand is then one contiguous 32 KB piece
+// (row-major rows lie Np or Pw bytes apart, and the dW main loop lost 12 % to that at K = 65536).
+__device__ __forceinline__ int64_t blocked_offset(int64_t row, int64_t k, int64_t kblocks) {
+  return (((row >> 8) * kblocks + (k >> 7)) * 256 + (row & 255)) * 128 + (k & 127);
+}
+constexpr int BLOCKED_KSTEP = 256 * BK;     // bytes from one K block of a tile to the next
+
+// Xt (blocked, dq rows, K = Np) = e4m3( X_q[i][j] * rho_i / xi ), transposed through LDS in 64 x 64 tiles.
+__global__ __launch_bounds__(256) void bwd_xt_kernel(const uint8_t* __restrict__ xq, int64_t dp, int64_t ldx, int64_t kbn,
                                                     const float* __restrict__ rho, const float* __restrict__ xi,
                                                     uint8_t* __restrict__ xt) {
   __shared__ uint8_t tile[64][68];
@@ -521,7 +529,7 @@ __global__ __launch_bounds__(256) void bwd_xt_kernel(const uint8_t* __restrict__
     out[m] = (uint32_t)tile[ic + 4 * m][jr] | ((uint32_t)tile[ic + 4 * m + 1][jr] << 8) |
              ((uint32_t)tile[ic + 4 * m + 2][jr] << 16) | ((uint32_t)tile[ic + 4 * m + 3][jr] << 24);
   }
-  *reinterpret_cast<v4i*>(xt + (j0 + jr) * ldn + i0 + ic) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
+  *reinterpret_cast<v4i*>(xt + blocked_offset(j0 + jr, i0 + ic, kbn)) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
 }
 
 struct RecomputeParams {
@@ -529,8 +537,9 @@ struct RecomputeParams {
   const uint8_t* wqt;    // [Vp][dp]
   const float* crow;     // offset to the panel's first row
   uint8_t* ghat;         // [P][Vp]
-  uint8_t* ghat_t;       // [Vp][Pw], already offset to this panel's first column
-  int64_t dp, ldx, ldv, ldw;   // K extent; row strides of xq / wqt, of ghat and of ghat_t
+  uint8_t* ghat_t;       // Vp rows, K = Pw, blocked
+  int64_t dp, ldx, ldv;        // K extent; row strides of xq / wqt and of ghat
+  int64_t kbw, kb0;            // ghat_t (blocked): K blocks per tile, K block of this panel's first row
   int RT, CT, V;
   float k1, c2;          // as in FwdParams
 };
@@ -600,12 +609,12 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   if (edge) form_g(std::true_type{}); else form_g(std::false_type{});
   __syncthreads();
   uint8_t* grow = p.ghat + (int64_t)rt * 256 * p.ldv + (int64_t)ct * 256;
-  uint8_t* gcol = p.ghat_t + (int64_t)ct * 256 * p.ldw + (int64_t)rt * 256;
+  uint8_t* gcol = p.ghat_t + ((int64_t)ct * p.kbw + p.kb0 + 2 * rt) * BLOCKED_KSTEP;   // two K blocks of 256 rows x 128 B
 #pragma unroll
   for (int n = 0; n < 16; ++n) {
     const int cidx = t + 256 * n, row = cidx >> 4, col = (cidx & 15) * 16;
     *reinterpret_cast<v4i*>(grow + (int64_t)row * p.ldv + col) = *reinterpret_cast<const v4i*>(T + row * STG_PITCH + col);
-    *reinterpret_cast<v4i*>(gcol + (int64_t)row * p.ldw + col) = *reinterpret_cast<const v4i*>(TT + row * STG_PITCH + col);
+    *reinterpret_cast<v4i*>(gcol + (col >> 7) * BLOCKED_KSTEP + row * BK + (col & 127)) = *reinterpret_cast<const v4i*>(TT + row * STG_PITCH + col);
   }
 }
 
@@ -723,10 +732,10 @@ __global__ __launch_bounds__(256) void bwd_dx_finish_kernel(DxParams p) {
 }
 
 struct DwParams {
-  const uint8_t* xt;      // [dq][Np], offset to the first row of the dW panel   A side (rows j)
-  const uint8_t* ghat_t;  // [Vp][Pw]                                             B side (rows v)
+  const uint8_t* xt;      // dq rows, K = Np, blocked                             A side (rows j)
+  const uint8_t* ghat_t;  // Vp rows, K = Pw, blocked                             B side (rows v)
   float* dwacc;           // [dq][Vp] fp32
-  int64_t ldn, ldw, Vp;   // row strides of xt and of ghat_t; row length of dwacc
+  int64_t kbn, kbw, kb0, Vp;   // K blocks per tile of xt and of ghat_t; first K block of xt in this launch; row length of dwacc
   int RT, CT, KT, accumulate;
 };
 
@@ -736,7 +745,8 @@ __global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
   if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
-  mfma_mainloop(p.xt + (int64_t)rt * 256 * p.ldn, p.ldn, p.ghat_t + (int64_t)ct * 256 * p.ldw, p.ldw, p.KT, smem, acc, ct & 7, 2 * (rt & 3));
+  mfma_mainloop<false, NoHook, BLOCKED_KSTEP>(p.xt + ((int64_t)rt * p.kbn + p.kb0) * BLOCKED_KSTEP, BK, p.ghat_t + (int64_t)ct * p.kbw * BLOCKED_KSTEP, BK, p.KT,
+                                              smem, acc, ct & 7, 2 * (rt & 3));
   const int jbase = rt * 256 + wa * 128 + 4 * (lane >> 5);
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
@@ -1030,7 +1040,6 @@ constexpr size_t DX_PART_BYTES = (size_t)256 * 256 * 256 * 4;
 static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int nparts, int K) {
   BwdLayout B;
   B.P = P; B.Pw = Pw; B.nparts = nparts;
-  B.ldn = row_stride(S.Np); B.ldw = row_stride(Pw);
   size_t o = 0;
   auto take = [&](size_t bytes) { size_t r = o; o += (bytes + 255) / 256 * 256; return r; };
   B.off_crow = take((size_t)S.Np * 4);
@@ -1038,7 +1047,7 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int npa
   B.off_hcoef = take((size_t)S.Np * 4 * K);
   B.off_blockmax = take((size_t)(S.Np / 256) * 4);
   B.off_xi = take(256);
-  B.off_xt = take((size_t)S.dq * B.ldn);
+  B.off_xt = take((size_t)S.dq * S.Np);
   B.off_perm = take((size_t)S.N * K * 4 * 2);  // sorted values + unsorted values, one entry per (offset, row)
   B.off_keys = take((size_t)S.N * K * 4 * 2);  // sorted keys + unsorted keys
   B.off_segoff = take((size_t)(S.V + 2) * 4);
@@ -1049,7 +1058,7 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int npa
   B.off_dxpart = take(DX_PART_BYTES);
   B.fixed = o;
   B.off_ghat = take((size_t)P * S.ldv);
-  B.off_ghat_t = take((size_t)S.Vp * B.ldw);
+  B.off_ghat_t = take((size_t)S.Vp * Pw);
   B.part_stride = ((size_t)S.dq * S.Vp * 4 + 255) / 256 * 256;
   B.off_dwacc = take(B.part_stride * (size_t)nparts);     // fp32 dW partials, one per dW launch
   B.total = o;
@@ -1068,7 +1077,7 @@ static int64_t default_panel(const SavedLayout& S) {
 // Rows per dW launch: several dX panels are gathered (transposed) before dW runs, so that its
 // fp32 accumulator is read and rewritten less often and its K loop is long.
 static int64_t default_dw_panel(const SavedLayout& S, int64_t P) {
-  int64_t m = 40960 / P;
+  int64_t m = 131072 / P;
   if (m < 1) m = 1;
   int64_t Pw = m * P;
   const int64_t cap = round_up(S.Np, P);
@@ -1270,8 +1279,8 @@ extern "C" int sce_backward(const sce_args* a) {
   const BwdLayout Bmin = bwd_layout(S, 256, 256, 1, K);
   if (a->workspace_bytes < Bmin.total) return fail(SCE_EINVAL, "backward workspace too small: %zu < %zu", a->workspace_bytes, Bmin.total);
   // panel sizes from what the caller gave: P rows per recompute/dX panel, Pw = m * P rows per dW launch
-  // bytes left for the two e4m3 copies of dlogits: P rows of ldv bytes and Vp rows of Pw + 128 bytes
-  const int64_t room = (int64_t)(a->workspace_bytes - Bmin.fixed - Bmin.part_stride) - 128 * S.Vp;
+  // bytes left for the two e4m3 copies of dlogits: P rows of ldv bytes and Vp rows of Pw bytes
+  const int64_t room = (int64_t)(a->workspace_bytes - Bmin.fixed - Bmin.part_stride);
   int64_t P = default_panel(S);
   if (a->panel_rows > 0) {
     if (a->panel_rows % 256) return fail(SCE_EINVAL, "panel_rows must be a multiple of 256");
@@ -1330,7 +1339,7 @@ extern "C" int sce_backward(const sce_args* a) {
   bwd_xi_kernel<<<1, 1024, 0, st>>>(blockmax, nblk, xi);
   {
     dim3 g((unsigned)(S.Np / 64), (unsigned)(S.dq / 64));
-    bwd_xt_kernel<<<g, 256, 0, st>>>(xq, S.dp, S.ldx, B.ldn, rho, xi, xt);
+    bwd_xt_kernel<<<g, 256, 0, st>>>(xq, S.dp, S.ldx, S.Np / BK, rho, xi, xt);
   }
   // rows grouped by target, for the one-hot part of dW
   {
@@ -1352,8 +1361,8 @@ extern "C" int sce_backward(const sce_args* a) {
     const int64_t prow = (S.Np - p0 < P) ? (S.Np - p0) : P;     // multiple of 256
     const int RTp = (int)(prow / 256);
     RecomputeParams rp;
-    rp.xq = xq + p0 * S.ldx; rp.wqt = wqt; rp.crow = crow + p0; rp.ghat = ghat; rp.ghat_t = ghat_t + (p0 - w0);
-    rp.dp = S.dp; rp.ldx = S.ldx; rp.ldv = S.ldv; rp.ldw = B.ldw; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2;
+    rp.xq = xq + p0 * S.ldx; rp.wqt = wqt; rp.crow = crow + p0; rp.ghat = ghat; rp.ghat_t = ghat_t;
+    rp.dp = S.dp; rp.ldx = S.ldx; rp.ldv = S.ldv; rp.kbw = Pw / BK; rp.kb0 = (p0 - w0) / BK; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2;
     {
       KernelTimer tm(SCE_K_RECOMPUTE, st);
       bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_RECOMPUTE, st>>>(rp);
@@ -1394,8 +1403,8 @@ extern "C" int sce_backward(const sce_args* a) {
     if (gathered + P > Pw || p0 + prow >= S.Np) {      // the transposed scratch is full, or this was the last panel
       DwParams wp;
       const int part = launch < nparts ? launch : nparts - 1;
-      wp.xt = xt + w0; wp.ghat_t = ghat_t; wp.dwacc = (float*)((uint8_t*)dwacc + (size_t)part * B.part_stride);
-      wp.ldn = B.ldn; wp.ldw = B.ldw; wp.Vp = S.Vp;
+      wp.xt = xt; wp.ghat_t = ghat_t; wp.dwacc = (float*)((uint8_t*)dwacc + (size_t)part * B.part_stride);
+      wp.kbn = S.Np / BK; wp.kbw = Pw / BK; wp.kb0 = w0 / BK; wp.Vp = S.Vp;
       wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(gathered / BK); wp.accumulate = launch >= nparts ? 1 : 0;
       {
         KernelTimer tm(SCE_K_DW, st);

@@ -82,7 +82,7 @@ struct NoHook { __device__ __forceinline__ void operator()(int) const {} };
 
 // `hook(i)` is called after MFMA i (0..63) of every pair of K blocks: a place for vector ALU work that
 // does not depend on the accumulators (it runs while the matrix pipe is busy).
-template <bool PREFETCHED = false, class Hook = NoHook>
+template <bool PREFETCHED = false, class Hook = NoHook, int KSTEP = BK>
 __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, int64_t lda,
                                               const uint8_t* __restrict__ Bg, int64_t ldb, int KD,
                                               uint8_t* smem, v16f (&acc)[4][4], int rot_a, int rot_b, Hook&& hook = NoHook()) {
@@ -114,7 +114,7 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
 #pragma unroll
     for (int n = 0; n < 16; ++n) ld.issue<0>(n, Ag, Bg);
 #pragma unroll
-    for (int n = 0; n < 8; ++n) ld.issue<1>(n, Ag + BK, Bg + BK);
+    for (int n = 0; n < 8; ++n) ld.issue<1>(n, Ag + KSTEP, Bg + KSTEP);
   }
   asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
   v8i fa[2][4], fb[2][4];
@@ -142,7 +142,7 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
     for (int i = 0; i < 8; ++i) {
       mm(0, i);
       hook(0 + (i & 7));
-      ld.issue<1>(8 + i, ga + BK, gb + BK);
+      ld.issue<1>(8 + i, ga + KSTEP, gb + KSTEP);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
@@ -165,7 +165,7 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
       mm(1, i);
       hook(24 + (i & 7));
       rfrag1(1, 0, i - 8, fa[0], fb[0]);
-      if (more) ld.issue<0>(i - 8, ga + 2 * BK, gb + 2 * BK);
+      if (more) ld.issue<0>(i - 8, ga + 2 * KSTEP, gb + 2 * KSTEP);
       __builtin_amdgcn_sched_barrier(0);
     }
     // ---- block 2p + 1 (slot 1)
@@ -173,7 +173,7 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
     for (int i = 0; i < 8; ++i) {
       mm(0, i);
       hook(32 + (i & 7));
-      if (more) ld.issue<0>(8 + i, ga + 2 * BK, gb + 2 * BK);
+      if (more) ld.issue<0>(8 + i, ga + 2 * KSTEP, gb + 2 * KSTEP);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
@@ -197,15 +197,15 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
       hook(56 + (i & 7));
       if (more) {
         rfrag1(0, 0, i - 8, fa[0], fb[0]);
-        ld.issue<1>(i - 8, ga + 3 * BK, gb + 3 * BK);
+        ld.issue<1>(i - 8, ga + 3 * KSTEP, gb + 3 * KSTEP);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
   for (int p = 0; p < (KD >> 1) - 1; ++p) {
     pair(true);
-    ga += 2 * BK;
-    gb += 2 * BK;
+    ga += 2 * KSTEP;
+    gb += 2 * KSTEP;
   }
   pair(false);
   // all LDS reads of this tile are complete in every wave before the caller reuses the buffer
