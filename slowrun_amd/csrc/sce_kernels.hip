@@ -557,6 +557,10 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   int rt, ct;
   if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
+  // The tile order goes through the columns in groups of 8, and it does so from the last group to the first:
+  // the dX kernel that follows starts its K loop at column 0, with the part of G that was written last and is
+  // still in the memory-side cache.
+  ct = p.CT - 1 - ct;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
   mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 2 * (rt & 3), ct & 7);
