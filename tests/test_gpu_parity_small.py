@@ -252,3 +252,22 @@ def test_fixed_scales_of_the_trainer_and_overflow_to_nan():
     ok = torch.ones(300, dtype=torch.bool, device="cuda")
     ok[17] = False
     assert float((ours["loss"][ok] - ref["loss"][ok]).abs().max()) < 1e-3
+
+
+def test_frequent_target_segments_are_chunked():
+    """One target shared by 3000 rows (its one-hot part of dW is summed in three chunks), one by 70 rows
+    (a single chunk) and the rest spread out (summed in the final kernel)."""
+    inp = _small("tiny_track", 4096, 128, 512)
+    inp.targets[:3000] = 7
+    inp.targets[3000:3070] = 11
+    ours = pu.run_ours(inp, "mean")
+    ref = pu.run_oracle(inp, ours, "mean")
+    print(pu.check_parity(ours, ref, "mean"))
+
+
+def test_dx_panel_with_few_tiles_is_k_split():
+    """512 rows x d = 256 is two dX tiles: each tile's K loop (V) is shared by several workgroups."""
+    inp = _small("limited_2p7b", 512, 256, 8192)
+    ours = pu.run_ours(inp, "none", x_dtype=torch.float32)
+    ref = pu.run_oracle(inp, ours, "none")
+    print(pu.check_parity(ours, ref, "none"))
