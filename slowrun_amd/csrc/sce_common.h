@@ -26,6 +26,16 @@ constexpr float LOG2E = 1.4426950408889634f;
 constexpr int LONG_SEG = 64;     // target columns hit by at least this many rows get their own reduction kernel
 constexpr int LONG_CHUNK = 1024; // ... which handles at most about this many rows per workgroup
 
+// Lane index within the wavefront, computed from the execution mask each time it is asked for.  Kernels
+// that loop over tiles use this (and a wave index kept in a scalar register) instead of threadIdx.x:
+// a value derived from threadIdx.x stays live across the main loop, is spilled there, and its reload
+// -- a vector memory load -- makes the next wait count include the tile loads already in flight.
+__device__ __forceinline__ int lane_id() {
+  int l = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  asm volatile("" : "+v"(l));
+  return l;
+}
+
 static inline int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 // Row stride of an MFMA operand with K = k bytes (a multiple of 256): the next odd multiple of 128.
 // With an even multiple the 256 rows of a tile fall on few L2 channels (measured: up to 9 % slower).

@@ -272,31 +272,56 @@ __device__ __forceinline__ void fwd_epilogue(const v16f (&acc)[4][4], const FwdP
   }
 }
 
+// The row statistics of a workgroup's walk (12 values per lane) wait in LDS behind the two K slots while the
+// main loop runs: kept in registers they are spilled around it, and the reload (a vector memory load) makes
+// the epilogue wait for the tile loads that were just put in flight for the next tile.
+constexpr int SMEM_FWD = SMEM_BYTES + 12 * 4 * NTHREADS;
+
 __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  const int bid = blockIdx.x, xcd = bid & 7, slot = bid >> 3;
-  const int s = slot % p.S, rt = (slot / p.S) * 8 + xcd;
-  if (rt >= p.RT) return;
+  int rt, s;
+  if (!map_tile(blockIdx.x, p.RT, p.S, rt, s)) return;
   const int ct0 = (int)((int64_t)p.CT * s / p.S), ct1 = (int)((int64_t)p.CT * (s + 1) / p.S);
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
-
-  float sum[4], amax[4];
-  int uarg[4];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wa = wave >> 1, wb = wave & 1;
+  float* stat = reinterpret_cast<float*>(smem + SMEM_BYTES) + wave * 64 + lane_id();   // [12][256]: sum, amax, uarg of the 4 row blocks
 #pragma unroll
-  for (int b = 0; b < 4; ++b) { sum[b] = 0.f; amax[b] = -INFINITY; uarg[b] = 0x7fffffff; }
+  for (int b = 0; b < 4; ++b) {
+    stat[(0 + b) * NTHREADS] = 0.f;
+    stat[(4 + b) * NTHREADS] = -INFINITY;
+    stat[(8 + b) * NTHREADS] = __int_as_float(0x7fffffff);
+  }
   v16f acc[4][4];
   const uint8_t* Bg = p.xq + (int64_t)rt * 256 * p.ldx;
   const int KT = (int)(p.dp / BK);
   // of the workgroups that start together on this XCD, those with the same split share the W tiles, those with the same rt the X rows
-  const int rot_a = 2 * ((slot / p.S) & 3), rot_b = s & 7;
-  // the first K blocks of the next tile travel while the epilogue of this one runs (it does not touch LDS)
-  if (ct0 < ct1) mfma_prefetch(p.wqt + (int64_t)ct0 * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b);
+  const int rot_a = 2 * (rt & 3), rot_b = s & 7;
+  // the first K blocks of the next tile travel while the epilogue of this one runs (it does not touch the K slots)
+  if (ct0 < ct1) mfma_prefetch(p.wqt + (int64_t)ct0 * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
   for (int ct = ct0; ct < ct1; ++ct) {
-    mfma_mainloop<true>(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, Bg, p.ldx, KT, smem, acc, rot_a, rot_b);
-    if (ct + 1 < ct1) mfma_prefetch(p.wqt + (int64_t)(ct + 1) * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b);
-    const int vbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
+    mfma_mainloop<true>(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, Bg, p.ldx, KT, smem, acc, rot_a, rot_b, wave);
+    if (ct + 1 < ct1) mfma_prefetch(p.wqt + (int64_t)(ct + 1) * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
+    float sum[4], amax[4];
+    int uarg[4];
+    float* stat = reinterpret_cast<float*>(smem + SMEM_BYTES) + wave * 64 + lane_id();
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      sum[b] = stat[(0 + b) * NTHREADS]; amax[b] = stat[(4 + b) * NTHREADS]; uarg[b] = __float_as_int(stat[(8 + b) * NTHREADS]);
+    }
+    const int vbase = ct * 256 + wa * 128 + 4 * (lane_id() >> 5);
     if (ct * 256 + 256 > p.V) fwd_epilogue<true>(acc, p, vbase, sum, amax, uarg);
     else fwd_epilogue<false>(acc, p, vbase, sum, amax, uarg);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      stat[(0 + b) * NTHREADS] = sum[b]; stat[(4 + b) * NTHREADS] = amax[b]; stat[(8 + b) * NTHREADS] = __int_as_float(uarg[b]);
+    }
+  }
+  float sum[4], amax[4];
+  int uarg[4];
+  const int lane = lane_id();
+  stat = reinterpret_cast<float*>(smem + SMEM_BYTES) + wave * 64 + lane;
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    sum[b] = stat[(0 + b) * NTHREADS]; amax[b] = stat[(4 + b) * NTHREADS]; uarg[b] = __float_as_int(stat[(8 + b) * NTHREADS]);
   }
   // the two half-waves hold different columns of the same rows
 #pragma unroll
@@ -563,7 +588,7 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   ct = p.CT - 1 - ct;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
-  mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 2 * (rt & 3), ct & 7);
+  mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave));
   uint8_t* T = smem;                         // [256 rows i][STG_PITCH]: columns v contiguous
   uint8_t* TT = smem + 256 * STG_PITCH;      // [256 columns v][STG_PITCH]: rows i contiguous
   const int vloc0 = wa * 128 + 4 * (lane >> 5);
@@ -690,7 +715,7 @@ __global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p) {
   }
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
-  mfma_mainloop(p.wq + (int64_t)ct * 256 * p.ldv + k0, p.ldv, p.ghat + (int64_t)rt * 256 * p.ldv + k0, p.ldv, KD, smem, acc, 2 * (rt & 3), ct & 7);
+  mfma_mainloop(p.wq + (int64_t)ct * 256 * p.ldv + k0, p.ldv, p.ghat + (int64_t)rt * 256 * p.ldv + k0, p.ldv, KD, smem, acc, 2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave));
   const int jbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
   T* dx = reinterpret_cast<T*>(p.dx);
 #pragma unroll
@@ -750,7 +775,7 @@ __global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
   mfma_mainloop<false, NoHook, BLOCKED_KSTEP>(p.xt + ((int64_t)rt * p.kbn + p.kb0) * BLOCKED_KSTEP, BK, p.ghat_t + (int64_t)ct * p.kbw * BLOCKED_KSTEP, BK, p.KT,
-                                              smem, acc, ct & 7, 2 * (rt & 3));
+                                              smem, acc, ct & 7, 2 * (rt & 3), __builtin_amdgcn_readfirstlane(wave));
   const int jbase = rt * 256 + wa * 128 + 4 * (lane >> 5);
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
@@ -1006,7 +1031,7 @@ static int check_device(int dev) {
     g_arch_ok[dev] = strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : -1;
     if (g_arch_ok[dev] == 1) {
       // the MFMA kernels hold two 64 KB K-slots in LDS
-      HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+      HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_recompute_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_RECOMPUTE));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
@@ -1248,7 +1273,7 @@ extern "C" int sce_forward(const sce_args* a) {
   const int grid = 8 * nsplit * ((RT + 7) / 8);
   {
     KernelTimer tm(SCE_K_FWD, st);
-    fwd_kernel<<<grid, NTHREADS, SMEM_BYTES, st>>>(p);
+    fwd_kernel<<<grid, NTHREADS, SMEM_FWD, st>>>(p);
   }
   KernelTimer tm_red(SCE_K_FWD_REDUCE, st);
   float* s_lse = (float*)(sv + S.off_lse);

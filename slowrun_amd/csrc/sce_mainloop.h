@@ -39,9 +39,8 @@ struct TileLoads {
   uint32_t vo[16];    // per-lane byte offset of load n; even n: A, odd n: B
   uint32_t lds[16];   // LDS address of load n in slot 0 (wave-uniform)
   // load n of an operand covers the 8-row chunk (n / 2 + rot) % 8 of the wave's 64 rows
-  __device__ __forceinline__ TileLoads(int64_t lda, int64_t ldb, uint8_t* smem, int rot_a, int rot_b) {
-    const int t = threadIdx.x, lane = t & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  __device__ __forceinline__ TileLoads(int64_t lda, int64_t ldb, uint8_t* smem, int rot_a, int rot_b, int wave) {
+    const int lane = lane_id();
     const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
     // one wave instruction covers 8 rows x 128 B; a wave fills rows [64 w, 64 w + 64) of A and of B
     const int lr = lane >> 3, pc = lane & 7;
@@ -68,8 +67,8 @@ struct TileLoads {
 // main loop that follows with PREFETCHED = true expects exactly these 24 loads to be the wave's newest
 // vector memory operations.
 __device__ __forceinline__ void mfma_prefetch(const uint8_t* __restrict__ Ag, int64_t lda, const uint8_t* __restrict__ Bg,
-                                              int64_t ldb, uint8_t* smem, int rot_a, int rot_b) {
-  const TileLoads ld(lda, ldb, smem, rot_a, rot_b);
+                                              int64_t ldb, uint8_t* smem, int rot_a, int rot_b, int wave) {
+  const TileLoads ld(lda, ldb, smem, rot_a, rot_b, wave);
 #pragma unroll
   for (int n = 0; n < 16; ++n) ld.issue<0>(n, Ag, Bg);
 #pragma unroll
@@ -77,7 +76,7 @@ __device__ __forceinline__ void mfma_prefetch(const uint8_t* __restrict__ Ag, in
 }
 
 // lda, ldb: row strides in bytes, multiples of 16, at most 2^24; KD = K / 128, even, >= 2;
-// rot_a, rot_b in [0, 8), uniform over the workgroup.
+// rot_a, rot_b in [0, 8), uniform over the workgroup; wave: index of the wavefront in the workgroup (scalar).
 struct NoHook { __device__ __forceinline__ void operator()(int) const {} };
 
 // `hook(i)` is called after MFMA i (0..63) of every pair of K blocks: a place for vector ALU work that
@@ -85,10 +84,10 @@ struct NoHook { __device__ __forceinline__ void operator()(int) const {} };
 template <bool PREFETCHED = false, class Hook = NoHook, int KSTEP = BK>
 __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, int64_t lda,
                                               const uint8_t* __restrict__ Bg, int64_t ldb, int KD,
-                                              uint8_t* smem, v16f (&acc)[4][4], int rot_a, int rot_b, Hook&& hook = NoHook()) {
-  const int t = threadIdx.x, lane = t & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(t >> 6), wa = wave >> 1, wb = wave & 1;
-  const TileLoads ld(lda, ldb, smem, rot_a, rot_b);
+                                              uint8_t* smem, v16f (&acc)[4][4], int rot_a, int rot_b, int wave, Hook&& hook = NoHook()) {
+  const int lane = lane_id();
+  const int wa = wave >> 1, wb = wave & 1;
+  const TileLoads ld(lda, ldb, smem, rot_a, rot_b, wave);
   // fragments: lane reads row l%32 of a 32-row block, 32 bytes of K at (l/32)*32 within the sub-step
   const int r = lane & 31, h = lane >> 5;
   const int sw = (r & 7) ^ ((r >> 3) & 1);
