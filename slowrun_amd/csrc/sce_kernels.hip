@@ -77,6 +77,13 @@ template <> struct Elem<bf16_t> {
 // row, so that 32 consecutive tiles form a 4 x 8 block sharing A-side and B-side rows) and every
 // XCD takes one contiguous eighth of that order: equal shares, and neighbours in the order run on
 // the same L2 at about the same time.
+__device__ __forceinline__ void tile_from_index(int idx, int RT, int CT, int& rt, int& ct) {
+  const int gsz = 8 * RT;                 // tiles in a full group of 8 columns
+  const int g = idx / gsz, rem = idx - g * gsz;
+  const int gw = (CT - g * 8) < 8 ? (CT - g * 8) : 8;
+  rt = rem / gw;
+  ct = g * 8 + (rem - rt * gw);
+}
 __device__ __forceinline__ bool map_tile(int bid, int RT, int CT, int& rt, int& ct) {
   const int T = RT * CT;
   const int per = (T + 7) >> 3;
@@ -84,11 +91,7 @@ __device__ __forceinline__ bool map_tile(int bid, int RT, int CT, int& rt, int& 
   if (local >= per) return false;
   const int idx = xcd * per + local;
   if (idx >= T) return false;
-  const int gsz = 8 * RT;                 // tiles in a full group of 8 columns
-  const int g = idx / gsz, rem = idx - g * gsz;
-  const int gw = (CT - g * 8) < 8 ? (CT - g * 8) : 8;
-  rt = rem / gw;
-  ct = g * 8 + (rem - rt * gw);
+  tile_from_index(idx, RT, CT, rt, ct);
   return true;
 }
 static inline int map_tile_grid(int RT, int CT) { return 8 * ((RT * CT + 7) / 8); }

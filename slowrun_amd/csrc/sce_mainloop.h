@@ -64,15 +64,22 @@ struct TileLoads {
 
 // Puts K block 0 and the first half of the loads of K block 1 of a tile in flight (24 loads per wave).
 // Both LDS slots must be free: every wave is past the closing barrier of the previous main loop.  A
-// main loop that follows with PREFETCHED = true expects exactly these 24 loads to be the wave's newest
-// vector memory operations.
+// main loop that follows with PREFETCHED = true expects these 24 loads to be the wave's newest
+// vector memory loads, in this order (stores issued in between do not disturb the count it waits for:
+// loads complete in order, so fewer than 9 operations outstanding means block 0 has landed).
+// PARTS: 1 = block 0 only (slot 0), 2 = the 8 loads of block 1 only (slot 1), 3 = both.
+template <int PARTS = 3>
 __device__ __forceinline__ void mfma_prefetch(const uint8_t* __restrict__ Ag, int64_t lda, const uint8_t* __restrict__ Bg,
                                               int64_t ldb, uint8_t* smem, int rot_a, int rot_b, int wave) {
   const TileLoads ld(lda, ldb, smem, rot_a, rot_b, wave);
+  if (PARTS & 1) {
 #pragma unroll
-  for (int n = 0; n < 16; ++n) ld.issue<0>(n, Ag, Bg);
+    for (int n = 0; n < 16; ++n) ld.issue<0>(n, Ag, Bg);
+  }
+  if (PARTS & 2) {
 #pragma unroll
-  for (int n = 0; n < 8; ++n) ld.issue<1>(n, Ag + BK, Bg + BK);
+    for (int n = 0; n < 8; ++n) ld.issue<1>(n, Ag + BK, Bg + BK);
+  }
 }
 
 // lda, ldb: row strides in bytes, multiples of 16, at most 2^24; KD = K / 128, even, >= 2;
