@@ -31,9 +31,9 @@ constexpr int LONG_CHUNK = 1024; // ... which handles at most about this many ro
 // a value derived from threadIdx.x stays live across the main loop, is spilled there, and its reload
 // -- a vector memory load -- makes the next wait count include the tile loads already in flight.
 __device__ __forceinline__ int lane_id() {
-  int l = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-  asm volatile("" : "+v"(l));
-  return l;
+  unsigned all = ~0u;
+  asm volatile("" : "+s"(all));      // a value the optimiser cannot see through: every call computes the index anew
+  return (int)__builtin_amdgcn_mbcnt_hi(all, __builtin_amdgcn_mbcnt_lo(all, 0u));
 }
 
 static inline int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }

@@ -768,9 +768,11 @@ struct DwParams {
   const uint8_t* ghat_t;  // Vp rows, K = Pw, blocked                             B side (rows v)
   float* dwacc;           // [dq][Vp] fp32
   int64_t kbn, kbw, kb0, Vp;   // K blocks per tile of xt and of ghat_t; first K block of xt in this launch; row length of dwacc
-  int RT, CT, KT, accumulate;
+  int RT, CT, KT;
 };
 
+// ACC: add to what the partial holds (only when there are more dW launches than partial buffers)
+template <bool ACC>
 __global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   int rt, ct;
@@ -789,7 +791,7 @@ __global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
       for (int r = 0; r < 16; ++r) {
         const int j = jbase + a * 32 + 8 * (r >> 2) + (r & 3);
         float* dst = p.dwacc + (int64_t)j * p.Vp + v;
-        *dst = p.accumulate ? (*dst + acc[a][b][r]) : acc[a][b][r];
+        *dst = ACC ? (*dst + acc[a][b][r]) : acc[a][b][r];
       }
     }
   }
@@ -1040,7 +1042,8 @@ static int check_device(int dev) {
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
-      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
     }
   }
   if (g_arch_ok[dev] != 1) return fail(SCE_EARCH, "device %d is not gfx950", dev);
@@ -1437,10 +1440,11 @@ extern "C" int sce_backward(const sce_args* a) {
       const int part = launch < nparts ? launch : nparts - 1;
       wp.xt = xt; wp.ghat_t = ghat_t; wp.dwacc = (float*)((uint8_t*)dwacc + (size_t)part * B.part_stride);
       wp.kbn = S.Np / BK; wp.kbw = Pw / BK; wp.kb0 = w0 / BK; wp.Vp = S.Vp;
-      wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(gathered / BK); wp.accumulate = launch >= nparts ? 1 : 0;
+      wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(gathered / BK);
       {
         KernelTimer tm(SCE_K_DW, st);
-        bwd_dw_kernel<<<map_tile_grid(CTd, CTv), NTHREADS, SMEM_BYTES, st>>>(wp);
+        if (launch >= nparts) bwd_dw_kernel<true><<<map_tile_grid(CTd, CTv), NTHREADS, SMEM_BYTES, st>>>(wp);
+        else bwd_dw_kernel<false><<<map_tile_grid(CTd, CTv), NTHREADS, SMEM_BYTES, st>>>(wp);
       }
       ++launch;
       w0 = p0 + prow;

@@ -108,13 +108,6 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
     const v8i f = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     if (n < 4) fa[n] = f; else fb[n - 4] = f;
   };
-#pragma unroll
-  for (int a = 0; a < 4; ++a)
-#pragma unroll
-    for (int b = 0; b < 4; ++b)
-#pragma unroll
-      for (int q = 0; q < 16; ++q) acc[a][b][q] = 0.f;
-
   // prologue: K block 0 and half of block 1 in flight, block 0 visible, fragments of sub-step 0 in registers
   if (!PREFETCHED) {
 #pragma unroll
@@ -130,6 +123,12 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
     const int a = i >> 2, b = i & 3;
     acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[cur][a], fb[cur][b], acc[a][b], 0, 0, 0, 0, 0, 0);
   };
+  // the very first MFMA of each accumulator block takes a zero constant instead of the register: nothing clears them
+  auto mm0 = [&](int i) {
+    const int a = i >> 2, b = i & 3;
+    const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[0][a], fb[0][b], zero, 0, 0, 0, 0, 0, 0);
+  };
   // One K block = two sub-steps of 16 MFMAs; register set 0 feeds the first, set 1 the second.  The
   // loop body handles the blocks in pairs (slot 0, then slot 1) so that every LDS address and every
   // load offset is a constant.  While block k (slot s) is consumed:
@@ -142,18 +141,18 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
   // ga / gb point at the first block of the current pair; MORE tells whether a further pair follows.
   const uint8_t* ga = Ag;
   const uint8_t* gb = Bg;
-  auto pair = [&](bool more) {
+  auto pair = [&](bool first, bool more) {
     // ---- block 2p (slot 0)
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      mm(0, i);
+      if (first) mm0(i); else mm(0, i);
       hook(0 + (i & 7));
       ld.issue<1>(8 + i, ga + KSTEP, gb + KSTEP);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 8; i < 16; ++i) {
-      mm(0, i);
+      if (first) mm0(i); else mm(0, i);
       hook(8 + (i & 7));
       rfrag1(0, 1, i - 8, fa[1], fb[1]);
       __builtin_amdgcn_sched_barrier(0);
@@ -208,12 +207,20 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  for (int p = 0; p < (KD >> 1) - 1; ++p) {
-    pair(true);
+  const int P = KD >> 1;
+  if (P == 1) {
+    pair(true, false);
+  } else {
+    pair(true, true);
     ga += 2 * KSTEP;
     gb += 2 * KSTEP;
+    for (int p = 1; p < P - 1; ++p) {
+      pair(false, true);
+      ga += 2 * KSTEP;
+      gb += 2 * KSTEP;
+    }
+    pair(false, false);
   }
-  pair(false);
   // all LDS reads of this tile are complete in every wave before the caller reuses the buffer
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
