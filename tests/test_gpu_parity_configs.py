@@ -1,4 +1,4 @@
-"""GPU parity at the benchmark shapes (BASELINE.json configs 2-5 in full, config 1
+"""GPU parity at the benchmark shapes (the four fp8 configurations in full, the fp32 one
 with amax scales), HIP path vs the oracle evaluated row-chunked with stock torch on
 the same device and the same bf16 inputs.  Tolerances: parity_util."""
 import pytest
