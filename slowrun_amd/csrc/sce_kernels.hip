@@ -564,22 +564,21 @@ struct RecomputeParams {
   const uint8_t* xq;     // [Np][dp], already offset to the panel's first row
   const uint8_t* wqt;    // [Vp][dp]
   const float* crow;     // offset to the panel's first row
-  uint8_t* ghat;         // [P][Vp]
   uint8_t* ghat_t;       // Vp rows, K = Pw, blocked
-  int64_t dp, ldx, ldv;        // K extent; row strides of xq / wqt and of ghat
+  int64_t dp, ldx;             // K extent and row stride of xq / wqt
   int64_t kbw, kb0;            // ghat_t (blocked): K blocks per tile, K block of this panel's first row
   int RT, CT, V;
   float k1, c2;          // as in FwdParams
 };
 
-// Recompute a 256 x 256 logit tile and leave G = 256 (1 - t^2) e^{z - zmax_row} in e4m3, once
-// row-major (operand of dX) and once transposed (operand of dW).  Both copies are assembled in LDS
-// (free once the main loop is done) and leave the chip as fully coalesced 16-byte stores.  The
-// transposed copy is formed in registers first: the four lanes of a quad hold four consecutive
-// rows of the same four columns, and two quad-permute + byte-permute steps turn that 4 x 4 byte
-// block around.
+// Recompute a 256 x 256 logit tile and leave G = 256 (1 - t^2) e^{z - zmax_row} in e4m3, transposed and tile by
+// tile ([v tile][K block of 128 rows i][256 v][128 i]): the operand layout of dW, which dX reads as well (its main
+// loop forms the fragments of G with the transposing LDS read).  The tile is assembled in LDS (free once the main
+// loop is done) and leaves the chip as 64 KB of consecutive 16-byte stores.  The transposition happens in registers:
+// the four lanes of a quad hold four consecutive rows of the same four columns, and two quad-permute + byte-permute
+// steps turn that 4 x 4 byte block around.
 constexpr int STG_PITCH = 272;                               // 256 + 16: 16-byte aligned, rows shifted by 4 banks
-constexpr int SMEM_RECOMPUTE = 2 * 256 * STG_PITCH;          // 139264 B >= the main loop's 131072 B
+constexpr int SMEM_RECOMPUTE = SMEM_BYTES;                   // the main loop's two K slots; the staging tile (69632 B) reuses them
 
 __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -592,8 +591,7 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
   mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave));
-  uint8_t* T = smem;                         // [256 rows i][STG_PITCH]: columns v contiguous
-  uint8_t* TT = smem + 256 * STG_PITCH;      // [256 columns v][STG_PITCH]: rows i contiguous
+  uint8_t* TT = smem;                        // [256 columns v][STG_PITCH]: rows i contiguous
   const int vloc0 = wa * 128 + 4 * (lane >> 5);
   const bool edge = ct * 256 + 256 > p.V;
   const int vlim = p.V - ct * 256;           // columns >= vlim of this tile do not exist
@@ -627,7 +625,6 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
             for (int m = 0; m < 4; ++m) gg[4 * q + m] = (vloc + m >= vlim) ? 0.f : gg[4 * q + m];
           }
           const uint32_t w = cvt4_e4m3(gg[4 * q], gg[4 * q + 1], gg[4 * q + 2], gg[4 * q + 3]);
-          *reinterpret_cast<uint32_t*>(T + iloc * STG_PITCH + vloc) = w;
           // 4 x 4 byte transpose inside the quad: lane k ends up with column vloc + k, rows (iloc & ~3) .. +3
           const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xB1, 0xF, 0xF, false);    // lane ^ 1
           const uint32_t x = __builtin_amdgcn_perm(p1, w, sel1);
@@ -640,26 +637,25 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   };
   if (edge) form_g(std::true_type{}); else form_g(std::false_type{});
   __syncthreads();
-  uint8_t* grow = p.ghat + (int64_t)rt * 256 * p.ldv + (int64_t)ct * 256;
   uint8_t* gcol = p.ghat_t + ((int64_t)ct * p.kbw + p.kb0 + 2 * rt) * BLOCKED_KSTEP;   // two K blocks of 256 rows x 128 B
 #pragma unroll
   for (int n = 0; n < 16; ++n) {
     const int cidx = t + 256 * n, row = cidx >> 4, col = (cidx & 15) * 16;
-    *reinterpret_cast<v4i*>(grow + (int64_t)row * p.ldv + col) = *reinterpret_cast<const v4i*>(T + row * STG_PITCH + col);
     *reinterpret_cast<v4i*>(gcol + (col >> 7) * BLOCKED_KSTEP + row * BK + (col & 127)) = *reinterpret_cast<const v4i*>(TT + row * STG_PITCH + col);
   }
 }
 
 struct DxParams {
   const uint8_t* wq;      // [dq][Vp]   A side (rows j)
-  const uint8_t* ghat;    // [P][Vp]    B side (rows i of the panel)
+  const uint8_t* ghat_t;  // G^T, blocked; already at the K block of the panel's first row    B side (rows i of the panel)
   const uint8_t* wqt;     // [Vp][dp]   for the one-hot gather
   const float* rho;       // offset to the panel
   const float* hcoef;     // [n_predict][Np], offset to the panel
   const int64_t* targets; // offset to the panel
   void* dx;               // offset to the panel's first row
   float* part;            // [ksplit][RT * 256][dq] fp32 partial sums (ksplit > 1 only)
-  int64_t dx_ld, Vp, ldv, ldx, Np, dq;   // Vp: K extent; ldv: row stride of wq / ghat; ldx: of wqt
+  int64_t dx_ld, Vp, ldv, ldx, Np, dq;   // Vp: K extent; ldv: row stride of wq; ldx: of wqt
+  int64_t kbw;                           // K blocks (of 128 rows i) per v tile of ghat_t
   int RT, CT, rows, d, V;  // rows: valid rows in this panel
   int n_predict, rows_left; // rows_left: N - (first row of the panel), bounds the target look-ahead
   int ksplit;              // the K loop (V) is cut into this many parts, one workgroup each
@@ -718,7 +714,11 @@ __global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p) {
   }
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
-  mfma_mainloop(p.wq + (int64_t)ct * 256 * p.ldv + k0, p.ldv, p.ghat + (int64_t)rt * 256 * p.ldv + k0, p.ldv, KD, smem, acc, 2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave));
+  // B = G^T: K (v) is the slow index there.  The 128 v rows of a K block are half a v tile; the 256 panel rows of this
+  // tile are the two 128-byte pieces of i blocks 2 rt and 2 rt + 1 (BLOCKED_KSTEP apart).
+  const int64_t bpair = p.kbw * BLOCKED_KSTEP;                     // from one v tile (two K blocks) to the next
+  mfma_mainloop<false, NoHook, BK, true>(p.wq + (int64_t)ct * 256 * p.ldv + k0, p.ldv, p.ghat_t + 2 * (int64_t)rt * BLOCKED_KSTEP + (k0 / (2 * BK)) * bpair,
+                                         BLOCKED_KSTEP, KD, smem, acc, 2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave), NoHook(), 128 * BK, bpair);
   const int jbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
   T* dx = reinterpret_cast<T*>(p.dx);
 #pragma unroll
@@ -1092,7 +1092,6 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int npa
   B.off_sorttmp = take(B.sorttmp_bytes);
   B.off_dxpart = take(DX_PART_BYTES);
   B.fixed = o;
-  B.off_ghat = take((size_t)P * S.ldv);
   B.off_ghat_t = take((size_t)S.Vp * Pw);
   B.part_stride = ((size_t)S.dq * S.Vp * 4 + 255) / 256 * 256;
   B.off_dwacc = take(B.part_stride * (size_t)nparts);     // fp32 dW partials, one per dW launch
@@ -1314,17 +1313,17 @@ extern "C" int sce_backward(const sce_args* a) {
   const BwdLayout Bmin = bwd_layout(S, 256, 256, 1, K);
   if (a->workspace_bytes < Bmin.total) return fail(SCE_EINVAL, "backward workspace too small: %zu < %zu", a->workspace_bytes, Bmin.total);
   // panel sizes from what the caller gave: P rows per recompute/dX panel, Pw = m * P rows per dW launch
-  // bytes left for the two e4m3 copies of dlogits: P rows of ldv bytes and Vp rows of Pw bytes
+  // bytes left for the e4m3 dlogits: Vp rows of Pw bytes
   const int64_t room = (int64_t)(a->workspace_bytes - Bmin.fixed - Bmin.part_stride);
   int64_t P = default_panel(S);
   if (a->panel_rows > 0) {
     if (a->panel_rows % 256) return fail(SCE_EINVAL, "panel_rows must be a multiple of 256");
     P = a->panel_rows < S.Np ? a->panel_rows : S.Np;
   }
-  if (P * (S.ldv + S.Vp) > room) P = room / (S.ldv + S.Vp) / 256 * 256;
+  if (P * S.Vp > room) P = room / S.Vp / 256 * 256;
   if (P < 256) P = 256;                                  // Bmin fits, as checked above
   int64_t Pw = default_dw_panel(S, P);
-  if (P * S.ldv + Pw * S.Vp > room) Pw = (room - P * S.ldv) / S.Vp / P * P;
+  if (Pw * S.Vp > room) Pw = room / S.Vp / P * P;
   if (Pw < P) Pw = P;
   int nparts = dw_launches(S, Pw);
   // the estimate above ignores the 256-byte alignment of each region: settle on a layout that fits
@@ -1363,7 +1362,6 @@ extern "C" int sce_backward(const sce_args* a) {
   int32_t* segoff = (int32_t*)(ws + B.off_segoff);
   int32_t* longlist = (int32_t*)(ws + B.off_longlist);
   float* longsum = (float*)(ws + B.off_longsum);
-  uint8_t* ghat = ws + B.off_ghat;
   uint8_t* ghat_t = ws + B.off_ghat_t;
 
   const int nblk = (int)(S.Np / 256);
@@ -1396,15 +1394,15 @@ extern "C" int sce_backward(const sce_args* a) {
     const int64_t prow = (S.Np - p0 < P) ? (S.Np - p0) : P;     // multiple of 256
     const int RTp = (int)(prow / 256);
     RecomputeParams rp;
-    rp.xq = xq + p0 * S.ldx; rp.wqt = wqt; rp.crow = crow + p0; rp.ghat = ghat; rp.ghat_t = ghat_t;
-    rp.dp = S.dp; rp.ldx = S.ldx; rp.ldv = S.ldv; rp.kbw = Pw / BK; rp.kb0 = (p0 - w0) / BK; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2;
+    rp.xq = xq + p0 * S.ldx; rp.wqt = wqt; rp.crow = crow + p0; rp.ghat_t = ghat_t;
+    rp.dp = S.dp; rp.ldx = S.ldx; rp.kbw = Pw / BK; rp.kb0 = (p0 - w0) / BK; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2;
     {
       KernelTimer tm(SCE_K_RECOMPUTE, st);
       bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_RECOMPUTE, st>>>(rp);
     }
 
     DxParams dp_;
-    dp_.wq = wq; dp_.ghat = ghat; dp_.wqt = wqt; dp_.rho = rho + p0; dp_.hcoef = hcoef + p0; dp_.targets = a->targets + p0;
+    dp_.wq = wq; dp_.ghat_t = ghat_t + ((p0 - w0) / BK) * BLOCKED_KSTEP; dp_.kbw = Pw / BK; dp_.wqt = wqt; dp_.rho = rho + p0; dp_.hcoef = hcoef + p0; dp_.targets = a->targets + p0;
     dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.ldv = S.ldv; dp_.ldx = S.ldx; dp_.Np = S.Np; dp_.dq = S.dq; dp_.RT = RTp; dp_.CT = CTd;
     dp_.n_predict = K; dp_.rows_left = (int)(N - p0 > 0 ? N - p0 : 0);
     dp_.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); dp_.d = (int)d; dp_.V = (int)Vl; dp_.w_s = a->w_s;

@@ -35,6 +35,13 @@ __device__ __forceinline__ void lds_direct_16(uint32_t lds_addr, uint32_t voff, 
 }
 
 // Global -> LDS loads of one tile: per wave, 16 instructions per K block (8 for A, 8 for B).
+//
+// TRB = false: both operands are K-contiguous in memory (rows lda / ldb bytes apart) and in LDS.
+// TRB = true : the B operand comes from an array that has the B rows (N) contiguous and K as the slow index,
+//              stored in 128-byte pieces: for each of the 128 K rows of a K block, 128 bytes of N in one piece
+//              and the next 128 bytes in a second piece `ldb` bytes further on.  In LDS the K block is
+//              [2 pieces][128 K rows][128 B]; fragments are formed with the transposing LDS read (see below).
+template <bool TRB = false>
 struct TileLoads {
   uint32_t vo[16];    // per-lane byte offset of load n; even n: A, odd n: B
   uint32_t lds[16];   // LDS address of load n in slot 0 (wave-uniform)
@@ -50,7 +57,8 @@ struct TileLoads {
       const int rowa = wave * 64 + ca * 8 + lr, rowb = wave * 64 + cb * 8 + lr;
       const int swa = (rowa & 7) ^ ((rowa >> 3) & 1), swb = (rowb & 7) ^ ((rowb >> 3) & 1);
       vo[2 * n] = (uint32_t)(rowa * lda + ((pc ^ swa) * 16));
-      vo[2 * n + 1] = (uint32_t)(rowb * ldb + ((pc ^ swb) * 16));
+      if (TRB) vo[2 * n + 1] = (uint32_t)((rowb >> 7) * ldb + (rowb & 127) * BK + ((pc ^ (rowb & 7)) * 16));
+      else vo[2 * n + 1] = (uint32_t)(rowb * ldb + ((pc ^ swb) * 16));
       lds[2 * n] = lds0 + wave * 64 * BK + ca * 8 * BK;
       lds[2 * n + 1] = lds0 + TM * BK + wave * 64 * BK + cb * 8 * BK;
     }
@@ -71,7 +79,7 @@ struct TileLoads {
 template <int PARTS = 3>
 __device__ __forceinline__ void mfma_prefetch(const uint8_t* __restrict__ Ag, int64_t lda, const uint8_t* __restrict__ Bg,
                                               int64_t ldb, uint8_t* smem, int rot_a, int rot_b, int wave) {
-  const TileLoads ld(lda, ldb, smem, rot_a, rot_b, wave);
+  const TileLoads<false> ld(lda, ldb, smem, rot_a, rot_b, wave);
   if (PARTS & 1) {
 #pragma unroll
     for (int n = 0; n < 16; ++n) ld.issue<0>(n, Ag, Bg);
@@ -88,19 +96,41 @@ struct NoHook { __device__ __forceinline__ void operator()(int) const {} };
 
 // `hook(i)` is called after MFMA i (0..63) of every pair of K blocks: a place for vector ALU work that
 // does not depend on the accumulators (it runs while the matrix pipe is busy).
-template <bool PREFETCHED = false, class Hook = NoHook, int KSTEP = BK>
+// TRB (see TileLoads): the K blocks of B lie bk1 bytes apart within a pair and bk2 bytes from pair to pair
+// (for TRB = false they are KSTEP and 2 KSTEP and the two arguments are ignored).
+template <bool PREFETCHED = false, class Hook = NoHook, int KSTEP = BK, bool TRB = false>
 __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, int64_t lda,
                                               const uint8_t* __restrict__ Bg, int64_t ldb, int KD,
-                                              uint8_t* smem, v16f (&acc)[4][4], int rot_a, int rot_b, int wave, Hook&& hook = NoHook()) {
+                                              uint8_t* smem, v16f (&acc)[4][4], int rot_a, int rot_b, int wave, Hook&& hook = NoHook(),
+                                              int64_t bk1_arg = 0, int64_t bk2_arg = 0) {
   const int lane = lane_id();
   const int wa = wave >> 1, wb = wave & 1;
-  const TileLoads ld(lda, ldb, smem, rot_a, rot_b, wave);
+  const int64_t bk1 = TRB ? bk1_arg : (int64_t)KSTEP, bk2 = TRB ? bk2_arg : (int64_t)(2 * KSTEP);
+  const TileLoads<TRB> ld(lda, ldb, smem, rot_a, rot_b, wave);
   // fragments: lane reads row l%32 of a 32-row block, 32 bytes of K at (l/32)*32 within the sub-step
   const int r = lane & 31, h = lane >> 5;
   const int sw = (r & 7) ^ ((r >> 3) & 1);
   const int abase = wa * 128 * BK + r * BK, bbase = TM * BK + wb * 128 * BK + r * BK;
   // fragment n (0-3: A, 4-7: B) of the sub-step with K half `half` in LDS slot `slot`
   auto rfrag1 = [&](int slot, int half, int n, v8i (&fa)[4], v8i (&fb)[4]) {
+    if (TRB && n >= 4) {
+      // B block b = n - 4 from the [K row][N] layout.  ds_read_b64_tr_b8 works on groups of 16 lanes: lane j of a
+      // group points at 8 bytes -- here the half (j & 1) of the 16-byte N chunk of K row (j >> 1) -- and gets byte j of
+      // each of the group's 8 rows: 8 consecutive K values of its own N.  Four reads give the lane its 32 K values.
+      // Group g = lane / 16 holds N chunk 2 b + (g & 1) and K half g / 2; the chunks of a row are XOR-swizzled by
+      // (K row & 7) = j >> 1 (the loader stores them so).
+      const int b = n - 4, g = lane >> 4, j = lane & 15;
+      const uint8_t* s = smem + slot * SLOT_BYTES + TM * BK + wb * 128 * BK + (64 * half + 32 * (g >> 1) + (j >> 1)) * BK +
+                         (((2 * b + (g & 1)) ^ (j >> 1)) << 4) + 8 * (j & 1);
+      v8i f;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const v2i r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)(s + c * 8 * BK));
+        f[2 * c] = r2[0]; f[2 * c + 1] = r2[1];
+      }
+      fb[b] = f;
+      return;
+    }
     const int c0 = ((4 * half + 2 * h) ^ sw) * 16;
     const uint8_t* s = smem + slot * SLOT_BYTES + ((n < 4) ? abase + n * 32 * BK : bbase + (n - 4) * 32 * BK);
     const v4i lo = *reinterpret_cast<const v4i*>(s + c0);
@@ -111,9 +141,9 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
   // prologue: K block 0 and half of block 1 in flight, block 0 visible, fragments of sub-step 0 in registers
   if (!PREFETCHED) {
 #pragma unroll
-    for (int n = 0; n < 16; ++n) ld.issue<0>(n, Ag, Bg);
+    for (int n = 0; n < 16; ++n) ld.template issue<0>(n, Ag, Bg);
 #pragma unroll
-    for (int n = 0; n < 8; ++n) ld.issue<1>(n, Ag + KSTEP, Bg + KSTEP);
+    for (int n = 0; n < 8; ++n) ld.template issue<1>(n, Ag + KSTEP, Bg + bk1);
   }
   asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
   v8i fa[2][4], fb[2][4];
@@ -147,7 +177,7 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
     for (int i = 0; i < 8; ++i) {
       if (first) mm0(i); else mm(0, i);
       hook(0 + (i & 7));
-      ld.issue<1>(8 + i, ga + KSTEP, gb + KSTEP);
+      ld.template issue<1>(8 + i, ga + KSTEP, gb + bk1);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
@@ -170,7 +200,7 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
       mm(1, i);
       hook(24 + (i & 7));
       rfrag1(1, 0, i - 8, fa[0], fb[0]);
-      if (more) ld.issue<0>(i - 8, ga + 2 * KSTEP, gb + 2 * KSTEP);
+      if (more) ld.template issue<0>(i - 8, ga + 2 * KSTEP, gb + bk2);
       __builtin_amdgcn_sched_barrier(0);
     }
     // ---- block 2p + 1 (slot 1)
@@ -178,7 +208,7 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
     for (int i = 0; i < 8; ++i) {
       mm(0, i);
       hook(32 + (i & 7));
-      if (more) ld.issue<0>(8 + i, ga + 2 * KSTEP, gb + 2 * KSTEP);
+      if (more) ld.template issue<0>(8 + i, ga + 2 * KSTEP, gb + bk2);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
@@ -202,7 +232,7 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
       hook(56 + (i & 7));
       if (more) {
         rfrag1(0, 0, i - 8, fa[0], fb[0]);
-        ld.issue<1>(i - 8, ga + 3 * KSTEP, gb + 3 * KSTEP);
+        ld.template issue<1>(i - 8, ga + 3 * KSTEP, gb + bk2 + bk1);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -213,11 +243,11 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
   } else {
     pair(true, true);
     ga += 2 * KSTEP;
-    gb += 2 * KSTEP;
+    gb += bk2;
     for (int p = 1; p < P - 1; ++p) {
       pair(false, true);
       ga += 2 * KSTEP;
-      gb += 2 * KSTEP;
+      gb += bk2;
     }
     pair(false, false);
   }
