@@ -271,3 +271,47 @@ def test_dx_panel_with_few_tiles_is_k_split():
     ours = pu.run_ours(inp, "none", x_dtype=torch.float32)
     ref = pu.run_oracle(inp, ours, "none")
     print(pu.check_parity(ours, ref, "none"))
+
+
+def test_captured_in_a_hip_graph_and_replayed():
+    """Every launch of forward and backward goes to the caller's stream and nothing synchronises, so the
+    pair can be captured once and replayed on new contents of the same buffers (tiny/train.py:1254 compiles
+    the model; a trainer that captures its step needs this).  Each replay is compared bit for bit with
+    the same calls issued directly."""
+    from slowrun_amd import cuda_kernels as ck
+    inp = _small("limited_2p7b", 1500, 256, 2100)
+    N, d, V = inp.shape
+    x = inp.x.cuda().bfloat16()
+    w = inp.w.cuda().bfloat16()
+    y = inp.targets.cuda()
+    go = torch.ones((), device="cuda")
+
+    def step():
+        loss, saved, _lse, _am, _nv = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, "mean")
+        dx, dw = ck.ce_backward(saved, y, go, N, d, V, inp.x_s, inp.w_s, inp.cap, 1.0, "mean", torch.bfloat16, torch.bfloat16)
+        return loss, dx, dw
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    gen = torch.Generator().manual_seed(21)
+    for trial in range(4):
+        amax = float(inp.x.abs().max())            # the scale x_s was taken from this: stay inside e4m3's range
+        x.copy_((inp.x * (1.0 - 0.1 * trial) + 0.05 * torch.randn(inp.x.shape, generator=gen)).clamp(-amax, amax).bfloat16())
+        y.copy_(torch.randint(0, V, (N,), generator=gen))
+        if trial == 2:
+            y[::7] = -1
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        want = step()
+        torch.cuda.synchronize()
+        for g, e, name in zip(got, want, ("loss", "dx", "dw")):
+            assert torch.equal(g, e), f"replay {trial}: {name} differs from the direct calls"
+        assert torch.isfinite(got[0])
