@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SCE_VERSION 2
+#define SCE_VERSION 3
 
 enum { SCE_F32 = 0, SCE_BF16 = 1 };               /* element types of X, W, dX, dW          */
 enum { SCE_REDUCE_NONE = 0, SCE_REDUCE_MEAN = 1 }; /* F.cross_entropy(reduction=...)         */
@@ -103,6 +103,11 @@ typedef struct sce_args {
                                 forward fills it unless wcache_valid, backward reads it          */
   size_t wcache_bytes;
   int32_t wcache_valid;      /* non-zero: wcache already holds e4m3(W / w_s) of this very W      */
+  int32_t norm;              /* non-zero: x is the hidden state h before the trunk's last operation,
+                                x = F.rms_norm(h, (d,), eps = norm_eps) (tiny/train.py:397-398,734): forward
+                                normalises inside the quantiser, backward needs x again and returns the
+                                gradient with respect to h in dx                                  */
+  float norm_eps;
   int32_t pad5;
 } sce_args;
 

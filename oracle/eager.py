@@ -98,6 +98,37 @@ def softcapped_ce(x, w, targets, x_s=None, w_s=None, cap=15.0, reduction="mean",
     return dict(loss=loss, losses=losses, lse=lse, argmax=argmax, dx=dx, dw=dw, n_valid=n_valid)
 
 
+def rms_norm(h, eps=None):
+    """F.rms_norm(h, (d,)) without weight (tiny/train.py:397-398) in fp32 with one rounding to h's dtype, which
+    is what torch computes for bf16 input; eps=None is torch's default, the machine epsilon of the type it
+    computes in (float32 for bf16 and fp32 input).  Returns (normalised rows in h's dtype, rstd (N, 1) in fp32)."""
+    eps = torch.finfo(torch.float64 if h.dtype == torch.float64 else torch.float32).eps if eps is None else eps
+    hf = h.float()
+    rstd = torch.rsqrt(hf.pow(2).mean(dim=-1, keepdim=True) + eps)
+    return (hf * rstd).to(h.dtype), rstd
+
+
+def rms_norm_backward(h, rstd, g):
+    """Gradient of rms_norm with respect to h for an upstream gradient g of the normalised rows:
+    dh = rstd * (g - xhat * mean(g * xhat)), xhat = h * rstd."""
+    xhat = h.float() * rstd
+    gf = g.float()
+    return rstd * (gf - xhat * (gf * xhat).mean(dim=-1, keepdim=True))
+
+
+def norm_softcapped_ce(h, w, targets, x_s, w_s, cap=15.0, reduction="mean", eps=None, **kw):
+    """The trunk's final norm followed by the head (tiny/train.py:734 then :682-696): softcapped_ce on
+    rms_norm(h), with the head's gradient (rounded to h's dtype, as the unfused path stores it) taken back
+    through the norm.  Returns softcapped_ce's dict with dx replaced by the gradient with respect to h."""
+    x, rstd = rms_norm(h, eps)
+    res = softcapped_ce(x, w, targets, x_s, w_s, cap, reduction, **kw)
+    if res["dx"] is not None:
+        res["dx_normalised"] = res["dx"]
+        res["dx"] = rms_norm_backward(h, rstd, res["dx"].to(h.dtype))
+    res["x"] = x
+    return res
+
+
 def softcapped_ce_mtp(x, w, targets, mtp_weights, x_s=None, w_s=None, cap=15.0,
                       grad_output=None, want_grads=True, row_chunk=2048, dtype=torch.float32):
     """Multi-token-prediction variant, reduction 'none' (tiny/cuda_kernels.py:226-240).

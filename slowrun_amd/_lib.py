@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(HERE, "libslowrun_ce.so")
 
 SCE_F32, SCE_BF16 = 0, 1
 SCE_REDUCE_NONE, SCE_REDUCE_MEAN = 0, 1
-SCE_VERSION = 2
+SCE_VERSION = 3
 
 EXPORTS = ("sce_version", "sce_last_error", "sce_sizes_for", "sce_quantize_e4m3", "sce_transpose_bytes",
            "sce_forward", "sce_backward", "sce_timing_enable", "sce_timing_read")
@@ -45,7 +45,7 @@ class SceArgs(C.Structure):
         ("dw", C.c_void_p), ("dw_dtype", C.c_int32), ("pad4", C.c_int32), ("dw_ld", C.c_int64),
         ("panel_rows", C.c_int64),
         ("vocab_limit", C.c_int64), ("wcache", C.c_void_p), ("wcache_bytes", C.c_size_t),
-        ("wcache_valid", C.c_int32), ("pad5", C.c_int32),
+        ("wcache_valid", C.c_int32), ("norm", C.c_int32), ("norm_eps", C.c_float), ("pad5", C.c_int32),
     ]
 
 

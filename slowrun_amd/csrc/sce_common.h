@@ -47,7 +47,7 @@ static inline int64_t row_stride(int64_t k) { return k + 128; }
 struct SavedLayout {
   int64_t ldx, ldv;                  // row strides in bytes of the [..][dp] and of the [..][Vp] e4m3 arrays
   int64_t N, d, V, Np, dp, dq, Vp;   // all padded sizes are multiples of 256 (every K loop runs over an even number of 128-byte blocks); dp = dq
-  size_t off_hdr, off_xq, off_lse, off_umax, off_zy, x_total;
+  size_t off_hdr, off_xq, off_lse, off_umax, off_zy, off_rstd, x_total;
   size_t rel_wqt, rel_wq, w_total;   // relative to the start of the W region
   size_t total;                      // x_total + w_total
 };
@@ -65,6 +65,7 @@ static inline SavedLayout saved_layout(int64_t N, int64_t d, int64_t V, int n_pr
   L.off_lse = take((size_t)L.Np * 4);
   L.off_umax = take((size_t)L.Np * 4);
   L.off_zy = take((size_t)L.Np * 4 * n_predict);
+  L.off_rstd = take((size_t)L.Np * 4);         // 1 / rms of each row when the final norm is part of the call
   L.x_total = o;
   o = 0;
   L.rel_wqt = take((size_t)L.Vp * L.ldx);      // W_q^T [Vp][dp], row stride ldx

@@ -147,6 +147,129 @@ __global__ __launch_bounds__(256) void quantize_pad_kernel(const T* __restrict__
   }
 }
 
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// The trunk's last operation fused into the quantiser (F.rms_norm without weight, tiny/train.py:397-398,734):
+// dst row = e4m3(round_T(h * rstd) / scale) with rstd = 1 / sqrt(mean(h^2) + eps), the normalised row rounded to
+// the input's type as the unfused path has it in memory.  One wave per row; rstd is kept for backward.
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_quantize_kernel(const T* __restrict__ src, int64_t ld, int64_t rows,
+                                                              int64_t cols, float eps, uint8_t* __restrict__ dst,
+                                                              int64_t rows_p, int64_t cols_p, int64_t dst_ld, float scale,
+                                                              float* __restrict__ rstd_out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows_p) return;
+  const int64_t chunks = cols_p / 16;
+  if (r >= rows) {
+    for (int64_t c = lane; c < chunks; c += 64) *reinterpret_cast<v4i*>(dst + r * dst_ld + c * 16) = (v4i){0, 0, 0, 0};
+    if (lane == 0) rstd_out[r] = 0.f;
+    return;
+  }
+  const T* row = src + r * ld;
+  float ss = 0.f;
+  for (int64_t c = lane; c * 16 < cols; c += 64) {
+    float v[16];
+    load16_scaled<T>(row + c * 16, cols - c * 16, 1.0f, v);      // a division by 1 is exact: the values themselves
+#pragma unroll
+    for (int m = 0; m < 16; ++m) ss = fmaf(v[m], v[m], ss);
+  }
+  ss = wave_sum(ss);
+  const float rstd = 1.0f / sqrtf(ss / (float)cols + eps);
+  if (lane == 0) rstd_out[r] = rstd;
+  for (int64_t c = lane; c < chunks; c += 64) {
+    uint32_t out[4] = {0, 0, 0, 0};
+    if (c * 16 < cols) {
+      float v[16];
+      load16_scaled<T>(row + c * 16, cols - c * 16, 1.0f, v);
+#pragma unroll
+      for (int m = 0; m < 16; ++m) {
+        float y = v[m] * rstd;
+        if constexpr (sizeof(T) == 2) y = round_to_bf16(y);
+        v[m] = Elem<T>::div_round(y, scale);
+      }
+#pragma unroll
+      for (int m = 0; m < 4; ++m) out[m] = cvt4_e4m3(v[4 * m], v[4 * m + 1], v[4 * m + 2], v[4 * m + 3]);
+    }
+    *reinterpret_cast<v4i*>(dst + r * dst_ld + c * 16) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
+  }
+}
+
+// 8 consecutive elements as floats, and back; `vec`: the run is 16-byte (bf16) / 32-byte (fp32) aligned.
+template <typename T>
+__device__ __forceinline__ void load8(const T* __restrict__ p, bool vec, float (&v)[8]) {
+  if (vec) {
+    if constexpr (sizeof(T) == 2) {
+      const v4i r = *reinterpret_cast<const v4i*>(p);
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        v[2 * m] = __uint_as_float((uint32_t)r[m] << 16);
+        v[2 * m + 1] = __uint_as_float((uint32_t)r[m] & 0xffff0000u);
+      }
+    } else {
+      const v4f a = *reinterpret_cast<const v4f*>(p), b = *reinterpret_cast<const v4f*>(p + 4);
+#pragma unroll
+      for (int m = 0; m < 4; ++m) { v[m] = a[m]; v[4 + m] = b[m]; }
+    }
+  } else {
+#pragma unroll
+    for (int m = 0; m < 8; ++m) v[m] = Elem<T>::load(p + m);
+  }
+}
+template <typename T>
+__device__ __forceinline__ void store8(T* __restrict__ p, bool vec, const float (&v)[8]) {
+  if (vec) {
+    if constexpr (sizeof(T) == 2) {
+      v4i r;
+#pragma unroll
+      for (int m = 0; m < 4; ++m) r[m] = (int)((uint32_t)float_to_bf16_bits(v[2 * m]) | ((uint32_t)float_to_bf16_bits(v[2 * m + 1]) << 16));
+      *reinterpret_cast<v4i*>(p) = r;
+    } else {
+      *reinterpret_cast<v4f*>(p) = (v4f){v[0], v[1], v[2], v[3]};
+      *reinterpret_cast<v4f*>(p + 4) = (v4f){v[4], v[5], v[6], v[7]};
+    }
+  } else {
+#pragma unroll
+    for (int m = 0; m < 8; ++m) Elem<T>::store(p + m, v[m]);
+  }
+}
+
+// Backward of that norm, in place on the finished dX: with xhat = h * rstd and g the gradient of the normalised row,
+// dh = rstd * (g - xhat * mean(g * xhat)).  One wave per row; cols is a multiple of 8.
+template <typename TG, typename TH>
+__global__ __launch_bounds__(256) void rmsnorm_backward_kernel(TG* __restrict__ g, int64_t g_ld, const TH* __restrict__ h,
+                                                              int64_t h_ld, const float* __restrict__ rstd_in, int64_t rows,
+                                                              int64_t cols) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const float rstd = rstd_in[r];
+  TG* grow = g + r * g_ld;
+  const TH* hrow = h + r * h_ld;
+  const bool gvec = (((uintptr_t)grow) & (8 * sizeof(TG) - 1)) == 0, hvec = (((uintptr_t)hrow) & (8 * sizeof(TH) - 1)) == 0;
+  float dot = 0.f;
+  for (int64_t c = 8 * lane; c < cols; c += 512) {
+    float gv[8], hv[8];
+    load8<TG>(grow + c, gvec, gv);
+    load8<TH>(hrow + c, hvec, hv);
+#pragma unroll
+    for (int m = 0; m < 8; ++m) dot = fmaf(gv[m], hv[m] * rstd, dot);
+  }
+  dot = wave_sum(dot) / (float)cols;
+  for (int64_t c = 8 * lane; c < cols; c += 512) {
+    float gv[8], hv[8];
+    load8<TG>(grow + c, gvec, gv);
+    load8<TH>(hrow + c, hvec, hv);
+#pragma unroll
+    for (int m = 0; m < 8; ++m) gv[m] = rstd * (gv[m] - hv[m] * rstd * dot);
+    store8<TG>(grow + c, gvec, gv);
+  }
+}
+
 // W (d, V) -> W_q [dq][Vp] (same orientation) and W_q^T [Vp][dp]; 64 x 64 tiles through LDS.
 template <typename T>
 __global__ __launch_bounds__(256) void quantize_w_kernel(const T* __restrict__ w, int64_t ld, int64_t d, int64_t V,
@@ -1257,7 +1380,13 @@ extern "C" int sce_forward(const sce_args* a) {
   {
     KernelTimer tm(SCE_K_QUANT, st);
     const int grid = grid_for((size_t)S.Np * (S.dp / 16), 256);
-    if (a->x_dtype == SCE_F32)
+    float* rstd = (float*)(sv + S.off_rstd);
+    const int ngrid = (int)((S.Np + 3) / 4);
+    if (a->norm && a->x_dtype == SCE_F32)
+      rmsnorm_quantize_kernel<float><<<ngrid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, a->norm_eps, xq, S.Np, S.dp, S.ldx, a->x_s, rstd);
+    else if (a->norm && a->x_dtype == SCE_BF16)
+      rmsnorm_quantize_kernel<bf16_t><<<ngrid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, a->norm_eps, xq, S.Np, S.dp, S.ldx, a->x_s, rstd);
+    else if (a->x_dtype == SCE_F32)
       quantize_pad_kernel<float><<<grid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, S.ldx, a->x_s);
     else if (a->x_dtype == SCE_BF16)
       quantize_pad_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, S.ldx, a->x_s);
@@ -1300,6 +1429,11 @@ extern "C" int sce_backward(const sce_args* a) {
   const int64_t N = a->shape.N, d = a->shape.d, V = a->shape.V;
   if (!a->grad_output) return fail(SCE_EINVAL, "grad_output is NULL");
   if (!a->dx || !a->dw) return fail(SCE_EINVAL, "dx or dw is NULL");
+  if (a->norm) {
+    if (!a->x) return fail(SCE_EINVAL, "norm is set: backward needs x (the hidden state given to forward)");
+    if (a->x_dtype != SCE_F32 && a->x_dtype != SCE_BF16) return fail(SCE_EINVAL, "unsupported x dtype %d", a->x_dtype);
+    if (a->x_ld < d) return fail(SCE_EINVAL, "row strides smaller than the row length");
+  }
   if (a->dx_ld < d || a->dw_ld < V) return fail(SCE_EINVAL, "row strides smaller than the row length");
   if ((a->dx_dtype != SCE_F32 && a->dx_dtype != SCE_BF16) || (a->dw_dtype != SCE_F32 && a->dw_dtype != SCE_BF16))
     return fail(SCE_EINVAL, "unsupported gradient dtype");
@@ -1447,6 +1581,15 @@ extern "C" int sce_backward(const sce_args* a) {
       ++launch;
       w0 = p0 + prow;
     }
+  }
+  if (a->norm) {       // dX so far is the gradient of the normalised rows: take it through the norm, in place
+    const float* rstd = (const float*)(sv + S.off_rstd);
+    const int ngrid = (int)((N + 3) / 4);
+    const bool gf = a->dx_dtype == SCE_F32, hf = a->x_dtype == SCE_F32;
+    if (gf && hf) rmsnorm_backward_kernel<float, float><<<ngrid, 256, 0, st>>>((float*)a->dx, a->dx_ld, (const float*)a->x, a->x_ld, rstd, N, d);
+    else if (gf) rmsnorm_backward_kernel<float, bf16_t><<<ngrid, 256, 0, st>>>((float*)a->dx, a->dx_ld, (const bf16_t*)a->x, a->x_ld, rstd, N, d);
+    else if (hf) rmsnorm_backward_kernel<bf16_t, float><<<ngrid, 256, 0, st>>>((bf16_t*)a->dx, a->dx_ld, (const float*)a->x, a->x_ld, rstd, N, d);
+    else rmsnorm_backward_kernel<bf16_t, bf16_t><<<ngrid, 256, 0, st>>>((bf16_t*)a->dx, a->dx_ld, (const bf16_t*)a->x, a->x_ld, rstd, N, d);
   }
   KernelTimer tm_fin(SCE_K_DW_FINAL, st);
   bwd_dw_long_kernel<<<dim3((unsigned)(NE / LONG_SEG + 1), (unsigned)(S.dq / 256)), 256, 0, st>>>(longlist, segoff, perm, hcoef, xq, S.dp, S.ldx, S.dq, (int)S.Np, longsum);

@@ -115,8 +115,11 @@ class WeightCache:
 
 
 def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_weights=None, vocab_size=None,
-               weight_cache=None):
-    """One call of sce_forward.  Returns (out, saved, lse, argmax, n_valid)."""
+               weight_cache=None, norm_eps=None):
+    """One call of sce_forward.  Returns (out, saved, lse, argmax, n_valid).
+
+    norm_eps: when given, ``x`` is the hidden state before the trunk's final ``F.rms_norm(x, (d,))``
+    (tiny/train.py:397-398,734) and the norm is applied inside the quantiser."""
     _check_inputs(x, w, targets)
     n_predict, mtp_w = _mtp(mtp_weights, x.device)
     if n_predict > 1 and reduction != "none":
@@ -143,6 +146,8 @@ def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_w
     a.saved, a.saved_bytes = saved.data_ptr(), saved.numel()
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
     a.vocab_limit = 0 if vocab_size is None else int(vocab_size)
+    if norm_eps is not None:
+        a.norm, a.norm_eps = 1, float(norm_eps)
     if weight_cache is not None:
         wbuf, valid = weight_cache.prepare(w, w_s, sz.wcache_bytes)
         a.wcache, a.wcache_bytes, a.wcache_valid = wbuf.data_ptr(), wbuf.numel(), int(valid)
@@ -152,8 +157,12 @@ def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_w
 
 
 def ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale, reduction, x_dtype, w_dtype,
-                panel_rows=0, workspace_bytes=None, mtp_weights=None, vocab_size=None, weight_cache=None):
-    """One call of sce_backward.  Returns (dx (N,d) in x_dtype, dw (d,V) in w_dtype)."""
+                panel_rows=0, workspace_bytes=None, mtp_weights=None, vocab_size=None, weight_cache=None,
+                hidden=None, norm_eps=None):
+    """One call of sce_backward.  Returns (dx (N,d) in x_dtype, dw (d,V) in w_dtype).
+
+    hidden, norm_eps: the pre-norm hidden state and eps given to ce_forward(norm_eps=...); dx is then the
+    gradient with respect to that hidden state."""
     dev = saved.device
     n_predict, mtp_w = _mtp(mtp_weights, dev)
     sz = _lib.sizes_for(N, d, V, n_predict)
@@ -175,6 +184,12 @@ def ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale,
     a.dw, a.dw_dtype, a.dw_ld = dw.data_ptr(), _DTYPES[w_dtype], V
     a.panel_rows = panel_rows
     a.vocab_limit = 0 if vocab_size is None else int(vocab_size)
+    if norm_eps is not None:
+        if hidden is None or tuple(hidden.shape) != (N, d) or hidden.device != dev:
+            raise ValueError("backward through the fused norm needs the (N, d) hidden state given to forward")
+        hidden = hidden if hidden.stride(1) == 1 else hidden.contiguous()
+        a.norm, a.norm_eps = 1, float(norm_eps)
+        a.x, a.x_dtype, a.x_ld = hidden.data_ptr(), _dtype_code(hidden, "hidden"), hidden.stride(0)
     if weight_cache is not None:
         a.wcache, a.wcache_bytes, a.wcache_valid = weight_cache.buf.data_ptr(), weight_cache.buf.numel(), 1
     _lib.check(_lib.lib().sce_backward(C.byref(a)), "sce_backward")
@@ -218,6 +233,32 @@ def _ce_backward_fake(saved, targets, grad_output, mtp_weights, N, d, V, x_s, w_
             saved.new_empty((d, V), dtype=torch.bfloat16 if w_bf16 else torch.float32))
 
 
+@torch.library.custom_op("slowrun_amd::norm_ce_forward", mutates_args=())
+def norm_ce_forward_op(h: torch.Tensor, w: torch.Tensor, targets: torch.Tensor, mtp_weights: Optional[torch.Tensor],
+                       x_s: float, w_s: float, cap: float, mean: bool, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    out, saved, _lse, _am, _nv = ce_forward(h, w, targets, x_s, w_s, cap, "mean" if mean else "none", mtp_weights=mtp_weights,
+                                            norm_eps=eps)
+    return out, saved
+
+
+norm_ce_forward_op.register_fake(lambda h, w, targets, mtp_weights, x_s, w_s, cap, mean, eps:
+                                 _ce_forward_fake(h, w, targets, mtp_weights, x_s, w_s, cap, mean))
+
+
+@torch.library.custom_op("slowrun_amd::norm_ce_backward", mutates_args=())
+def norm_ce_backward_op(saved: torch.Tensor, h: torch.Tensor, targets: torch.Tensor, grad_output: torch.Tensor,
+                        mtp_weights: Optional[torch.Tensor], V: int, x_s: float, w_s: float, cap: float, grad_scale: float,
+                        mean: bool, w_bf16: bool, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    N, d = h.shape
+    return ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale, "mean" if mean else "none",
+                       h.dtype, torch.bfloat16 if w_bf16 else torch.float32, mtp_weights=mtp_weights, hidden=h, norm_eps=eps)
+
+
+@norm_ce_backward_op.register_fake
+def _norm_ce_backward_fake(saved, h, targets, grad_output, mtp_weights, V, x_s, w_s, cap, grad_scale, mean, w_bf16, eps):
+    return torch.empty_like(h), h.new_empty((h.shape[1], V), dtype=torch.bfloat16 if w_bf16 else torch.float32)
+
+
 class FusedSoftcappedCrossEntropy(torch.autograd.Function):
     """Same call as tiny/cuda_kernels.py:336-414; see the module docstring."""
 
@@ -243,6 +284,38 @@ class FusedSoftcappedCrossEntropy(torch.autograd.Function):
         dx, dw = ce_backward_op(saved, targets, grad_output.contiguous(), mtp_w if has_mtp else None, N, d, V, xs, ws_, cap,
                                 gscale, mean, x_bf16, w_bf16)
         return dx, None, None, dw, None, None, None, None, None, None
+
+
+class FusedNormSoftcappedCrossEntropy(torch.autograd.Function):
+    """``FusedSoftcappedCrossEntropy.apply(F.rms_norm(h, (d,), eps=eps), ...)`` in one call: the trunk's final norm
+    (tiny/train.py:397-398,734) runs inside the quantiser, so the normalised activations are never written, and
+    backward returns the gradient with respect to ``h``.  ``eps=None`` is torch's default, float32's machine
+    epsilon for bf16 and fp32 input.  Same argument order as FusedSoftcappedCrossEntropy with ``h`` in place of ``x``."""
+
+    @staticmethod
+    def forward(ctx, h, targets, mtp_weights, lm_head_weight, x_s, w_s, grad_s, grad_scale, cap=15.0, reduction="none",
+                eps=None):
+        if reduction not in ("none", "mean"):
+            raise ValueError("reduction must be 'none' or 'mean'")
+        _dtype_code(h, "h")
+        _dtype_code(lm_head_weight, "lm_head_weight")
+        eps = float(torch.finfo(torch.float32).eps if eps is None else eps)
+        xs, ws_ = _scale_value(x_s, h), _scale_value(w_s, lm_head_weight)
+        hd = h.detach()
+        out, saved = norm_ce_forward_op(hd, lm_head_weight.detach(), targets, mtp_weights, xs, ws_, float(cap),
+                                        reduction == "mean", eps)
+        ctx.save_for_backward(saved, hd, targets, mtp_weights if mtp_weights is not None else torch.empty(0, device=h.device))
+        ctx.params = (lm_head_weight.shape[1], xs, ws_, float(cap), float(grad_scale), reduction == "mean",
+                      lm_head_weight.dtype == torch.bfloat16, mtp_weights is not None, eps)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        saved, h, targets, mtp_w = ctx.saved_tensors
+        V, xs, ws_, cap, gscale, mean, w_bf16, has_mtp, eps = ctx.params
+        dh, dw = norm_ce_backward_op(saved, h, targets, grad_output.contiguous(), mtp_w if has_mtp else None, V, xs, ws_, cap,
+                                     gscale, mean, w_bf16, eps)
+        return dh, None, None, dw, None, None, None, None, None, None, None
 
 
 def softcapped_cross_entropy(x, lm_head_weight, targets, x_s, w_s, cap=15.0, vocab_size=None, reduction="mean"):

@@ -36,7 +36,7 @@ def test_header_functions_are_exported(lib):
 
 
 def test_version(lib):
-    assert lib.sce_version() == _lib.SCE_VERSION == 2
+    assert lib.sce_version() == _lib.SCE_VERSION == 3
 
 
 def test_struct_layout_matches_c(tmp_path):
@@ -56,8 +56,8 @@ def test_struct_layout_matches_c(tmp_path):
 
 def test_sizes_for_and_shape_errors(lib):
     s = _lib.sizes_for(65536, 2560, 50304)
-    # X_q + W_q^T + W_q in e4m3 (rows padded by 128 bytes) plus three per-row statistics: nothing N x V sized is kept for backward
-    assert s.saved_bytes < (65536 + 50432) * (2560 + 128) + 2560 * (50432 + 128) + 4 * 65536 * 4
+    # X_q + W_q^T + W_q in e4m3 (rows padded by 128 bytes) plus four per-row statistics: nothing N x V sized is kept for backward
+    assert s.saved_bytes < (65536 + 50432) * (2560 + 128) + 2560 * (50432 + 128) + 5 * 65536 * 4
     assert s.bwd_workspace_min_bytes <= s.bwd_workspace_bytes
     assert s.bwd_panel_rows % 256 == 0 and s.bwd_panel_rows * 10 <= 256 * 256
     for bad in [(0, 128, 100), (10, 100, 100), (10, 128, 0), (1 << 25, 128, 100)]:
@@ -115,3 +115,7 @@ def test_custom_ops_have_fake_implementations():
     assert out2.shape == ()
     dx, dw = ck.ce_backward_op(saved, y, out, mw, 512, 128, 1024, 0.1, 0.1, 15.0, 1.0, False, True, False)
     assert dx.shape == (512, 128) and dx.dtype == torch.bfloat16 and dw.shape == (128, 1024) and dw.dtype == torch.float32
+    out3, saved3 = ck.norm_ce_forward_op(x, w, y, None, 0.1, 0.1, 15.0, True, 1e-6)
+    assert out3.shape == () and saved3.numel() == _lib.sizes_for(512, 128, 1024, 1).saved_bytes
+    dh, dw2 = ck.norm_ce_backward_op(saved3, x, y, out3, None, 1024, 0.1, 0.1, 15.0, 1.0, True, True, 1e-6)
+    assert dh.shape == (512, 128) and dh.dtype == torch.bfloat16 and dw2.shape == (128, 1024) and dw2.dtype == torch.bfloat16

@@ -315,3 +315,50 @@ def test_captured_in_a_hip_graph_and_replayed():
         for g, e, name in zip(got, want, ("loss", "dx", "dw")):
             assert torch.equal(g, e), f"replay {trial}: {name} differs from the direct calls"
         assert torch.isfinite(got[0])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_final_norm_fused_into_the_head(dtype):
+    """tiny/train.py:734 then :682-696: x = F.rms_norm(h, (d,)) feeds the head.  With the norm inside the quantiser
+    the result must match the oracle (norm restated in fp32, head as everywhere else) and the unfused pair
+    torch rms_norm -> FusedSoftcappedCrossEntropy on the same kernels."""
+    import torch.nn.functional as F
+    from oracle import eager
+    from slowrun_amd.cuda_kernels import FusedNormSoftcappedCrossEntropy, FusedSoftcappedCrossEntropy
+    inp = _small("irregular", 700, 256, 1500)
+    N, d, V = inp.shape
+    gen = torch.Generator().manual_seed(3)
+    h_cpu = (inp.x * (0.5 + 2.5 * torch.rand(N, 1, generator=gen))).to(dtype)
+    w_cpu = inp.w.to(dtype)
+    x_ref, _ = eager.rms_norm(h_cpu)
+    x_s = float(x_ref.float().abs().max()) / 448.0
+    assert int((inp.targets == -1).sum()) > 0
+    ref = eager.norm_softcapped_ce(h_cpu, w_cpu, inp.targets, x_s, inp.w_s, inp.cap, "mean")
+    y = inp.targets.cuda()
+    res = []
+    for fused in (True, False):
+        h = h_cpu.cuda().requires_grad_(True)
+        w = w_cpu.cuda().requires_grad_(True)
+        if fused:
+            loss = FusedNormSoftcappedCrossEntropy.apply(h, y, None, w, x_s, inp.w_s, 0.0, 1.0, inp.cap, "mean")
+        else:
+            loss = FusedSoftcappedCrossEntropy.apply(F.rms_norm(h, (d,)), y, None, w, x_s, inp.w_s, 0.0, 1.0, inp.cap, "mean")
+        loss.backward()
+        res.append((loss.detach().cpu(), h.grad.float().cpu(), w.grad.float().cpu()))
+    (loss, dh, dw), (loss_u, dh_u, dw_u) = res
+    assert abs(float(loss) - float(ref["loss"])) <= 1e-3 * abs(float(ref["loss"]))
+    for name, got, want in (("dh", dh, ref["dx"].float()), ("dw", dw, ref["dw"].float())):
+        mr, cs = pu.maxrel(got, want), pu.cosine(got, want)
+        print(name, mr, cs)
+        assert mr <= 2e-2 and cs > 0.9995, (name, mr, cs)
+    ignored = inp.targets == -1
+    assert float(dh[ignored].abs().max()) == 0.0
+    # torch's GPU rms_norm sums the squares in another order: in fp32 the last bit may differ, in bf16 a few
+    # elements may round to the neighbouring value
+    x_torch = F.rms_norm(h_cpu.cuda(), (d,)).cpu()
+    if dtype == torch.float32:
+        assert pu.maxrel(x_torch, x_ref) < 1e-6
+    else:
+        assert float((x_torch != x_ref).float().mean()) < 1e-3
+    assert abs(float(loss) - float(loss_u)) <= 1e-5 * abs(float(loss_u))
+    assert pu.maxrel(dh, dh_u) < 1e-2 and pu.maxrel(dw, dw_u) < 1e-2

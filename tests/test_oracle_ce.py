@@ -237,3 +237,24 @@ def test_mtp_reference_kernel_formula_on_valid_targets():
                 want[i] += wk * (f["lse"][i] - f["z"][i, y[i + k]])
     o = eager.softcapped_ce_mtp(x, w, y, wts, cap=cap, dtype=torch.float64)
     np.testing.assert_allclose(o["loss"].numpy(), want, atol=1e-12)
+
+
+def test_rms_norm_restatement_vs_library_and_autograd():
+    """oracle.eager.rms_norm / rms_norm_backward against F.rms_norm and its autograd gradient (fp32 and fp64)."""
+    g = torch.Generator().manual_seed(5)
+    h = torch.randn(37, 48, generator=g) * 2.5
+    x, rstd = eager.rms_norm(h)
+    assert torch.equal(x, F.rms_norm(h, (48,)))
+    x2, _ = eager.rms_norm(h, eps=1e-3)
+    assert torch.equal(x2, F.rms_norm(h, (48,), eps=1e-3))
+    hd = h.double().requires_grad_(True)
+    up = torch.randn(37, 48, generator=g, dtype=torch.float64)
+    F.rms_norm(hd, (48,), eps=1e-3).backward(up)
+    _, rstd64 = eager.rms_norm(h.double(), eps=1e-3)
+    ours = eager.rms_norm_backward(h.double(), rstd64.double(), up)
+    # float() inside the restatement limits this to fp32 accuracy
+    assert (ours.double() - hd.grad).abs().max() < 1e-5 * hd.grad.abs().max()
+    # bf16 input: fp32 arithmetic, float32's epsilon by default, a single rounding: bit-identical to the library
+    hb = (torch.randn(300, 2560, generator=g) * 3).bfloat16()
+    assert torch.equal(eager.rms_norm(hb)[0], F.rms_norm(hb, (2560,)))
+    assert torch.equal(eager.rms_norm(hb, eps=1e-6)[0], F.rms_norm(hb, (2560,), eps=1e-6))
