@@ -350,7 +350,7 @@ struct FwdParams {
   int N, V, Np, RT, CT, S;
   float sc;                // x_s * w_s
   float k1;                // x_s * w_s * 2 log2(e) / cap : exp2(acc * k1) = e^{2u/cap}
-  float c2;                // -2 cap log2(e)
+  float ic2;               // 1 / c2, c2 = -2 cap log2(e): e^{z - cap} = exp2(c2 / (1 + e^{2u/cap}))
 };
 
 // Per 256 x 256 tile and per row a lane owns: add up e^{z - cap} over its 64 columns and keep the
@@ -370,8 +370,8 @@ __device__ __forceinline__ void fwd_epilogue(const v16f (&acc)[4][4], const FwdP
       for (int r = 0; r < 16; ++r) {
         const int vo = a * 32 + 8 * (r >> 2) + (r & 3);
         float x = acc[a][b][r];
-        const float rr = fast_rcp(fast_exp2(x * p.k1) + 1.0f);
-        float pt = fast_exp2(p.c2 * rr);
+        // z - cap = c2 / (1 + e^{2u/cap}) in units of log2: the reciprocal of (1 + e) / c2 gives it in one step
+        float pt = fast_exp2(fast_rcp(fmaf(fast_exp2(x * p.k1), p.ic2, p.ic2)));
         if (EDGE) {
           if (vo >= p.V - vbase) { pt = 0.f; x = -INFINITY; }
         }
@@ -1403,7 +1403,7 @@ extern "C" int sce_forward(const sce_args* a) {
   FwdParams p;
   p.xq = xq; p.wqt = wqt; p.partials = (float4*)a->workspace;
   p.dp = S.dp; p.ldx = S.ldx; p.N = (int)N; p.V = (int)Vl; p.Np = (int)S.Np; p.RT = RT; p.CT = CT; p.S = nsplit;
-  p.sc = a->x_s * a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.c2 = -2.0f * a->cap * LOG2E;
+  p.sc = a->x_s * a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.ic2 = 1.0f / (-2.0f * a->cap * LOG2E);
   const int grid = 8 * nsplit * ((RT + 7) / 8);
   {
     KernelTimer tm(SCE_K_FWD, st);
