@@ -701,7 +701,7 @@ struct RecomputeParams {
 // the four lanes of a quad hold four consecutive rows of the same four columns, and two quad-permute + byte-permute
 // steps turn that 4 x 4 byte block around.
 constexpr int STG_PITCH = 272;                               // 256 + 16: 16-byte aligned, rows shifted by 4 banks
-constexpr int SMEM_RECOMPUTE = SMEM_BYTES;                   // the main loop's two K slots; the staging tile (69632 B) reuses them
+constexpr int SMEM_RECOMPUTE = SMEM_BYTES + 2048;      // two K-block slots (the staging tile, 69632 B, reuses them) + 128 row constants per wave
 
 __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -712,6 +712,17 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   // still in the memory-side cache.
   ct = p.CT - 1 - ct;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
+  // The row constants of the wave's 128 rows go straight to LDS, behind the two slots: requested before the
+  // K loop (whose waits for its own, younger loads cover them), read after it, no register held in between.
+  {
+    const int wu = __builtin_amdgcn_readfirstlane(wave);
+    const uint32_t dst = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)(smem + SMEM_BYTES)) + wu * 512;
+    const float* src = p.crow + rt * 256 + (wu & 1) * 128;
+    // the instruction's offset moves the memory address and the LDS address alike: the second half of the rows
+    asm volatile("s_add_u32 m0, %0, 0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n\t"
+                 "global_load_lds_dword %1, %2 offset:256"
+                 ::"s"(dst), "v"(lane * 4), "s"(src) : "memory", "scc");
+  }
   v16f acc[4][4];
   mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave));
   uint8_t* TT = smem;                        // [256 columns v][STG_PITCH]: rows i contiguous
@@ -726,20 +737,29 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       const int iloc = wb * 128 + b * 32 + (lane & 31);        // row within the tile
-      const float c = p.crow[rt * 256 + iloc];
+      const float c = *reinterpret_cast<const float*>(smem + SMEM_BYTES + wave * 512 + (b * 32 + (lane & 31)) * 4);
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
         // stage by stage over the 16 values of the block: the transcendental unit is pipelined, a chain
-        // of dependent exp2 / rcp / exp2 on one value at a time is not
+        // of dependent exp2 / rcp / exp2 on one value at a time is not (the scheduler would rebuild the
+        // chains to save registers, hence the barriers)
+        constexpr int NB = 8;        // values per batch: 4, 8 and 16 measure alike
         float rr[16], gg[16];
 #pragma unroll
-        for (int m = 0; m < 16; ++m) rr[m] = fast_exp2(acc[a][b][m] * p.k1);
+        for (int g0 = 0; g0 < 16; g0 += NB) {
 #pragma unroll
-        for (int m = 0; m < 16; ++m) rr[m] = fast_rcp(rr[m] + 1.0f);
+          for (int m = g0; m < g0 + NB; ++m) rr[m] = fast_exp2(acc[a][b][m] * p.k1);
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int m = 0; m < 16; ++m) gg[m] = fast_exp2(fmaf(p.c2, rr[m], c));
+          for (int m = g0; m < g0 + NB; ++m) rr[m] = fast_rcp(rr[m] + 1.0f);
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int m = 0; m < 16; ++m) gg[m] *= rr[m] - rr[m] * rr[m];
+          for (int m = g0; m < g0 + NB; ++m) gg[m] = fast_exp2(fmaf(p.c2, rr[m], c));
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int m = g0; m < g0 + NB; ++m) gg[m] *= rr[m] - rr[m] * rr[m];
+          __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int vloc = vloc0 + a * 32 + 8 * q;
@@ -749,9 +769,9 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
           }
           const uint32_t w = cvt4_e4m3(gg[4 * q], gg[4 * q + 1], gg[4 * q + 2], gg[4 * q + 3]);
           // 4 x 4 byte transpose inside the quad: lane k ends up with column vloc + k, rows (iloc & ~3) .. +3
-          const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xB1, 0xF, 0xF, false);    // lane ^ 1
+          const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xB1, 0xF, 0xF, true);     // lane ^ 1
           const uint32_t x = __builtin_amdgcn_perm(p1, w, sel1);
-          const uint32_t p2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, false);    // lane ^ 2
+          const uint32_t p2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, true);     // lane ^ 2
           const uint32_t yv = __builtin_amdgcn_perm(p2, x, sel2);
           *reinterpret_cast<uint32_t*>(TT + (vloc + k) * STG_PITCH + (iloc & ~3)) = yv;
         }
