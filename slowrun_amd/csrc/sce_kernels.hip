@@ -779,12 +779,14 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
     }
   };
   if (edge) form_g(std::true_type{}); else form_g(std::false_type{});
-  __syncthreads();
-  uint8_t* gcol = p.ghat_t + ((int64_t)ct * p.kbw + p.kb0 + 2 * rt) * BLOCKED_KSTEP;   // two K blocks of 256 rows x 128 B
+  // Each wave takes its own quadrant out (128 columns v x 128 rows i = one contiguous 16 KB run of the K block
+  // wb): it reads only what it wrote itself, so no barrier is needed and no wave waits for the slowest one.
+  uint8_t* gcol = p.ghat_t + ((int64_t)ct * p.kbw + p.kb0 + 2 * rt + wb) * BLOCKED_KSTEP + wa * 128 * BK;
+  const uint8_t* tq = TT + wa * 128 * STG_PITCH + wb * 128;
 #pragma unroll
   for (int n = 0; n < 16; ++n) {
-    const int cidx = t + 256 * n, row = cidx >> 4, col = (cidx & 15) * 16;
-    *reinterpret_cast<v4i*>(gcol + (col >> 7) * BLOCKED_KSTEP + row * BK + (col & 127)) = *reinterpret_cast<const v4i*>(TT + row * STG_PITCH + col);
+    const int cidx = lane + 64 * n, row = cidx >> 3, col = (cidx & 7) * 16;
+    *reinterpret_cast<v4i*>(gcol + row * BK + col) = *reinterpret_cast<const v4i*>(tq + row * STG_PITCH + col);
   }
 }
 
