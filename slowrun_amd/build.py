@@ -37,6 +37,23 @@ def build_library(verbose=True, jobs=2):
     return LIB_PATH
 
 
+def build_abi_example(verbose=True):
+    """tests/abi_example.c -> tests/bin/abi_example: a plain C caller of the library (gcc, no hipcc), linked against
+    libslowrun_ce.so and the HIP runtime.  Run by tests/test_c_abi.py on a GPU."""
+    root = os.path.dirname(HERE)
+    out_dir = os.path.join(root, "tests", "bin")
+    os.makedirs(out_dir, exist_ok=True)
+    exe = os.path.join(out_dir, "abi_example")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = ["gcc", "-std=c11", "-O2", "-Wall", "-D__HIP_PLATFORM_AMD__", f"-I{rocm}/include", f"-I{os.path.join(root, 'include')}",
+           os.path.join(root, "tests", "abi_example.c"), "-o", exe, f"-L{rocm}/lib", "-lamdhip64", f"-L{HERE}", "-lslowrun_ce", "-lm",
+           "-Wl,-rpath,$ORIGIN/../../slowrun_amd", f"-Wl,-rpath,{rocm}/lib"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return exe
+
+
 def _wait(procs, verbose):
     while procs:
         src, p = procs.pop(0)
@@ -50,4 +67,5 @@ def _wait(procs, verbose):
 
 if __name__ == "__main__":
     print(build_library())
+    print(build_abi_example())
     sys.exit(0)
