@@ -119,3 +119,27 @@ def test_custom_ops_have_fake_implementations():
     assert out3.shape == () and saved3.numel() == _lib.sizes_for(512, 128, 1024, 1).saved_bytes
     dh, dw2 = ck.norm_ce_backward_op(saved3, x, y, out3, None, 1024, 0.1, 0.1, 15.0, 1.0, True, True, 1e-6)
     assert dh.shape == (512, 128) and dh.dtype == torch.bfloat16 and dw2.shape == (128, 1024) and dw2.dtype == torch.bfloat16
+
+
+def test_error_messages_are_per_thread(lib):
+    """sce_last_error is thread-local: concurrent callers that fail in different ways each read their own message."""
+    import threading
+    results = {}
+
+    def worker(tag, shape_args, needle):
+        ok = True
+        for _ in range(200):
+            shape = _lib.SceShape(*shape_args)
+            out = _lib.SceSizes()
+            rc = lib.sce_sizes_for(C.byref(shape), C.byref(out))
+            ok = ok and rc == 1 and needle in lib.sce_last_error()
+        results[tag] = ok
+
+    threads = [threading.Thread(target=worker, args=("d", (10, 100, 100, 1, 0), b"multiple of 16")),
+               threading.Thread(target=worker, args=("k", (10, 128, 100, 7, 0), b"n_predict")),
+               threading.Thread(target=worker, args=("n", (0, 128, 100, 1, 0), b"positive"))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert results == {"d": True, "k": True, "n": True}
