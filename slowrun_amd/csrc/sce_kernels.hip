@@ -518,41 +518,71 @@ __device__ __forceinline__ bool target_valid(const int64_t* __restrict__ targets
   return (y != ignore_index) && y >= 0 && y < V;
 }
 
+// What a block of 256 rows contributes to the mean loss: left by fwd_combine_kernel in the first 16 bytes of the
+// block's own rows of the partial records (which it has consumed by then), summed by fwd_reduce_kernel.
+struct BlockLoss {
+  double sum;      // sum of lse_i - z[i, y_i] over the valid rows
+  int32_t cnt;     // valid rows
+  int32_t bad;     // targets outside [0, V) other than ignore_index
+};
+static_assert(sizeof(BlockLoss) == 16, "one float4 slot");
+
 // one thread per row: fold the V-splits, write lse / loss / argmax and the saved row statistics
-__global__ __launch_bounds__(256) void fwd_combine_kernel(const float4* __restrict__ partials, int S, int N, int Np, int V,
+__global__ __launch_bounds__(256) void fwd_combine_kernel(float4* __restrict__ partials, int S, int N, int Np, int V,
                                                          const int64_t* __restrict__ targets, int64_t ignore_index, float cap,
                                                          const float* __restrict__ mtp_weights, int n_predict,
                                                          float* __restrict__ s_lse, float* __restrict__ s_umax,
                                                          const float* __restrict__ s_zy, float* __restrict__ losses,
                                                          float* __restrict__ lse_out, int32_t* __restrict__ argmax_out) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= Np) return;
-  if (i >= N) { s_lse[i] = 0.f; s_umax[i] = 0.f; return; }
-  float sum = 0.f, umax = -INFINITY;
-  int uarg = 0x7fffffff;
-  for (int s = 0; s < S; ++s) {
-    const float4 o = partials[(int64_t)s * Np + i];
-    const int ua = __float_as_int(o.z);
-    sum += o.x;
-    if (o.y > umax || (o.y == umax && ua < uarg)) { umax = o.y; uarg = ua; }
+  __shared__ double ssum[256];
+  __shared__ int scnt[256], sbad[256];
+  const int t = threadIdx.x, i = blockIdx.x * 256 + t;      // the grid covers Np = 256 * gridDim.x rows exactly
+  double term = 0.0;
+  int cnt = 0, bad = 0;
+  if (i >= N) {
+    s_lse[i] = 0.f; s_umax[i] = 0.f;
+  } else {
+    float sum = 0.f, umax = -INFINITY;
+    int uarg = 0x7fffffff;
+    for (int s = 0; s < S; ++s) {
+      const float4 o = partials[(int64_t)s * Np + i];
+      const int ua = __float_as_int(o.z);
+      sum += o.x;
+      if (o.y > umax || (o.y == umax && ua < uarg)) { umax = o.y; uarg = ua; }
+    }
+    const float lse = cap + logf(sum);
+    s_lse[i] = lse; s_umax[i] = umax;
+    if (losses) {
+      // loss_i = sum_k w_k (lse_i - z[i, y_{i+k}]) over the offsets that take part (tiny/cuda_kernels.py:226-240)
+      float l = 0.f;
+      for (int k = 0; k < n_predict; ++k)
+        if (target_valid(targets, ignore_index, i + k, N, V))
+          l += (mtp_weights ? mtp_weights[k] : 1.0f) * (lse - s_zy[(int64_t)k * Np + i]);
+      losses[i] = l;
+    }
+    if (lse_out) lse_out[i] = lse;
+    if (argmax_out) argmax_out[i] = (uarg == 0x7fffffff) ? 0 : uarg;
+    const int64_t y = targets[i];
+    if (y != ignore_index) {
+      if (y < 0 || y >= V) bad = 1;
+      else { term = (double)(lse - s_zy[i]); cnt = 1; }
+    }
   }
-  const float lse = cap + logf(sum);
-  s_lse[i] = lse; s_umax[i] = umax;
-  if (losses) {
-    // loss_i = sum_k w_k (lse_i - z[i, y_{i+k}]) over the offsets that take part (tiny/cuda_kernels.py:226-240)
-    float l = 0.f;
-    for (int k = 0; k < n_predict; ++k)
-      if (target_valid(targets, ignore_index, i + k, N, V))
-        l += (mtp_weights ? mtp_weights[k] : 1.0f) * (lse - s_zy[(int64_t)k * Np + i]);
-    losses[i] = l;
+  ssum[t] = term; scnt[t] = cnt; sbad[t] = bad;
+  __syncthreads();               // also: every row of this block has read its partial records
+  for (int w = 128; w > 0; w >>= 1) {
+    if (t < w) { ssum[t] += ssum[t + w]; scnt[t] += scnt[t + w]; sbad[t] += sbad[t + w]; }
+    __syncthreads();
   }
-  if (lse_out) lse_out[i] = lse;
-  if (argmax_out) argmax_out[i] = (uarg == 0x7fffffff) ? 0 : uarg;
+  if (t == 0) {
+    BlockLoss bl;
+    bl.sum = ssum[0]; bl.cnt = scnt[0]; bl.bad = sbad[0];
+    *reinterpret_cast<BlockLoss*>(partials + (int64_t)blockIdx.x * 256) = bl;
+  }
 }
 
-// single workgroup: n_valid, number of out-of-range targets, mean loss (deterministic order)
-__global__ __launch_bounds__(1024) void fwd_reduce_kernel(const float* __restrict__ s_lse, const float* __restrict__ s_zy,
-                                                         const int64_t* __restrict__ targets, int64_t ignore_index, int N, int V,
+// single workgroup: n_valid, number of out-of-range targets, mean loss from the per-block sums (fixed order)
+__global__ __launch_bounds__(1024) void fwd_reduce_kernel(const float4* __restrict__ partials, int nblk,
                                                          int32_t* __restrict__ hdr, float* __restrict__ loss_out,
                                                          int32_t* __restrict__ nvalid_out) {
   __shared__ double ssum[1024];
@@ -560,12 +590,9 @@ __global__ __launch_bounds__(1024) void fwd_reduce_kernel(const float* __restric
   const int t = threadIdx.x;
   double acc = 0.0;
   int cnt = 0, bad = 0;
-  for (int i = t; i < N; i += 1024) {
-    const int64_t y = targets[i];
-    if (y == ignore_index) continue;
-    if (y < 0 || y >= V) { ++bad; continue; }
-    acc += (double)(s_lse[i] - s_zy[i]);
-    ++cnt;
+  for (int b = t; b < nblk; b += 1024) {
+    const BlockLoss bl = *reinterpret_cast<const BlockLoss*>(partials + (int64_t)b * 256);
+    acc += bl.sum; cnt += bl.cnt; bad += bl.bad;
   }
   ssum[t] = acc; scnt[t] = cnt; sbad[t] = bad;
   __syncthreads();
@@ -1440,7 +1467,7 @@ extern "C" int sce_forward(const sce_args* a) {
   fwd_combine_kernel<<<(int)(S.Np / 256), 256, 0, st>>>(p.partials, nsplit, (int)N, (int)S.Np, (int)Vl, a->targets, a->ignore_index,
                                                        a->cap, a->mtp_weights, a->shape.n_predict, s_lse, s_umax, s_zy, a->losses, a->lse,
                                                        a->argmax);
-  fwd_reduce_kernel<<<1, 1024, 0, st>>>(s_lse, s_zy, a->targets, a->ignore_index, (int)N, (int)Vl, (int32_t*)(sv + S.off_hdr),
+  fwd_reduce_kernel<<<1, 1024, 0, st>>>(p.partials, (int)(S.Np / 256), (int32_t*)(sv + S.off_hdr),
                                         a->reduction == SCE_REDUCE_MEAN ? a->loss : nullptr, a->n_valid);
   HIP_TRY(hipGetLastError());
   return SCE_OK;
