@@ -29,6 +29,12 @@ closed_form.backward            central finite differences of closed_form.forwar
                                 dX row, autograd (torch float64) on the same inputs.
 eager.softcapped_ce_mtp         n_predict=1 == plain path bit for bit;
                                 weights [1,0,0] == [1]; against closed_form MTP.
+eager.rms_norm                  bit-identical to F.rms_norm (fp32 and bf16 input,
+                                default and explicit eps).
+eager.rms_norm_backward         against torch's autograd through F.rms_norm in
+                                float64.
+eager.norm_softcapped_ce        is the composition of the two above with
+                                softcapped_ce.
 
 The reference holds no golden vectors, tests or fixtures for this path, and its
 fused CUDA kernel cannot be imported on this toolchain, so the reference's own
