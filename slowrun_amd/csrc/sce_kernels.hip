@@ -1160,6 +1160,8 @@ struct DeviceGuard {
 
 static std::mutex g_mu;
 static int g_arch_ok[64];   // 0 unknown, 1 gfx950, -1 other
+static int g_cus[64];       // compute units, filled with g_arch_ok
+static inline int device_cus_or_default(int dev) { return (dev >= 0 && dev < 64 && g_cus[dev] > 0) ? g_cus[dev] : 256; }
 
 // Optional per-kernel timing with HIP events on the caller's stream (off by default).
 struct TimingState {
@@ -1206,6 +1208,7 @@ static int check_device(int dev) {
     hipDeviceProp_t prop;
     HIP_TRY(hipGetDeviceProperties(&prop, dev));
     g_arch_ok[dev] = strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : -1;
+    g_cus[dev] = prop.multiProcessorCount;
     if (g_arch_ok[dev] == 1) {
       // the MFMA kernels hold two 64 KB K-slots in LDS
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
@@ -1330,6 +1333,19 @@ extern "C" int sce_timing_read(sce_timing* out) {
 }
 extern "C" const char* sce_last_error(void) { return g_err; }
 
+// Forward splits V among S workgroups per row tile (each walks CT / S column tiles).  8 keeps the partial records
+// small and gives every workgroup a long walk; more (up to 16) only where 8 would leave the last round of
+// workgroups, one per CU, mostly empty.
+constexpr int FWD_MAX_SPLITS = 16;
+static int fwd_splits(int RT, int CT, int ncu) {
+  if (CT <= 8) return CT;
+  auto fill = [&](int S) { const int64_t wg = (int64_t)RT * S; return (double)wg / (double)((wg + ncu - 1) / ncu * ncu); };
+  int best = 8;
+  for (int S = 9; S <= FWD_MAX_SPLITS && S <= CT; ++S)
+    if (fill(S) > fill(best) + 0.03) best = S;
+  return best;
+}
+
 extern "C" int sce_sizes_for(const sce_shape* shape, sce_sizes* out) {
   if (int rc = check_shape(shape)) return rc;
   if (!out) return fail(SCE_EINVAL, "out is NULL");
@@ -1337,7 +1353,7 @@ extern "C" int sce_sizes_for(const sce_shape* shape, sce_sizes* out) {
   out->saved_bytes = S.total;
   out->saved_x_bytes = S.x_total;
   out->wcache_bytes = S.w_total;
-  out->fwd_workspace_bytes = (size_t)8 * S.Np * 16 + 256;
+  out->fwd_workspace_bytes = (size_t)FWD_MAX_SPLITS * S.Np * 16 + 256;
   out->bwd_workspace_min_bytes = bwd_layout(S, 256, 256, 1, shape->n_predict).total;
   out->bwd_panel_rows = default_panel(S);
   {
@@ -1414,7 +1430,7 @@ extern "C" int sce_forward(const sce_args* a) {
   if (a->wcache && a->wcache_bytes < S.w_total) return fail(SCE_EINVAL, "weight cache too small: %zu < %zu", a->wcache_bytes, S.w_total);
   const int64_t Vl = a->vocab_limit > 0 ? a->vocab_limit : V;       // columns that take part
   const int RT = (int)(S.Np / 256), CT = (int)((Vl + 255) / 256);
-  const int nsplit = CT < 8 ? CT : 8;
+  const int nsplit = fwd_splits(RT, CT, device_cus_or_default(a->device));
   const size_t need_ws = (size_t)nsplit * S.Np * 16;
   if (!a->workspace || a->workspace_bytes < need_ws) return fail(SCE_EINVAL, "forward workspace too small: %zu < %zu", a->workspace_bytes, need_ws);
   DeviceGuard guard(a->device);
