@@ -96,6 +96,19 @@ __device__ __forceinline__ bool map_tile(int bid, int RT, int CT, int& rt, int& 
 }
 static inline int map_tile_grid(int RT, int CT) { return 8 * ((RT * CT + 7) / 8); }
 
+// The same order, dealt out differently: blocks of 32 consecutive tiles go round-robin to the XCDs, so that the
+// 256 workgroups that run at one time work on 256 consecutive tiles of the order (8 neighbouring 4 x 8 blocks).
+// What the XCDs stream from memory at one time is then the same few operand tiles, not eight distant sets.
+__device__ __forceinline__ bool map_tile_rr(int bid, int RT, int CT, int& rt, int& ct) {
+  const int T = RT * CT;
+  const int xcd = bid & 7, local = bid >> 3;
+  const int idx = (((local >> 5) << 3) + xcd) * 32 + (local & 31);
+  if (idx >= T) return false;
+  tile_from_index(idx, RT, CT, rt, ct);
+  return true;
+}
+static inline int map_tile_rr_grid(int RT, int CT) { return 256 * ((RT * CT + 255) / 256); }
+
 // ------------------------------------------------------------------------------------------
 // quantisation
 // ------------------------------------------------------------------------------------------
@@ -948,7 +961,7 @@ template <bool ACC>
 __global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   int rt, ct;
-  if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
+  if (!map_tile_rr(blockIdx.x, p.RT, p.CT, rt, ct)) return;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
   mfma_mainloop<false, NoHook, BLOCKED_KSTEP>(p.xt + ((int64_t)rt * p.kbn + p.kb0) * BLOCKED_KSTEP, BK, p.ghat_t + (int64_t)ct * p.kbw * BLOCKED_KSTEP, BK, p.KT,
@@ -1640,8 +1653,8 @@ extern "C" int sce_backward(const sce_args* a) {
       wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(gathered / BK);
       {
         KernelTimer tm(SCE_K_DW, st);
-        if (launch >= nparts) bwd_dw_kernel<true><<<map_tile_grid(CTd, CTv), NTHREADS, SMEM_BYTES, st>>>(wp);
-        else bwd_dw_kernel<false><<<map_tile_grid(CTd, CTv), NTHREADS, SMEM_BYTES, st>>>(wp);
+        if (launch >= nparts) bwd_dw_kernel<true><<<map_tile_rr_grid(CTd, CTv), NTHREADS, SMEM_BYTES, st>>>(wp);
+        else bwd_dw_kernel<false><<<map_tile_rr_grid(CTd, CTv), NTHREADS, SMEM_BYTES, st>>>(wp);
       }
       ++launch;
       w0 = p0 + prow;
