@@ -45,7 +45,7 @@ static inline int64_t row_stride(int64_t k) { return k + 128; }
 // quantised copies of W come last; with a caller-provided weight cache they live there instead
 // (same relative offsets) and `saved` ends at x_total.
 struct SavedLayout {
-  int64_t ldx, ldv;                  // row strides in bytes of the [..][dp] and of the [..][Vp] e4m3 arrays
+  int64_t ldx;                       // row stride in bytes of the [..][dp] e4m3 arrays
   int64_t N, d, V, Np, dp, dq, Vp;   // all padded sizes are multiples of 256 (every K loop runs over an even number of 128-byte blocks); dp = dq
   size_t off_hdr, off_xq, off_lse, off_umax, off_zy, off_rstd, x_total;
   size_t rel_wqt, rel_wq, w_total;   // relative to the start of the W region
@@ -57,7 +57,7 @@ static inline SavedLayout saved_layout(int64_t N, int64_t d, int64_t V, int n_pr
   SavedLayout L;
   L.N = N; L.d = d; L.V = V;
   L.Np = round_up(N, 256); L.dp = round_up(d, 256); L.dq = round_up(d, 256); L.Vp = round_up(V, 256);
-  L.ldx = row_stride(L.dp); L.ldv = row_stride(L.Vp);
+  L.ldx = row_stride(L.dp);
   size_t o = 0;
   auto take = [&](size_t bytes) { size_t r = o; o += (bytes + 255) / 256 * 256; return r; };
   L.off_hdr = take(256);
@@ -69,7 +69,7 @@ static inline SavedLayout saved_layout(int64_t N, int64_t d, int64_t V, int n_pr
   L.x_total = o;
   o = 0;
   L.rel_wqt = take((size_t)L.Vp * L.ldx);      // W_q^T [Vp][dp], row stride ldx
-  L.rel_wq = take((size_t)L.dq * L.ldv);       // W_q   [dq][Vp], row stride ldv
+  L.rel_wq = take((size_t)L.dq * L.Vp);        // W_q: dq rows, K = Vp, tile by tile (256 rows x 128 B per K block)
   L.w_total = o;
   L.total = L.x_total + L.w_total;
   return L;

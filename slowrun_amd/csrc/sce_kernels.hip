@@ -283,11 +283,20 @@ __global__ __launch_bounds__(256) void rmsnorm_backward_kernel(TG* __restrict__ 
   }
 }
 
-// W (d, V) -> W_q [dq][Vp] (same orientation) and W_q^T [Vp][dp]; 64 x 64 tiles through LDS.
+// Operands with a long K (the two of dW, and W_q in dX) are stored tile by tile: for every 256 rows, K block
+// after K block, 256 rows of 128 bytes each.  A workgroup's load of one K block of one operand is then one
+// contiguous 32 KB piece (row-major rows lie Np, Pw or Vp bytes apart, and the dW main loop lost 12 % to that at
+// K = 65536).
+__device__ __forceinline__ int64_t blocked_offset(int64_t row, int64_t k, int64_t kblocks) {
+  return (((row >> 8) * kblocks + (k >> 7)) * 256 + (row & 255)) * 128 + (k & 127);
+}
+constexpr int BLOCKED_KSTEP = 256 * BK;     // bytes from one K block of a tile to the next
+
+// W (d, V) -> W_q (dq rows, K = Vp, tile by tile) and W_q^T [Vp][dp] (row-major); 64 x 64 tiles through LDS.
 template <typename T>
 __global__ __launch_bounds__(256) void quantize_w_kernel(const T* __restrict__ w, int64_t ld, int64_t d, int64_t V,
                                                         uint8_t* __restrict__ wq, uint8_t* __restrict__ wqt,
-                                                        int64_t dp, int64_t ldx, int64_t ldv, float scale) {
+                                                        int64_t dp, int64_t ldx, int64_t kbv, float scale) {
   __shared__ uint8_t tile[64][68];
   const int t = threadIdx.x;
   const int64_t j0 = (int64_t)blockIdx.y * 64, v0 = (int64_t)blockIdx.x * 64;
@@ -301,7 +310,7 @@ __global__ __launch_bounds__(256) void quantize_w_kernel(const T* __restrict__ w
 #pragma unroll
       for (int m = 0; m < 4; ++m) out[m] = cvt4_e4m3(x[4 * m], x[4 * m + 1], x[4 * m + 2], x[4 * m + 3]);
     }
-    *reinterpret_cast<v4i*>(wq + j * ldv + v) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
+    *reinterpret_cast<v4i*>(wq + blocked_offset(j, v, kbv)) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
 #pragma unroll
     for (int m = 0; m < 4; ++m) *reinterpret_cast<uint32_t*>(&tile[r][c + 4 * m]) = out[m];
   }
@@ -683,14 +692,6 @@ __global__ __launch_bounds__(1024) void bwd_xi_kernel(const float* __restrict__ 
   if (threadIdx.x == 0) xi[0] = (smax[0] > 0.f && isfinite(smax[0])) ? smax[0] : 1.0f;
 }
 
-// The two operands of dW are stored tile by tile: for every 256 rows, K block after K block, 256 rows of
-// 128 bytes each.  A workgroup's load of one K block of one operand is then one contiguous 32 KB piece
-// (row-major rows lie Np or Pw bytes apart, and the dW main loop lost 12 % to that at K = 65536).
-__device__ __forceinline__ int64_t blocked_offset(int64_t row, int64_t k, int64_t kblocks) {
-  return (((row >> 8) * kblocks + (k >> 7)) * 256 + (row & 255)) * 128 + (k & 127);
-}
-constexpr int BLOCKED_KSTEP = 256 * BK;     // bytes from one K block of a tile to the next
-
 // Xt (blocked, dq rows, K = Np) = e4m3( X_q[i][j] * rho_i / xi ), transposed through LDS in 64 x 64 tiles.
 __global__ __launch_bounds__(256) void bwd_xt_kernel(const uint8_t* __restrict__ xq, int64_t dp, int64_t ldx, int64_t kbn,
                                                     const float* __restrict__ rho, const float* __restrict__ xi,
@@ -831,7 +832,7 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
 }
 
 struct DxParams {
-  const uint8_t* wq;      // [dq][Vp]   A side (rows j)
+  const uint8_t* wq;      // dq rows, K = Vp, tile by tile: A side (rows j)
   const uint8_t* ghat_t;  // G^T, blocked; already at the K block of the panel's first row    B side (rows i of the panel)
   const uint8_t* wqt;     // [Vp][dp]   for the one-hot gather
   const float* rho;       // offset to the panel
@@ -839,7 +840,7 @@ struct DxParams {
   const int64_t* targets; // offset to the panel
   void* dx;               // offset to the panel's first row
   float* part;            // [ksplit][RT * 256][dq] fp32 partial sums (ksplit > 1 only)
-  int64_t dx_ld, Vp, ldv, ldx, Np, dq;   // Vp: K extent; ldv: row stride of wq; ldx: of wqt
+  int64_t dx_ld, Vp, ldx, Np, dq;        // Vp: K extent; ldx: row stride of wqt
   int64_t kbw;                           // K blocks (of 128 rows i) per v tile of ghat_t
   int RT, CT, rows, d, V;  // rows: valid rows in this panel
   int n_predict, rows_left; // rows_left: N - (first row of the panel), bounds the target look-ahead
@@ -902,8 +903,9 @@ __global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p) {
   // B = G^T: K (v) is the slow index there.  The 128 v rows of a K block are half a v tile; the 256 panel rows of this
   // tile are the two 128-byte pieces of i blocks 2 rt and 2 rt + 1 (BLOCKED_KSTEP apart).
   const int64_t bpair = p.kbw * BLOCKED_KSTEP;                     // from one v tile (two K blocks) to the next
-  mfma_mainloop<false, NoHook, BK, true>(p.wq + (int64_t)ct * 256 * p.ldv + k0, p.ldv, p.ghat_t + 2 * (int64_t)rt * BLOCKED_KSTEP + (k0 / (2 * BK)) * bpair,
-                                         BLOCKED_KSTEP, KD, smem, acc, 2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave), NoHook(), 128 * BK, bpair);
+  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, true>(p.wq + ((int64_t)ct * (p.Vp / BK) + k0 / BK) * BLOCKED_KSTEP, BK,
+                                                    p.ghat_t + 2 * (int64_t)rt * BLOCKED_KSTEP + (k0 / (2 * BK)) * bpair, BLOCKED_KSTEP, KD, smem, acc,
+                                                    2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave), NoHook(), 128 * BK, bpair);
   const int jbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
   T* dx = reinterpret_cast<T*>(p.dx);
 #pragma unroll
@@ -1473,9 +1475,9 @@ extern "C" int sce_forward(const sce_args* a) {
     if (a->wcache && a->wcache_valid) {
       // the caller vouches that the cache holds e4m3(W / w_s) of this W (unchanged since an earlier call)
     } else if (a->w_dtype == SCE_F32)
-      quantize_w_kernel<float><<<gw, 256, 0, st>>>((const float*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.ldv, a->w_s);
+      quantize_w_kernel<float><<<gw, 256, 0, st>>>((const float*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.Vp / BK, a->w_s);
     else if (a->w_dtype == SCE_BF16)
-      quantize_w_kernel<bf16_t><<<gw, 256, 0, st>>>((const bf16_t*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.ldv, a->w_s);
+      quantize_w_kernel<bf16_t><<<gw, 256, 0, st>>>((const bf16_t*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.Vp / BK, a->w_s);
     else return fail(SCE_EINVAL, "unsupported w dtype %d", a->w_dtype);
   }
   FwdParams p;
@@ -1615,7 +1617,7 @@ extern "C" int sce_backward(const sce_args* a) {
 
     DxParams dp_;
     dp_.wq = wq; dp_.ghat_t = ghat_t + ((p0 - w0) / BK) * BLOCKED_KSTEP; dp_.kbw = Pw / BK; dp_.wqt = wqt; dp_.rho = rho + p0; dp_.hcoef = hcoef + p0; dp_.targets = a->targets + p0;
-    dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.ldv = S.ldv; dp_.ldx = S.ldx; dp_.Np = S.Np; dp_.dq = S.dq; dp_.RT = RTp; dp_.CT = CTd;
+    dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.ldx = S.ldx; dp_.Np = S.Np; dp_.dq = S.dq; dp_.RT = RTp; dp_.CT = CTd;
     dp_.n_predict = K; dp_.rows_left = (int)(N - p0 > 0 ? N - p0 : 0);
     dp_.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); dp_.d = (int)d; dp_.V = (int)Vl; dp_.w_s = a->w_s;
     dp_.part = (float*)(ws + B.off_dxpart);
