@@ -318,15 +318,18 @@ class FusedNormSoftcappedCrossEntropy(torch.autograd.Function):
         return dh, None, None, dw, None, None, None, None, None, None, None
 
 
-def softcapped_cross_entropy(x, lm_head_weight, targets, x_s, w_s, cap=15.0, vocab_size=None, reduction="mean"):
+def softcapped_cross_entropy(x, lm_head_weight, targets, x_s, w_s, cap=15.0, vocab_size=None, reduction="mean",
+                             norm_eps=None):
     """Forward-only loss of the eager head (tiny/train.py:741-743) on the fused kernel:
     ``F.cross_entropy(cap * tanh((x @ W)[..., :vocab_size] / cap), targets, ignore_index=-1, reduction=...)`` with
-    fp8 operands; the N x V logits are never stored.  ``x`` may have leading batch dimensions."""
+    fp8 operands; the N x V logits are never stored.  ``x`` may have leading batch dimensions.  With ``norm_eps``
+    given, ``x`` is the hidden state before the final ``F.rms_norm(x, (d,), eps=norm_eps)`` (tiny/train.py:734),
+    which is then applied inside the quantiser."""
     lead = x.shape[:-1]
     x2 = x.reshape(-1, x.shape[-1])
     out, _saved, _lse, _am, _nv = ce_forward(x2.detach(), lm_head_weight.detach(), targets.reshape(-1),
                                              _scale_value(x_s, x2), _scale_value(w_s, lm_head_weight), float(cap),
-                                             reduction, vocab_size=vocab_size)
+                                             reduction, vocab_size=vocab_size, norm_eps=norm_eps)
     return out if reduction == "mean" else out.reshape(lead)
 
 

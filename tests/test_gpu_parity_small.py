@@ -393,3 +393,37 @@ def test_ragged_and_tiny_shapes(N, d, V):
     assert torch.equal(small["dx"], ours["dx"])
     assert pu.maxrel(small["dw"].float(), ours["dw"].float()) < 1e-2
     print(N, d, V, reduction, rep)
+
+
+def test_fused_norm_with_multi_token_prediction_and_eval_head():
+    """The fused norm composes with the other options: multi-token prediction in training, the vocabulary slice in
+    evaluation.  Reference: the same calls on torch's own rms_norm output (bit-identical to the fused norm for bf16)."""
+    import torch.nn.functional as F
+    from slowrun_amd.cuda_kernels import (FusedNormSoftcappedCrossEntropy, FusedSoftcappedCrossEntropy,
+                                          softcapped_cross_entropy)
+    inp = _small("tiny_track", 900, 128, 1300)
+    N, d, V = inp.shape
+    gen = torch.Generator().manual_seed(11)
+    h0 = (inp.x * (0.3 + 3.0 * torch.rand(N, 1, generator=gen))).bfloat16().cuda()
+    w0 = inp.w.bfloat16().cuda()
+    y = inp.targets.cuda()
+    y[::9] = -1
+    x_s = float(F.rms_norm(h0, (d,)).float().abs().max()) / 448.0
+    mw = torch.tensor([1.0, 0.6, 0.3], device="cuda")
+    res = []
+    for fused in (True, False):
+        h = h0.clone().requires_grad_(True)
+        w = w0.clone().requires_grad_(True)
+        if fused:
+            losses = FusedNormSoftcappedCrossEntropy.apply(h, y, mw, w, x_s, inp.w_s, 0.0, 1.0)
+        else:
+            losses = FusedSoftcappedCrossEntropy.apply(F.rms_norm(h, (d,)), y, mw, w, x_s, inp.w_s, 0.0, 1.0)
+        losses.mean().backward()
+        res.append((losses.detach(), h.grad, w.grad))
+    assert torch.equal(res[0][0], res[1][0])                  # same fp8 bytes in, same kernels: same losses
+    assert torch.equal(res[0][2], res[1][2])                  # and the same dW
+    assert pu.maxrel(res[0][1].float(), res[1][1].float()) < 1e-2 and pu.cosine(res[0][1].float(), res[1][1].float()) > 0.99999
+    ev_fused = softcapped_cross_entropy(h0, w0, y, x_s, inp.w_s, vocab_size=1250, reduction="none",
+                                        norm_eps=torch.finfo(torch.float32).eps)
+    ev_plain = softcapped_cross_entropy(F.rms_norm(h0, (d,)), w0, y, x_s, inp.w_s, vocab_size=1250, reduction="none")
+    assert torch.equal(ev_fused, ev_plain)
