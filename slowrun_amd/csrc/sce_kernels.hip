@@ -850,6 +850,10 @@ struct DxParams {
 
 // Row scale and one-hot term of four consecutive dX columns j..j+3 of panel row il:
 //   dX = rho_i w_s (G W_q^T) - sum_k h_ik w_s W_q^T[y_{i+k}, :]
+// LDS a wave uses to stage its quadrant of a dX tile on the way out: 128 rows of 64 fp32 (or bf16) plus 16 bytes
+constexpr int DX_STAGE_BYTES = 128 * (64 * 4 + 16);
+constexpr int SMEM_DX = 4 * DX_STAGE_BYTES > SMEM_BYTES ? 4 * DX_STAGE_BYTES : SMEM_BYTES;
+
 struct DxRowTerms {
   float rs;
   float hs[4];
@@ -868,13 +872,14 @@ struct DxRowTerms {
   }
   template <typename T>
   __device__ __forceinline__ void store4(const DxParams& p, T* dst, int j, float o0, float o1, float o2, float o3) const {
-    o0 *= rs; o1 *= rs; o2 *= rs; o3 *= rs;
+    // explicit roundings: the fast path of bwd_dx_kernel forms the same values and must give the same bits
+    o0 = __fmul_rn(o0, rs); o1 = __fmul_rn(o1, rs); o2 = __fmul_rn(o2, rs); o3 = __fmul_rn(o3, rs);
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       if (k < p.n_predict) {
         const uint32_t w = *reinterpret_cast<const uint32_t*>(wrow[k] + j);
-        o0 -= hs[k] * e4m3_to_float<0>(w); o1 -= hs[k] * e4m3_to_float<1>(w);
-        o2 -= hs[k] * e4m3_to_float<2>(w); o3 -= hs[k] * e4m3_to_float<3>(w);
+        o0 = __builtin_fmaf(-hs[k], e4m3_to_float<0>(w), o0); o1 = __builtin_fmaf(-hs[k], e4m3_to_float<1>(w), o1);
+        o2 = __builtin_fmaf(-hs[k], e4m3_to_float<2>(w), o2); o3 = __builtin_fmaf(-hs[k], e4m3_to_float<3>(w), o3);
       }
     }
     Elem<T>::store(dst + 0, o0); Elem<T>::store(dst + 1, o1);
@@ -908,6 +913,97 @@ __global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p) {
                                                     2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave), NoHook(), 128 * BK, bpair);
   const int jbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
   T* dx = reinterpret_cast<T*>(p.dx);
+  if (!SPLIT && p.n_predict == 1) {
+    // One wave per SIMD has nothing to hide a load behind, so the epilogue is written in three phases with all
+    // loads of a phase in flight together: the row terms of the lane's four rows, then the 64 words of the four
+    // W_q^T rows of their targets, then arithmetic and stores.
+    float rs[4], hs[4];
+    int64_t yy[4];
+    int il4[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int il = rt * 256 + wb * 128 + b * 32 + (lane & 31);
+      const bool live = il < p.rows;
+      il4[b] = live ? il : -1;
+      const int is = live ? il : 0;                       // row 0 exists whenever any row does
+      rs[b] = p.rho[is] * p.w_s;
+      hs[b] = p.hcoef[is] * p.w_s;
+      yy[b] = p.targets[is];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    uint32_t wv[4][16];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const bool hit = il4[b] >= 0 && hs[b] != 0.f && yy[b] >= 0 && yy[b] < p.V;
+      if (!hit) hs[b] = 0.f;
+      const uint8_t* wrow = p.wqt + (hit ? yy[b] : 0) * p.ldx + jbase;
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) wv[b][4 * a + q] = *reinterpret_cast<const uint32_t*>(wrow + a * 32 + 8 * q);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // Out through LDS (free now: every wave is past the closing barrier of the main loop), so that the stores are
+    // whole 16-byte runs of a row instead of 8-byte pieces of 32 different rows: each wave stages its own quadrant,
+    // 64 columns at a time, and reads only what it wrote itself (no barrier).
+    const bool vec = ((reinterpret_cast<uintptr_t>(p.dx) | (uintptr_t)(p.dx_ld * (int64_t)sizeof(T))) & 15) == 0;
+    if (vec) {
+      constexpr int RB = 64 * (int)sizeof(T), PITCH = RB + 16, CH = RB / 16;     // row bytes, staging pitch, chunks per row
+      uint8_t* stg = smem + wave * DX_STAGE_BYTES;
+#pragma unroll
+      for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          uint8_t* srow = stg + (b * 32 + (lane & 31)) * PITCH + 4 * (lane >> 5) * (int)sizeof(T);
+#pragma unroll
+          for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int a = 2 * pass + a2;
+              const uint32_t w = wv[b][4 * a + q];
+              const float o0 = __builtin_fmaf(-hs[b], e4m3_to_float<0>(w), __fmul_rn(acc[a][b][4 * q + 0], rs[b]));
+              const float o1 = __builtin_fmaf(-hs[b], e4m3_to_float<1>(w), __fmul_rn(acc[a][b][4 * q + 1], rs[b]));
+              const float o2 = __builtin_fmaf(-hs[b], e4m3_to_float<2>(w), __fmul_rn(acc[a][b][4 * q + 2], rs[b]));
+              const float o3 = __builtin_fmaf(-hs[b], e4m3_to_float<3>(w), __fmul_rn(acc[a][b][4 * q + 3], rs[b]));
+              uint8_t* dst = srow + (a2 * 32 + 8 * q) * (int)sizeof(T);
+              if constexpr (sizeof(T) == 2)
+                *reinterpret_cast<v2i*>(dst) = (v2i){(int)((uint32_t)float_to_bf16_bits(o0) | ((uint32_t)float_to_bf16_bits(o1) << 16)),
+                                                     (int)((uint32_t)float_to_bf16_bits(o2) | ((uint32_t)float_to_bf16_bits(o3) << 16))};
+              else
+                *reinterpret_cast<v4f*>(dst) = (v4f){o0, o1, o2, o3};
+            }
+        }
+#pragma unroll
+        for (int n = 0; n < 128 * CH / 64; ++n) {
+          const int c = lane + 64 * n, row = c / CH, k16 = c % CH;
+          const int il = rt * 256 + wb * 128 + row;
+          const int col = ct * 256 + wa * 128 + pass * 64 + k16 * (16 / (int)sizeof(T));
+          if (il < p.rows && col < p.d)
+            *reinterpret_cast<v4i*>(reinterpret_cast<uint8_t*>(dx) + ((int64_t)il * p.dx_ld + col) * (int64_t)sizeof(T)) =
+                *reinterpret_cast<const v4i*>(stg + row * PITCH + k16 * 16);
+        }
+      }
+      return;
+    }
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      if (il4[b] < 0) continue;
+      T* drow = dx + (int64_t)il4[b] * p.dx_ld;
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int j = jbase + a * 32 + 8 * q;
+          if (j >= p.d) continue;                       // d is a multiple of 4, so j..j+3 are in range together
+          const uint32_t w = wv[b][4 * a + q];
+          Elem<T>::store(drow + j + 0, __builtin_fmaf(-hs[b], e4m3_to_float<0>(w), __fmul_rn(acc[a][b][4 * q + 0], rs[b])));
+          Elem<T>::store(drow + j + 1, __builtin_fmaf(-hs[b], e4m3_to_float<1>(w), __fmul_rn(acc[a][b][4 * q + 1], rs[b])));
+          Elem<T>::store(drow + j + 2, __builtin_fmaf(-hs[b], e4m3_to_float<2>(w), __fmul_rn(acc[a][b][4 * q + 2], rs[b])));
+          Elem<T>::store(drow + j + 3, __builtin_fmaf(-hs[b], e4m3_to_float<3>(w), __fmul_rn(acc[a][b][4 * q + 3], rs[b])));
+        }
+    }
+    return;
+  }
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
     const int il = rt * 256 + wb * 128 + b * 32 + (lane & 31);
@@ -1228,10 +1324,10 @@ static int check_device(int dev) {
       // the MFMA kernels hold two 64 KB K-slots in LDS
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_recompute_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_RECOMPUTE));
-      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
-      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
-      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
-      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_DX));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_DX));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_DX));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_DX));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
     }
@@ -1632,15 +1728,15 @@ extern "C" int sce_backward(const sce_args* a) {
       const bool f32 = a->dx_dtype == SCE_F32;
       dp_.dx = f32 ? (void*)((float*)a->dx + p0 * a->dx_ld) : (void*)((bf16_t*)a->dx + p0 * a->dx_ld);
       if (ksplit == 1) {
-        if (f32) bwd_dx_kernel<float, false><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_BYTES, st>>>(dp_);
-        else bwd_dx_kernel<bf16_t, false><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_BYTES, st>>>(dp_);
+        if (f32) bwd_dx_kernel<float, false><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_DX, st>>>(dp_);
+        else bwd_dx_kernel<bf16_t, false><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_DX, st>>>(dp_);
       } else if (dp_.rows > 0) {
         const int fgrid = (int)(((int64_t)dp_.rows * (d / 4) + 255) / 256);
         if (f32) {
-          bwd_dx_kernel<float, true><<<map_tile_grid(RTp, CTd * ksplit), NTHREADS, SMEM_BYTES, st>>>(dp_);
+          bwd_dx_kernel<float, true><<<map_tile_grid(RTp, CTd * ksplit), NTHREADS, SMEM_DX, st>>>(dp_);
           bwd_dx_finish_kernel<float><<<fgrid, 256, 0, st>>>(dp_);
         } else {
-          bwd_dx_kernel<bf16_t, true><<<map_tile_grid(RTp, CTd * ksplit), NTHREADS, SMEM_BYTES, st>>>(dp_);
+          bwd_dx_kernel<bf16_t, true><<<map_tile_grid(RTp, CTd * ksplit), NTHREADS, SMEM_DX, st>>>(dp_);
           bwd_dx_finish_kernel<bf16_t><<<fgrid, 256, 0, st>>>(dp_);
         }
       }
