@@ -20,7 +20,7 @@ PEAK_FP8_TFLOPS = 5000.0        # MI355X dense fp8 MFMA, published
 # HBM-side bytes per launch (fetched + written) of the MFMA kernels at the full limited_2p7b shape, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB device copy (factors 2.0 / 1.0); the
 # summary is profiles/bench_limited_2p7b_pmc.txt.  None for any other workload.
-MEASURED_TRAFFIC_GIB = {"fwd": 17.638 + 0.008, "recompute": 1.481 + 0.284, "dx": 1.339 + 0.031, "dw": 13.687 + 0.481}
+MEASURED_TRAFFIC_GIB = {"fwd": 16.645 + 0.008, "recompute": 1.487 + 0.284, "dx": 1.331 + 0.031, "dw": 13.540 + 0.481}
 
 
 def cpu_baseline(inp, rows, threads):
