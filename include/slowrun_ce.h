@@ -45,7 +45,7 @@ enum {
 
 typedef struct sce_shape {
   int64_t N;           /* rows (tokens)                         */
-  int64_t d;           /* hidden size, multiple of 16           */
+  int64_t d;           /* hidden size, multiple of 16, < 2^22   */
   int64_t V;           /* vocabulary (columns of W); N, d, V < 2^24 */
   int32_t n_predict;   /* number of MTP offsets, 1..4           */
   int32_t reserved;

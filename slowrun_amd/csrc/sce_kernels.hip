@@ -1343,6 +1343,7 @@ static int check_shape(const sce_shape* s) {
   if (s->d % 16 != 0) return fail(SCE_EINVAL, "d = %lld must be a multiple of 16", (long long)s->d);
   if (s->N > (1ll << 24) - 256 || s->V > (1ll << 24) - 256 || s->d > (1ll << 24) - 256)
     return fail(SCE_EINVAL, "N, d and V must be below 2^24 (32-bit tile offsets)");
+  if (s->d > (1ll << 22) - 256) return fail(SCE_EINVAL, "d = %lld must be below 2^22 (a grid dimension of the layout kernels)", (long long)s->d);
   if (s->n_predict < 1 || s->n_predict > 4) return fail(SCE_EINVAL, "n_predict = %d must be between 1 and 4", s->n_predict);
   return SCE_OK;
 }
