@@ -74,9 +74,10 @@ def check_parity(ours, ref, reduction="mean", check_argmax=True, grad_maxrel=GRA
         # Bit-exact except on genuine near-ties: fp8 x fp8 products are exact in fp32, so two correct
         # evaluations differ only by the order of the fp32 accumulation.  A differing row is accepted
         # only if, with the logits recomputed exactly (float64 sums of exact products), our argmax is
-        # within the accumulation error of the true maximum: 32 * 2^-24 * sum_k |x_k w_k| (the MFMA's
-        # fp32 accumulation was measured at up to ~12 * 2^-24 of that sum; a gap of this size is a few
-        # parts in 10^6 of the logit).  The number of such rows is reported.
+        # within the accumulation error of the true maximum: 64 * 2^-24 * sum_k |x_k w_k| (two values are
+        # involved, and the MFMA's fp32 accumulation was measured at up to ~23 * 2^-24 of that sum on each,
+        # over 3e8 logits; a gap of this size is a few parts in 10^6 of the logit scale).  The number of such
+        # rows is reported.
         mism = (ours["argmax"].long() != ref["argmax"]).nonzero().flatten()
         report["argmax_near_ties"] = int(mism.numel())
         if mism.numel():
@@ -84,7 +85,7 @@ def check_parity(ours, ref, reduction="mean", check_argmax=True, grad_maxrel=GRA
             xq = eager.dequantize(eager.quantize_e4m3(ours["x"][mism], inp_scales(ours)[0]), inp_scales(ours)[0]).double()
             wq = eager.dequantize(eager.quantize_e4m3(ours["w"], inp_scales(ours)[1]), inp_scales(ours)[1]).double()
             u = xq @ wq
-            bound = 32 * 2.0 ** -24 * (xq.abs() @ wq.abs()).max(dim=1).values
+            bound = 64 * 2.0 ** -24 * (xq.abs() @ wq.abs()).max(dim=1).values
             got = u.gather(1, ours["argmax"][mism].long()[:, None])[:, 0]
             assert bool((got >= u.max(dim=1).values - bound).all()), "argmax differs on a row that is not a near-tie"
     return report

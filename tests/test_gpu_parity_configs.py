@@ -59,3 +59,15 @@ def test_irregular_full():
     assert torch.equal(ours2["lse"], ours["lse"][permd])
     assert torch.equal(ours2["dx"], ours["dx"][permd])
     assert pu.maxrel(ours2["dw"].float(), ours["dw"].float()) < 1e-2 and pu.cosine(ours2["dw"].float(), ours["dw"].float()) > 0.99999
+
+
+def test_more_rows_than_one_dw_window():
+    """N beyond the 131072 rows that one dW launch contracts over: dlogits are produced and consumed in two windows,
+    dW is the sum of two partials (and with a smaller workspace the second launch accumulates into the first)."""
+    inp = configs.make_inputs("tiny_track", N=150011, d=256, V=2048)
+    ours = pu.run_ours(inp, "mean")
+    ref = pu.run_oracle(inp, ours, "mean", row_chunk=16384)
+    print(pu.check_parity(ours, ref, "mean"))
+    from slowrun_amd import _lib
+    sz = _lib.sizes_for(*inp.shape)
+    assert sz.bwd_workspace_min_bytes < sz.bwd_workspace_bytes
