@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SCE_VERSION 3
+#define SCE_VERSION 4
 
 enum { SCE_F32 = 0, SCE_BF16 = 1 };               /* element types of X, W, dX, dW          */
 enum { SCE_REDUCE_NONE = 0, SCE_REDUCE_MEAN = 1 }; /* F.cross_entropy(reduction=...)         */
@@ -72,7 +72,11 @@ typedef struct sce_args {
   const void* w;  int32_t w_dtype;  int32_t pad1;  int64_t w_ld;   /* (d,V), row stride in elements */
   const int64_t* targets;    /* (N,)                                                         */
   const float* mtp_weights;  /* (n_predict,) on the device, or NULL for a single weight 1    */
-  float x_s, w_s;            /* fp8 scales: X_q = e4m3(X / x_s), W_q = e4m3(W / w_s)         */
+  double x_s, w_s;           /* fp8 scales: X_q = e4m3(X / x_s), W_q = e4m3(W / w_s).  Doubles, as the Python
+                                floats of the reference's call are (tiny/train.py:188-189): the quantiser
+                                multiplies by (float)(1.0 / x_s), the dequantiser by (float)x_s, which is
+                                what torch's GPU kernels make of x.div(x_s) and of the scales of
+                                _scaled_mm (tiny/cuda_kernels.py:340-350)                                   */
   float cap;                 /* z = cap * tanh(u / cap), 0 < cap <= 40                       */
   float grad_scale;          /* multiplies every gradient (tiny/cuda_kernels.py:265)         */
   int64_t ignore_index;
@@ -121,11 +125,14 @@ const char* sce_last_error(void);
  * FusedSoftcappedCrossEntropy.forward/backward (tiny/cuda_kernels.py:359-366,398-401). */
 int sce_sizes_for(const sce_shape* shape, sce_sizes* out);
 
-/* Per-tensor scaled cast to OCP e4m3: dst[i] = e4m3_rne(src[i] / scale), NaN code above
- * 464 like Tensor.to(float8_e4m3fn); bf16 input is divided in fp32 and rounded to bf16
- * first, as torch does.  Replaces x.div(x_s).to(torch.float8_e4m3fn)
- * (tiny/cuda_kernels.py:340-341). */
-int sce_quantize_e4m3(const void* src, int32_t src_dtype, void* dst, float scale, size_t n,
+/* Per-tensor scaled cast to OCP e4m3: dst[i] = e4m3_rne(src[i] * (float)(1.0 / scale)), NaN code
+ * above 464 like Tensor.to(float8_e4m3fn).  The reciprocal is taken once, in double, rounded to
+ * fp32 and multiplied in: this is how torch's GPU kernels divide a tensor by a host scalar (its
+ * CPU kernels divide element by element; the results differ in the last bit now and then, and
+ * that can move an fp8 tie); bf16 input is scaled in fp32 and rounded to bf16 first, as torch
+ * does.  sce_forward quantises X and W the same way.  Replaces
+ * x.div(x_s).to(torch.float8_e4m3fn) (tiny/cuda_kernels.py:340-341), which runs on the GPU. */
+int sce_quantize_e4m3(const void* src, int32_t src_dtype, void* dst, double scale, size_t n,
                       int32_t device, void* stream);
 
 /* dst (cols, rows) = transpose of src (rows, cols), one byte per element.  Replaces

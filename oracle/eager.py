@@ -28,7 +28,12 @@ IGNORE_INDEX = -1
 
 
 def quantize_e4m3(t, scale):
-    """tiny/cuda_kernels.py:340-341 - per-tensor scaled, RNE, non-saturating."""
+    """tiny/cuda_kernels.py:340-341 - per-tensor scaled, RNE, non-saturating.
+
+    The library's own division: for a Python-float scale torch's GPU kernels compute t * (1 / scale) with the
+    reciprocal taken once in fp32, its CPU kernels divide element by element.  The two differ in the last bit for
+    about one value in 10^5, which matters only where the quotient lands on an fp8 rounding tie; the reference
+    runs this line on the GPU."""
     return t.div(scale).to(torch.float8_e4m3fn)
 
 

@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(HERE, "libslowrun_ce.so")
 
 SCE_F32, SCE_BF16 = 0, 1
 SCE_REDUCE_NONE, SCE_REDUCE_MEAN = 0, 1
-SCE_VERSION = 3
+SCE_VERSION = 4
 
 EXPORTS = ("sce_version", "sce_last_error", "sce_sizes_for", "sce_quantize_e4m3", "sce_transpose_bytes",
            "sce_forward", "sce_backward", "sce_timing_enable", "sce_timing_read")
@@ -36,7 +36,7 @@ class SceArgs(C.Structure):
         ("x", C.c_void_p), ("x_dtype", C.c_int32), ("pad0", C.c_int32), ("x_ld", C.c_int64),
         ("w", C.c_void_p), ("w_dtype", C.c_int32), ("pad1", C.c_int32), ("w_ld", C.c_int64),
         ("targets", C.c_void_p), ("mtp_weights", C.c_void_p),
-        ("x_s", C.c_float), ("w_s", C.c_float), ("cap", C.c_float), ("grad_scale", C.c_float),
+        ("x_s", C.c_double), ("w_s", C.c_double), ("cap", C.c_float), ("grad_scale", C.c_float),
         ("ignore_index", C.c_int64), ("reduction", C.c_int32), ("pad2", C.c_int32),
         ("loss", C.c_void_p), ("losses", C.c_void_p), ("lse", C.c_void_p), ("argmax", C.c_void_p), ("n_valid", C.c_void_p),
         ("saved", C.c_void_p), ("saved_bytes", C.c_size_t), ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
@@ -68,7 +68,7 @@ def lib():
         L.sce_version.restype = C.c_int
         L.sce_last_error.restype = C.c_char_p
         L.sce_sizes_for.argtypes = [C.POINTER(SceShape), C.POINTER(SceSizes)]
-        L.sce_quantize_e4m3.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_float, C.c_size_t, C.c_int32, C.c_void_p]
+        L.sce_quantize_e4m3.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_double, C.c_size_t, C.c_int32, C.c_void_p]
         L.sce_transpose_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int32, C.c_void_p]
         L.sce_forward.argtypes = [C.POINTER(SceArgs)]
         L.sce_backward.argtypes = [C.POINTER(SceArgs)]

@@ -62,14 +62,16 @@ template <typename T> struct Elem;
 template <> struct Elem<float> {
   static __device__ __forceinline__ float load(const float* p) { return *p; }
   static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
-  static __device__ __forceinline__ float div_round(float x, float s) { return x / s; }
+  // x.div(s) with a host scalar s as torch's GPU kernels compute it: x * (1 / s), the reciprocal taken once in fp32
+  // (the CPU kernels divide; the two differ in the last bit now and then, which moves an fp8 tie)
+  static __device__ __forceinline__ float div_round(float x, float inv_s) { return x * inv_s; }
 };
 struct bf16_t { uint16_t bits; };
 template <> struct Elem<bf16_t> {
   static __device__ __forceinline__ float load(const bf16_t* p) { return bf16_bits_to_float(p->bits); }
   static __device__ __forceinline__ void store(bf16_t* p, float v) { p->bits = float_to_bf16_bits(v); }
-  // torch divides a bf16 tensor in fp32 and rounds the quotient back to bf16 before the fp8 cast
-  static __device__ __forceinline__ float div_round(float x, float s) { return round_to_bf16(x / s); }
+  // torch scales a bf16 tensor in fp32 and rounds the result back to bf16 before the fp8 cast
+  static __device__ __forceinline__ float div_round(float x, float inv_s) { return round_to_bf16(x * inv_s); }
 };
 
 // XCD-aware tile order.  Consecutive workgroup ids go round-robin to the 8 XCDs, each with its
@@ -112,10 +114,10 @@ static inline int map_tile_rr_grid(int RT, int CT) { return 256 * ((RT * CT + 25
 // ------------------------------------------------------------------------------------------
 // quantisation
 // ------------------------------------------------------------------------------------------
-// 16 consecutive elements starting at p as floats after the scaled division; elements at or beyond
+// 16 consecutive elements starting at p as floats after the scaling by 1 / s; elements at or beyond
 // `valid` are 0.  One or two 16/32-byte vector loads when the run is complete and 16-byte aligned.
 template <typename T>
-__device__ __forceinline__ void load16_scaled(const T* __restrict__ p, int64_t valid, float scale, float (&v)[16]) {
+__device__ __forceinline__ void load16_scaled(const T* __restrict__ p, int64_t valid, float scale, float (&v)[16]) {     // scale: 1 / s
   if (valid >= 16 && (((uintptr_t)p) & 15) == 0) {
     if constexpr (sizeof(T) == 2) {
       const v4i r0 = *reinterpret_cast<const v4i*>(p), r1 = *reinterpret_cast<const v4i*>(p + 8);
@@ -140,7 +142,8 @@ __device__ __forceinline__ void load16_scaled(const T* __restrict__ p, int64_t v
   }
 }
 
-// dst [rows_p][cols_p] e4m3 = src [rows][cols] / scale, zero outside; 16 outputs per thread.
+// dst [rows_p][cols_p] e4m3 = src [rows][cols] * scale, zero outside; 16 outputs per thread.  In all the
+// quantising kernels `scale` is the reciprocal 1 / s of the fp8 scale s, taken once on the host.
 template <typename T>
 __global__ __launch_bounds__(256) void quantize_pad_kernel(const T* __restrict__ src, int64_t ld, int64_t rows,
                                                           int64_t cols, uint8_t* __restrict__ dst,
@@ -187,7 +190,7 @@ __global__ __launch_bounds__(256) void rmsnorm_quantize_kernel(const T* __restri
   float ss = 0.f;
   for (int64_t c = lane; c * 16 < cols; c += 64) {
     float v[16];
-    load16_scaled<T>(row + c * 16, cols - c * 16, 1.0f, v);      // a division by 1 is exact: the values themselves
+    load16_scaled<T>(row + c * 16, cols - c * 16, 1.0f, v);      // scaling by 1 is exact: the values themselves
 #pragma unroll
     for (int m = 0; m < 16; ++m) ss = fmaf(v[m], v[m], ss);
   }
@@ -634,40 +637,53 @@ __global__ __launch_bounds__(1024) void fwd_reduce_kernel(const float4* __restri
 // ------------------------------------------------------------------------------------------
 // backward
 // ------------------------------------------------------------------------------------------
-// per row: c_row (exponent offset of G), rho (row scale of G), h_k (one-hot coefficients).
-//   dz_iv = g_i ( S_i p_iv - sum_k w_k [v = y_{i+k}] ),  S_i = sum of w_k over the offsets that take part.
-__global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__ s_lse, const float* __restrict__ s_umax,
+// per row: rho (row factor of the block-scaled dlogits) and h_k (one-hot coefficients).
+//   dz_iv = g_i ( S_i p_iv - sum_k w_k [v = y_{i+k}] ),  S_i = sum of w_k over the offsets that take part,
+//   S_i p_iv (1 - t^2) = rho_i D_iv  with  rho_i = g_i S_i e^{cap - lse_i}.
+// The target columns take no part in D (bwd_zero_targets_kernel clears them): their S_i p_iy goes into the
+// one-hot coefficient instead, h_ik = g_i (1 - t_y^2) (w_k - S_i p_iy), formed here in fp32 from lse and z_y.
+// Through e4m3 the difference S_i p_iy - w_k would carry the rounding error of p_iy alone, a relative
+// error of eps p / (1 - p) that grows without bound on rows the model is sure of.  When two offsets of a row
+// have the same target, the first one carries the S_i p_iy term.
+__global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__ s_lse,
                                                       const float* __restrict__ s_zy, const int64_t* __restrict__ targets,
                                                       int64_t ignore_index, const int32_t* __restrict__ hdr,
                                                       const float* __restrict__ grad_output, int per_row, float grad_scale,
                                                       const float* __restrict__ mtp_weights, int n_predict,
-                                                      float cap, int N, int Np, int V, float* __restrict__ crow,
+                                                      float cap, int N, int Np, int V,
                                                       float* __restrict__ rho, float* __restrict__ hcoef,
                                                       float* __restrict__ blockmax) {
   __shared__ float smax[256];
   const int i = blockIdx.x * 256 + threadIdx.x;
-  float c = -INFINITY, r = 0.f;
+  float r = 0.f;
   float h[4] = {0.f, 0.f, 0.f, 0.f};
   if (i < N) {
     const float g = (per_row ? grad_output[i] : grad_output[0] / (float)hdr[0]) * grad_scale;
     float sw = 0.f;
-    bool any = false;
+    bool ok[4] = {false, false, false, false};
+    int64_t yk[4] = {0, 0, 0, 0};
     for (int k = 0; k < n_predict; ++k) {
-      if (!target_valid(targets, ignore_index, i + k, N, V)) continue;
-      const float wk = mtp_weights ? mtp_weights[k] : 1.0f;
-      const float ty = s_zy[(int64_t)k * Np + i] / cap;
-      h[k] = g * wk * (1.0f - ty * ty);
-      sw += wk;
-      any = true;
+      ok[k] = target_valid(targets, ignore_index, i + k, N, V);
+      if (!ok[k]) continue;
+      yk[k] = targets[i + k];
+      sw += mtp_weights ? mtp_weights[k] : 1.0f;
     }
-    if (any) {
-      const float zmax = cap * tanhf(s_umax[i] / cap);
-      c = (cap - zmax) * LOG2E + 10.0f;        // G = 2^c * r(1-r) * e^{z-cap} = 256 (1-t^2) e^{z-zmax}
-      r = g * sw * expf(zmax - s_lse[i]) * (1.0f / 256.0f);
+    if (ok[0] || ok[1] || ok[2] || ok[3]) {
+      const float lse = s_lse[i];
+      for (int k = 0; k < n_predict; ++k) {
+        if (!ok[k]) continue;
+        const float wk = mtp_weights ? mtp_weights[k] : 1.0f;
+        const float zy = s_zy[(int64_t)k * Np + i];
+        const float ty = zy / cap;
+        bool first = true;
+        for (int k2 = 0; k2 < k; ++k2) first = first && !(ok[k2] && yk[k2] == yk[k]);
+        h[k] = g * (1.0f - ty * ty) * (wk - (first ? sw * expf(zy - lse) : 0.f));
+      }
+      r = g * sw * expf(cap - lse);
     }
   }
   if (i < Np) {
-    crow[i] = c; rho[i] = r;
+    rho[i] = r;
     for (int k = 0; k < n_predict; ++k) hcoef[(int64_t)k * Np + i] = h[k];
   }
   smax[threadIdx.x] = fabsf(r);
@@ -677,6 +693,18 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__
     __syncthreads();
   }
   if (threadIdx.x == 0) blockmax[blockIdx.x] = smax[0];
+}
+
+// Clears the target columns of the rows [i0, i0 + rows) in G^T (blocked; `g` points at the K block of row i0):
+// one thread per (offset, row) pair, one byte each.  Runs between the kernel that forms G and its readers.
+__global__ __launch_bounds__(256) void bwd_zero_targets_kernel(const int64_t* __restrict__ targets, int64_t ignore_index,
+                                                              int i0, int rows, int N, int V, int n_predict,
+                                                              uint8_t* __restrict__ g, int64_t kbw) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= rows * n_predict) return;
+  const int k = e / rows, il = e - k * rows;
+  if (!target_valid(targets, ignore_index, i0 + il + k, N, V)) return;
+  g[blocked_offset(targets[i0 + il + k], il, kbw)] = 0;
 }
 
 __global__ __launch_bounds__(1024) void bwd_xi_kernel(const float* __restrict__ blockmax, int n, float* __restrict__ xi) {
@@ -724,25 +752,156 @@ __global__ __launch_bounds__(256) void bwd_xt_kernel(const uint8_t* __restrict__
   *reinterpret_cast<v4i*>(xt + blocked_offset(j0 + jr, i0 + ic, kbn)) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
 }
 
+// ------------------------------------------------------------------------------------------
+// dlogits on chip
+// ------------------------------------------------------------------------------------------
+// The softmax part of dlogits, without the factors that belong to a whole row, is
+//   D_iv = (1 - t^2) e^{z - cap} = 4 r (1 - r) e^{z - cap},  r = 1 / (1 + e^{2u/cap}),   0 <= D <= 1,
+// and  du_iv = rho_i D_iv - (one-hot terms),  rho_i = g_i S_i e^{cap - lse_i}.  D is kept in e4m3 with one power-of-two
+// exponent per block of 32 rows i x 128 columns v (MX style: byte * 2^(E - 127), E in an E8M0 byte), taken from the
+// block's own largest logit, so that neither the row's final lse nor its maximum has to be known when the block is
+// formed -- the forward pass can emit it -- and a peak in one place of a row costs the rest of the row nothing.  The
+// dX and dW GEMMs apply the exponents inside the matrix instruction (mfma_mainloop, SCALE).
+//
+// Layout: G^T, tile by tile ([v tile][K block of 128 rows i][256 v][128 i] bytes): the B operand of dW as it lies,
+// and of dX through the transposing LDS read.  Exponents: one dword per (128 v, 128 i), byte c for rows [32 c, 32 c + 32),
+// as gexp[v / 128][i / 128].
+//
+// One wave turns its 128 (v) x 128 (i) quadrant of a finished logit tile into its quadrant of the staging tile TT
+// ([256 v][STG_PITCH], rows i contiguous) in LDS and returns the dword of exponents of its four 32-row blocks.  The
+// transposition happens in registers: the four lanes of a quad hold four consecutive rows of the same four
+// columns, and two quad-permute + byte-permute steps turn that 4 x 4 byte block around.
+// STATS: the forward pass's row statistics as well (sum of e^{z - cap}, largest raw logit and its column), kept in
+// `stat` (LDS, 12 floats per lane: [sum, max, argmax][4 row blocks], NTHREADS apart).
+constexpr int STG_PITCH = 272;                               // 256 + 16: 16-byte aligned, rows shifted by 4 banks
+constexpr int STG_BYTES = 256 * STG_PITCH;                   // 69632
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+template <bool EDGE, bool STATS>
+__device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float k1, float c2, int vlim, int vabs0,
+                                                 uint8_t* TT, int wa, int wb, float* stat) {
+  const int lane = lane_id();
+  const int vloc0 = wa * 128 + 4 * (lane >> 5);       // column (within the tile) of accumulator register 0 of block a = 0
+  const int k = lane & 3;
+  const uint32_t sel1 = (k & 1) ? 0x03070105u : 0x06020400u;
+  const uint32_t sel2 = (k & 2) ? 0x03020706u : 0x05040100u;
+  uint32_t expword = 0;
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int iloc = wb * 128 + b * 32 + (lane & 31);        // row within the tile
+    // the block's largest logit fixes its exponent: D * 2^s <= 2^(lg + s) <= 446 with lg = log2 e^{zmax - cap}
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float x = acc[a][b][r];
+        if (EDGE && vloc0 + a * 32 + 8 * (r >> 2) + (r & 3) >= vlim) x = -INFINITY;
+        tmax = fmaxf(tmax, x);
+      }
+    const float bmax = wave_max(tmax);
+    const float lg = c2 * fast_rcp(1.0f + fast_exp2(bmax * k1));
+    const float sb = floorf(8.8f - lg);                       // 8 .. 8 + 2 cap log2(e): at most 124 for cap <= 40
+    const float cs = sb + 2.0f;                               // the 4 of 4 r (1 - r) rides along
+    expword |= (uint32_t)(127 - (int)sb) << (8 * b);
+    float ssum = 0.f;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      // stage by stage over the 16 values of the block: the transcendental unit is pipelined, a chain
+      // of dependent exp2 / rcp / exp2 on one value at a time is not (the scheduler would rebuild the
+      // chains to save registers, hence the barriers)
+      constexpr int NB = 8;        // values per batch: 4, 8 and 16 measure alike
+      float rr[16], gg[16];
+#pragma unroll
+      for (int g0 = 0; g0 < 16; g0 += NB) {
+#pragma unroll
+        for (int m = g0; m < g0 + NB; ++m) rr[m] = fast_exp2(acc[a][b][m] * k1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = g0; m < g0 + NB; ++m) rr[m] = fast_rcp(rr[m] + 1.0f);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = g0; m < g0 + NB; ++m) gg[m] = fast_exp2(fmaf(c2, rr[m], cs));
+        __builtin_amdgcn_sched_barrier(0);
+        if (EDGE) {
+#pragma unroll
+          for (int m = g0; m < g0 + NB; ++m) gg[m] = (vloc0 + a * 32 + 8 * (m >> 2) + (m & 3) >= vlim) ? 0.f : gg[m];
+        }
+        if (STATS) {
+#pragma unroll
+          for (int m = g0; m < g0 + NB; ++m) ssum += gg[m];
+        }
+#pragma unroll
+        for (int m = g0; m < g0 + NB; ++m) gg[m] *= rr[m] - rr[m] * rr[m];
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int vloc = vloc0 + a * 32 + 8 * q;
+        const uint32_t w = cvt4_e4m3(gg[4 * q], gg[4 * q + 1], gg[4 * q + 2], gg[4 * q + 3]);
+        // 4 x 4 byte transpose inside the quad: lane k ends up with column vloc + k, rows (iloc & ~3) .. +3
+        const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xB1, 0xF, 0xF, true);     // lane ^ 1
+        const uint32_t x = __builtin_amdgcn_perm(p1, w, sel1);
+        const uint32_t p2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, true);     // lane ^ 2
+        const uint32_t yv = __builtin_amdgcn_perm(p2, x, sel2);
+        *reinterpret_cast<uint32_t*>(TT + (vloc + k) * STG_PITCH + (iloc & ~3)) = yv;
+      }
+    }
+    if (STATS) {
+      stat[(0 + b) * NTHREADS] += ssum * fast_exp2(-cs);
+      const float amax = stat[(4 + b) * NTHREADS];
+      // the column of the maximum is looked up only when a tile raises a lane's running maximum
+      if (__builtin_amdgcn_ballot_w64(tmax > amax) != 0) {
+        if (tmax > amax) {
+          int targ = 0x7fffffff;
+#pragma unroll
+          for (int a = 3; a >= 0; --a) {
+#pragma unroll
+            for (int r = 15; r >= 0; --r) {
+              const int vo = a * 32 + 8 * (r >> 2) + (r & 3);
+              if (acc[a][b][r] == tmax && (!EDGE || vloc0 + vo < vlim)) targ = vo;   // descending scan: lowest column wins
+            }
+          }
+          stat[(4 + b) * NTHREADS] = tmax;
+          stat[(8 + b) * NTHREADS] = __int_as_float(vabs0 + targ);
+        }
+      }
+    }
+  }
+  return expword;
+}
+
+// The wave's quadrant of the staging tile (128 columns v x 128 rows i) is one contiguous 16 KB run of G^T: out in
+// 16-byte stores.  A wave reads only what it wrote itself, so no barrier is needed between forming and storing.
+__device__ __forceinline__ void store_dlogits_quadrant(const uint8_t* TT, uint8_t* gcol, int wa, int wb) {
+  const int lane = lane_id();
+  const uint8_t* tq = TT + wa * 128 * STG_PITCH + wb * 128;
+#pragma unroll
+  for (int n = 0; n < 16; ++n) {
+    const int cidx = lane + 64 * n, row = cidx >> 3, col = (cidx & 7) * 16;
+    *reinterpret_cast<v4i*>(gcol + row * BK + col) = *reinterpret_cast<const v4i*>(tq + row * STG_PITCH + col);
+  }
+}
+
 struct RecomputeParams {
   const uint8_t* xq;     // [Np][dp], already offset to the panel's first row
   const uint8_t* wqt;    // [Vp][dp]
-  const float* crow;     // offset to the panel's first row
-  uint8_t* ghat_t;       // Vp rows, K = Pw, blocked
+  uint8_t* ghat_t;       // Vp rows, K = 128 * kbw, blocked
+  uint32_t* gexp;        // [Vp / 128][kbw]
   int64_t dp, ldx;             // K extent and row stride of xq / wqt
   int64_t kbw, kb0;            // ghat_t (blocked): K blocks per tile, K block of this panel's first row
   int RT, CT, V;
   float k1, c2;          // as in FwdParams
 };
 
-// Recompute a 256 x 256 logit tile and leave G = 256 (1 - t^2) e^{z - zmax_row} in e4m3, transposed and tile by
-// tile ([v tile][K block of 128 rows i][256 v][128 i]): the operand layout of dW, which dX reads as well (its main
-// loop forms the fragments of G with the transposing LDS read).  The tile is assembled in LDS (free once the main
-// loop is done) and leaves the chip as 64 KB of consecutive 16-byte stores.  The transposition happens in registers:
-// the four lanes of a quad hold four consecutive rows of the same four columns, and two quad-permute + byte-permute
-// steps turn that 4 x 4 byte block around.
-constexpr int STG_PITCH = 272;                               // 256 + 16: 16-byte aligned, rows shifted by 4 banks
-constexpr int SMEM_RECOMPUTE = SMEM_BYTES + 2048;      // two K-block slots (the staging tile, 69632 B, reuses them) + 128 row constants per wave
+// Recompute a 256 x 256 logit tile and leave its block-scaled dlogits in G^T.  The tile is assembled in LDS (free
+// once the main loop is done) and leaves the chip as 64 KB of consecutive 16-byte stores.
+constexpr int SMEM_RECOMPUTE = SMEM_BYTES > STG_BYTES ? SMEM_BYTES : STG_BYTES;
 
 __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -752,88 +911,21 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   // the dX kernel that follows starts its K loop at column 0, with the part of G that was written last and is
   // still in the memory-side cache.
   ct = p.CT - 1 - ct;
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
-  // The row constants of the wave's 128 rows go straight to LDS, behind the two slots: requested before the
-  // K loop (whose waits for its own, younger loads cover them), read after it, no register held in between.
-  {
-    const int wu = __builtin_amdgcn_readfirstlane(wave);
-    const uint32_t dst = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)(smem + SMEM_BYTES)) + wu * 512;
-    const float* src = p.crow + rt * 256 + (wu & 1) * 128;
-    // the instruction's offset moves the memory address and the LDS address alike: the second half of the rows
-    asm volatile("s_add_u32 m0, %0, 0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n\t"
-                 "global_load_lds_dword %1, %2 offset:256"
-                 ::"s"(dst), "v"(lane * 4), "s"(src) : "memory", "scc");
-  }
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
-  mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave));
-  uint8_t* TT = smem;                        // [256 columns v][STG_PITCH]: rows i contiguous
-  const int vloc0 = wa * 128 + 4 * (lane >> 5);
-  const bool edge = ct * 256 + 256 > p.V;
+  mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 2 * (rt & 3), ct & 7, wave);
   const int vlim = p.V - ct * 256;           // columns >= vlim of this tile do not exist
-  const int k = lane & 3;
-  const uint32_t sel1 = (k & 1) ? 0x03070105u : 0x06020400u;
-  const uint32_t sel2 = (k & 2) ? 0x03020706u : 0x05040100u;
-  auto form_g = [&](auto edge_tag) {
-    constexpr bool EDGE = decltype(edge_tag)::value;
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      const int iloc = wb * 128 + b * 32 + (lane & 31);        // row within the tile
-      const float c = *reinterpret_cast<const float*>(smem + SMEM_BYTES + wave * 512 + (b * 32 + (lane & 31)) * 4);
-#pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        // stage by stage over the 16 values of the block: the transcendental unit is pipelined, a chain
-        // of dependent exp2 / rcp / exp2 on one value at a time is not (the scheduler would rebuild the
-        // chains to save registers, hence the barriers)
-        constexpr int NB = 8;        // values per batch: 4, 8 and 16 measure alike
-        float rr[16], gg[16];
-#pragma unroll
-        for (int g0 = 0; g0 < 16; g0 += NB) {
-#pragma unroll
-          for (int m = g0; m < g0 + NB; ++m) rr[m] = fast_exp2(acc[a][b][m] * p.k1);
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int m = g0; m < g0 + NB; ++m) rr[m] = fast_rcp(rr[m] + 1.0f);
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int m = g0; m < g0 + NB; ++m) gg[m] = fast_exp2(fmaf(p.c2, rr[m], c));
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int m = g0; m < g0 + NB; ++m) gg[m] *= rr[m] - rr[m] * rr[m];
-          __builtin_amdgcn_sched_barrier(0);
-        }
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int vloc = vloc0 + a * 32 + 8 * q;
-          if (EDGE) {
-#pragma unroll
-            for (int m = 0; m < 4; ++m) gg[4 * q + m] = (vloc + m >= vlim) ? 0.f : gg[4 * q + m];
-          }
-          const uint32_t w = cvt4_e4m3(gg[4 * q], gg[4 * q + 1], gg[4 * q + 2], gg[4 * q + 3]);
-          // 4 x 4 byte transpose inside the quad: lane k ends up with column vloc + k, rows (iloc & ~3) .. +3
-          const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xB1, 0xF, 0xF, true);     // lane ^ 1
-          const uint32_t x = __builtin_amdgcn_perm(p1, w, sel1);
-          const uint32_t p2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, true);     // lane ^ 2
-          const uint32_t yv = __builtin_amdgcn_perm(p2, x, sel2);
-          *reinterpret_cast<uint32_t*>(TT + (vloc + k) * STG_PITCH + (iloc & ~3)) = yv;
-        }
-      }
-    }
-  };
-  if (edge) form_g(std::true_type{}); else form_g(std::false_type{});
-  // Each wave takes its own quadrant out (128 columns v x 128 rows i = one contiguous 16 KB run of the K block
-  // wb): it reads only what it wrote itself, so no barrier is needed and no wave waits for the slowest one.
-  uint8_t* gcol = p.ghat_t + ((int64_t)ct * p.kbw + p.kb0 + 2 * rt + wb) * BLOCKED_KSTEP + wa * 128 * BK;
-  const uint8_t* tq = TT + wa * 128 * STG_PITCH + wb * 128;
-#pragma unroll
-  for (int n = 0; n < 16; ++n) {
-    const int cidx = lane + 64 * n, row = cidx >> 3, col = (cidx & 7) * 16;
-    *reinterpret_cast<v4i*>(gcol + row * BK + col) = *reinterpret_cast<const v4i*>(tq + row * STG_PITCH + col);
-  }
+  uint32_t ew;
+  if (vlim < 256) ew = form_dlogits<true, false>(acc, p.k1, p.c2, vlim, 0, smem, wa, wb, nullptr);
+  else ew = form_dlogits<false, false>(acc, p.k1, p.c2, vlim, 0, smem, wa, wb, nullptr);
+  store_dlogits_quadrant(smem, p.ghat_t + ((int64_t)ct * p.kbw + p.kb0 + 2 * rt + wb) * BLOCKED_KSTEP + wa * 128 * BK, wa, wb);
+  if (lane_id() == 0) p.gexp[(int64_t)(2 * ct + wa) * p.kbw + p.kb0 + 2 * rt + wb] = ew;
 }
 
 struct DxParams {
   const uint8_t* wq;      // dq rows, K = Vp, tile by tile: A side (rows j)
   const uint8_t* ghat_t;  // G^T, blocked; already at the K block of the panel's first row    B side (rows i of the panel)
+  const uint32_t* gexp;   // its block exponents [Vp / 128][kbw], likewise at the panel's first row
   const uint8_t* wqt;     // [Vp][dp]   for the one-hot gather
   const float* rho;       // offset to the panel
   const float* hcoef;     // [n_predict][Np], offset to the panel
@@ -853,6 +945,10 @@ struct DxParams {
 // LDS a wave uses to stage its quadrant of a dX tile on the way out: 128 rows of 64 fp32 (or bf16) plus 16 bytes
 constexpr int DX_STAGE_BYTES = 128 * (64 * 4 + 16);
 constexpr int SMEM_DX = 4 * DX_STAGE_BYTES > SMEM_BYTES ? 4 * DX_STAGE_BYTES : SMEM_BYTES;
+// ... or the two K slots and, behind them, the block exponents of the K loop (one dword per K block and half of the rows)
+constexpr int SMEM_MAX = 160 * 1024;
+constexpr int MAX_SCALE_KBLOCKS = (SMEM_MAX - SMEM_BYTES) / 8;      // K blocks of one scaled main loop: 4096
+static inline int smem_scaled(int kblocks, int at_least) { const int n = SMEM_BYTES + 8 * kblocks; return n > at_least ? n : at_least; }
 
 struct DxRowTerms {
   float rs;
@@ -904,13 +1000,21 @@ __global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p) {
     k0 = (int64_t)q0 * 2 * BK; KD = 2 * (q1 - q0);
   }
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
+  // the block exponents of this tile's K loop wait in LDS behind the two K slots: [i half][K block]
+  uint32_t* lsc = reinterpret_cast<uint32_t*>(smem + SMEM_BYTES);
+  for (int e = t; e < 2 * KD; e += NTHREADS) {
+    const int w = e >= KD, kb = e - w * KD;
+    lsc[e] = p.gexp[(k0 / BK + kb) * p.kbw + 2 * rt + w];
+  }
+  __syncthreads();
   v16f acc[4][4];
   // B = G^T: K (v) is the slow index there.  The 128 v rows of a K block are half a v tile; the 256 panel rows of this
   // tile are the two 128-byte pieces of i blocks 2 rt and 2 rt + 1 (BLOCKED_KSTEP apart).
   const int64_t bpair = p.kbw * BLOCKED_KSTEP;                     // from one v tile (two K blocks) to the next
-  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, true>(p.wq + ((int64_t)ct * (p.Vp / BK) + k0 / BK) * BLOCKED_KSTEP, BK,
-                                                    p.ghat_t + 2 * (int64_t)rt * BLOCKED_KSTEP + (k0 / (2 * BK)) * bpair, BLOCKED_KSTEP, KD, smem, acc,
-                                                    2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave), NoHook(), 128 * BK, bpair);
+  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, true, 1>(p.wq + ((int64_t)ct * (p.Vp / BK) + k0 / BK) * BLOCKED_KSTEP, BK,
+                                                       p.ghat_t + 2 * (int64_t)rt * BLOCKED_KSTEP + (k0 / (2 * BK)) * bpair, BLOCKED_KSTEP, KD, smem, acc,
+                                                       2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave), NoHook(), 128 * BK, bpair,
+                                                       lsc + __builtin_amdgcn_readfirstlane(wb) * KD);
   const int jbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
   T* dx = reinterpret_cast<T*>(p.dx);
   if (!SPLIT && p.n_predict == 1) {
@@ -1048,7 +1152,8 @@ __global__ __launch_bounds__(256) void bwd_dx_finish_kernel(DxParams p) {
 
 struct DwParams {
   const uint8_t* xt;      // dq rows, K = Np, blocked                             A side (rows j)
-  const uint8_t* ghat_t;  // Vp rows, K = Pw, blocked                             B side (rows v)
+  const uint8_t* ghat_t;  // Vp rows, blocked, already at the first K block of this launch          B side (rows v)
+  const uint32_t* gexp;   // its block exponents [Vp / 128][kbw], likewise
   float* dwacc;           // [dq][Vp] fp32
   int64_t kbn, kbw, kb0, Vp;   // K blocks per tile of xt and of ghat_t; first K block of xt in this launch; row length of dwacc
   int RT, CT, KT;
@@ -1061,9 +1166,17 @@ __global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
   int rt, ct;
   if (!map_tile_rr(blockIdx.x, p.RT, p.CT, rt, ct)) return;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
+  // the block exponents of this tile's K loop wait in LDS behind the two K slots: [v half][K block]
+  uint32_t* lsc = reinterpret_cast<uint32_t*>(smem + SMEM_BYTES);
+  for (int e = t; e < 2 * p.KT; e += NTHREADS) {
+    const int w = e >= p.KT, kb = e - w * p.KT;
+    lsc[e] = p.gexp[(int64_t)(2 * ct + w) * p.kbw + kb];
+  }
+  __syncthreads();
   v16f acc[4][4];
-  mfma_mainloop<false, NoHook, BLOCKED_KSTEP>(p.xt + ((int64_t)rt * p.kbn + p.kb0) * BLOCKED_KSTEP, BK, p.ghat_t + (int64_t)ct * p.kbw * BLOCKED_KSTEP, BK, p.KT,
-                                              smem, acc, ct & 7, 2 * (rt & 3), __builtin_amdgcn_readfirstlane(wave));
+  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, false, 2>(p.xt + ((int64_t)rt * p.kbn + p.kb0) * BLOCKED_KSTEP, BK, p.ghat_t + (int64_t)ct * p.kbw * BLOCKED_KSTEP, BK, p.KT,
+                                                        smem, acc, ct & 7, 2 * (rt & 3), __builtin_amdgcn_readfirstlane(wave), NoHook(), 0, 0,
+                                                        lsc + __builtin_amdgcn_readfirstlane(wb) * p.KT);
   const int jbase = rt * 256 + wa * 128 + 4 * (lane >> 5);
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
@@ -1324,12 +1437,12 @@ static int check_device(int dev) {
       // the MFMA kernels hold two 64 KB K-slots in LDS
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_recompute_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_RECOMPUTE));
-      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_DX));
-      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_DX));
-      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_DX));
-      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_DX));
-      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
-      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
     }
   }
   if (g_arch_ok[dev] != 1) return fail(SCE_EARCH, "device %d is not gfx950", dev);
@@ -1343,6 +1456,8 @@ static int check_shape(const sce_shape* s) {
   if (s->d % 16 != 0) return fail(SCE_EINVAL, "d = %lld must be a multiple of 16", (long long)s->d);
   if (s->N > (1ll << 24) - 256 || s->V > (1ll << 24) - 256 || s->d > (1ll << 24) - 256)
     return fail(SCE_EINVAL, "N, d and V must be below 2^24 (32-bit tile offsets)");
+  if (s->V > (int64_t)MAX_SCALE_KBLOCKS * BK)
+    return fail(SCE_EINVAL, "V = %lld must be at most %d (the block exponents of a dX tile's K loop wait in LDS)", (long long)s->V, MAX_SCALE_KBLOCKS * BK);
   if (s->d > (1ll << 22) - 256) return fail(SCE_EINVAL, "d = %lld must be below 2^22 (a grid dimension of the layout kernels)", (long long)s->d);
   if (s->n_predict < 1 || s->n_predict > 4) return fail(SCE_EINVAL, "n_predict = %d must be between 1 and 4", s->n_predict);
   return SCE_OK;
@@ -1364,7 +1479,6 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int npa
   B.P = P; B.Pw = Pw; B.nparts = nparts;
   size_t o = 0;
   auto take = [&](size_t bytes) { size_t r = o; o += (bytes + 255) / 256 * 256; return r; };
-  B.off_crow = take((size_t)S.Np * 4);
   B.off_rho = take((size_t)S.Np * 4);
   B.off_hcoef = take((size_t)S.Np * 4 * K);
   B.off_blockmax = take((size_t)(S.Np / 256) * 4);
@@ -1380,6 +1494,7 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int npa
   B.off_dxpart = take(DX_PART_BYTES);
   B.fixed = o;
   B.off_ghat_t = take((size_t)S.Vp * Pw);
+  B.off_gexp = take((size_t)(S.Vp / 128) * (Pw / 128) * 4);      // block exponents of the dlogits
   B.part_stride = ((size_t)S.dq * S.Vp * 4 + 255) / 256 * 256;
   B.off_dwacc = take(B.part_stride * (size_t)nparts);     // fp32 dW partials, one per dW launch
   B.total = o;
@@ -1482,18 +1597,18 @@ static int grid_for(size_t work_items, int per_block) {
   return (int)g;
 }
 
-extern "C" int sce_quantize_e4m3(const void* src, int32_t src_dtype, void* dst, float scale, size_t n, int32_t device,
+extern "C" int sce_quantize_e4m3(const void* src, int32_t src_dtype, void* dst, double scale, size_t n, int32_t device,
                                  void* stream) {
   if (!src || !dst) return fail(SCE_EINVAL, "src/dst is NULL");
-  if (!(scale > 0.f)) return fail(SCE_EINVAL, "scale must be positive");
+  if (!(scale > 0.0)) return fail(SCE_EINVAL, "scale must be positive");
   if (int rc = check_device(device)) return rc;
   if (n == 0) return SCE_OK;
   DeviceGuard guard(device);
   if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", device);
   hipStream_t st = (hipStream_t)stream;
   const int grid = grid_for((n + 3) / 4, 256);
-  if (src_dtype == SCE_F32) quantize_flat_kernel<float><<<grid, 256, 0, st>>>((const float*)src, (uint8_t*)dst, n, scale);
-  else if (src_dtype == SCE_BF16) quantize_flat_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)src, (uint8_t*)dst, n, scale);
+  if (src_dtype == SCE_F32) quantize_flat_kernel<float><<<grid, 256, 0, st>>>((const float*)src, (uint8_t*)dst, n, (float)(1.0 / scale));
+  else if (src_dtype == SCE_BF16) quantize_flat_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)src, (uint8_t*)dst, n, (float)(1.0 / scale));
   else return fail(SCE_EINVAL, "unsupported dtype %d", src_dtype);
   HIP_TRY(hipGetLastError());
   return SCE_OK;
@@ -1518,7 +1633,7 @@ static int check_common(const sce_args* a) {
   if (int rc = check_shape(&a->shape)) return rc;
   if (!a->targets) return fail(SCE_EINVAL, "targets is NULL");
   if (!(a->cap > 0.f) || a->cap > 40.f) return fail(SCE_EINVAL, "cap = %g must be in (0, 40]", (double)a->cap);
-  if (!(a->x_s > 0.f) || !(a->w_s > 0.f)) return fail(SCE_EINVAL, "x_s and w_s must be positive");
+  if (!(a->x_s > 0.0) || !(a->w_s > 0.0)) return fail(SCE_EINVAL, "x_s and w_s must be positive");
   if (a->reduction != SCE_REDUCE_NONE && a->reduction != SCE_REDUCE_MEAN) return fail(SCE_EINVAL, "bad reduction %d", a->reduction);
   if (!a->saved) return fail(SCE_EINVAL, "saved is NULL");
   if (((uintptr_t)a->saved & 255) || ((uintptr_t)a->workspace & 255) || ((uintptr_t)a->wcache & 255))
@@ -1560,27 +1675,27 @@ extern "C" int sce_forward(const sce_args* a) {
     float* rstd = (float*)(sv + S.off_rstd);
     const int ngrid = (int)((S.Np + 3) / 4);
     if (a->norm && a->x_dtype == SCE_F32)
-      rmsnorm_quantize_kernel<float><<<ngrid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, a->norm_eps, xq, S.Np, S.dp, S.ldx, a->x_s, rstd);
+      rmsnorm_quantize_kernel<float><<<ngrid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, a->norm_eps, xq, S.Np, S.dp, S.ldx, (float)(1.0 / a->x_s), rstd);
     else if (a->norm && a->x_dtype == SCE_BF16)
-      rmsnorm_quantize_kernel<bf16_t><<<ngrid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, a->norm_eps, xq, S.Np, S.dp, S.ldx, a->x_s, rstd);
+      rmsnorm_quantize_kernel<bf16_t><<<ngrid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, a->norm_eps, xq, S.Np, S.dp, S.ldx, (float)(1.0 / a->x_s), rstd);
     else if (a->x_dtype == SCE_F32)
-      quantize_pad_kernel<float><<<grid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, S.ldx, a->x_s);
+      quantize_pad_kernel<float><<<grid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, S.ldx, (float)(1.0 / a->x_s));
     else if (a->x_dtype == SCE_BF16)
-      quantize_pad_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, S.ldx, a->x_s);
+      quantize_pad_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, S.ldx, (float)(1.0 / a->x_s));
     else return fail(SCE_EINVAL, "unsupported x dtype %d", a->x_dtype);
     dim3 gw((unsigned)(S.Vp / 64), (unsigned)(S.dq / 64));
     if (a->wcache && a->wcache_valid) {
       // the caller vouches that the cache holds e4m3(W / w_s) of this W (unchanged since an earlier call)
     } else if (a->w_dtype == SCE_F32)
-      quantize_w_kernel<float><<<gw, 256, 0, st>>>((const float*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.Vp / BK, a->w_s);
+      quantize_w_kernel<float><<<gw, 256, 0, st>>>((const float*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.Vp / BK, (float)(1.0 / a->w_s));
     else if (a->w_dtype == SCE_BF16)
-      quantize_w_kernel<bf16_t><<<gw, 256, 0, st>>>((const bf16_t*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.Vp / BK, a->w_s);
+      quantize_w_kernel<bf16_t><<<gw, 256, 0, st>>>((const bf16_t*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.Vp / BK, (float)(1.0 / a->w_s));
     else return fail(SCE_EINVAL, "unsupported w dtype %d", a->w_dtype);
   }
   FwdParams p;
   p.xq = xq; p.wqt = wqt; p.partials = (float4*)a->workspace;
   p.dp = S.dp; p.ldx = S.ldx; p.N = (int)N; p.V = (int)Vl; p.Np = (int)S.Np; p.RT = RT; p.CT = CT; p.S = nsplit;
-  p.sc = a->x_s * a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.ic2 = 1.0f / (-2.0f * a->cap * LOG2E);
+  p.sc = (float)a->x_s * (float)a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.ic2 = 1.0f / (-2.0f * a->cap * LOG2E);
   const int grid = 8 * nsplit * ((RT + 7) / 8);
   {
     KernelTimer tm(SCE_K_FWD, st);
@@ -1591,7 +1706,7 @@ extern "C" int sce_forward(const sce_args* a) {
   float* s_umax = (float*)(sv + S.off_umax);
   float* s_zy = (float*)(sv + S.off_zy);
   fwd_target_logit_kernel<<<dim3((unsigned)((N + 3) / 4), (unsigned)a->shape.n_predict), 256, 0, st>>>(
-      xq, wqt, S.dp, S.ldx, a->targets, a->ignore_index, (int)N, (int)S.Np, (int)Vl, a->x_s * a->w_s, a->cap, s_zy);
+      xq, wqt, S.dp, S.ldx, a->targets, a->ignore_index, (int)N, (int)S.Np, (int)Vl, (float)a->x_s * (float)a->w_s, a->cap, s_zy);
   fwd_combine_kernel<<<(int)(S.Np / 256), 256, 0, st>>>(p.partials, nsplit, (int)N, (int)S.Np, (int)Vl, a->targets, a->ignore_index,
                                                        a->cap, a->mtp_weights, a->shape.n_predict, s_lse, s_umax, s_zy, a->losses, a->lse,
                                                        a->argmax);
@@ -1630,6 +1745,7 @@ extern "C" int sce_backward(const sce_args* a) {
   if (a->panel_rows > 0) {
     if (a->panel_rows % 256) return fail(SCE_EINVAL, "panel_rows must be a multiple of 256");
     P = a->panel_rows < S.Np ? a->panel_rows : S.Np;
+    if (P > 131072) P = 131072;          // a dW launch covers at least one panel and at most MAX_SCALE_KBLOCKS K blocks
   }
   if (P * S.Vp > room) P = room / S.Vp / 256 * 256;
   if (P < 256) P = 256;                                  // Bmin fits, as checked above
@@ -1655,10 +1771,9 @@ extern "C" int sce_backward(const sce_args* a) {
   const uint8_t* wqt = wbase + S.rel_wqt;
   const uint8_t* wq = wbase + S.rel_wq;
   const float* s_lse = (const float*)(sv + S.off_lse);
-  const float* s_umax = (const float*)(sv + S.off_umax);
   const float* s_zy = (const float*)(sv + S.off_zy);
   const int32_t* hdr = (const int32_t*)(sv + S.off_hdr);
-  float* crow = (float*)(ws + B.off_crow);
+  uint32_t* gexp = (uint32_t*)(ws + B.off_gexp);
   float* rho = (float*)(ws + B.off_rho);
   float* hcoef = (float*)(ws + B.off_hcoef);
   float* blockmax = (float*)(ws + B.off_blockmax);
@@ -1677,9 +1792,9 @@ extern "C" int sce_backward(const sce_args* a) {
 
   const int nblk = (int)(S.Np / 256);
   KernelTimer* tm_prep = new KernelTimer(SCE_K_BWD_PREP, st);
-  bwd_prep_kernel<<<nblk, 256, 0, st>>>(s_lse, s_umax, s_zy, a->targets, a->ignore_index, hdr, a->grad_output,
+  bwd_prep_kernel<<<nblk, 256, 0, st>>>(s_lse, s_zy, a->targets, a->ignore_index, hdr, a->grad_output,
                                         a->reduction == SCE_REDUCE_NONE ? 1 : 0, a->grad_scale, a->mtp_weights, K, a->cap, (int)N,
-                                        (int)S.Np, (int)Vl, crow, rho, hcoef, blockmax);
+                                        (int)S.Np, (int)Vl, rho, hcoef, blockmax);
   bwd_xi_kernel<<<1, 1024, 0, st>>>(blockmax, nblk, xi);
   {
     dim3 g((unsigned)(S.Np / 64), (unsigned)(S.dq / 64));
@@ -1697,7 +1812,7 @@ extern "C" int sce_backward(const sce_args* a) {
     bwd_longlist_kernel<<<(int)((V + 255) / 256), 256, 0, st>>>(segoff, (int)V, longlist);
   }
   delete tm_prep;
-  const float k1 = a->x_s * a->w_s * 2.0f * LOG2E / a->cap, c2 = -2.0f * a->cap * LOG2E;
+  const float k1 = (float)a->x_s * (float)a->w_s * 2.0f * LOG2E / a->cap, c2 = -2.0f * a->cap * LOG2E;
   const int CTv = (int)(S.Vp / 256), CTd = (int)(S.dq / 256);
   int launch = 0;
   int64_t w0 = 0;                      // first row of the rows gathered for the next dW launch
@@ -1705,18 +1820,24 @@ extern "C" int sce_backward(const sce_args* a) {
     const int64_t prow = (S.Np - p0 < P) ? (S.Np - p0) : P;     // multiple of 256
     const int RTp = (int)(prow / 256);
     RecomputeParams rp;
-    rp.xq = xq + p0 * S.ldx; rp.wqt = wqt; rp.crow = crow + p0; rp.ghat_t = ghat_t;
+    rp.xq = xq + p0 * S.ldx; rp.wqt = wqt; rp.ghat_t = ghat_t; rp.gexp = gexp;
     rp.dp = S.dp; rp.ldx = S.ldx; rp.kbw = Pw / BK; rp.kb0 = (p0 - w0) / BK; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2;
     {
       KernelTimer tm(SCE_K_RECOMPUTE, st);
       bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_RECOMPUTE, st>>>(rp);
     }
+    if (p0 < N) {      // the target columns leave G: their part of dlogits is in the one-hot coefficients
+      KernelTimer tm(SCE_K_BWD_PREP, st);
+      const int rows = (int)(N - p0 < prow ? N - p0 : prow);
+      bwd_zero_targets_kernel<<<(rows * K + 255) / 256, 256, 0, st>>>(a->targets, a->ignore_index, (int)p0, rows, (int)N, (int)Vl, K,
+                                                                    ghat_t + ((p0 - w0) / BK) * BLOCKED_KSTEP, Pw / BK);
+    }
 
     DxParams dp_;
-    dp_.wq = wq; dp_.ghat_t = ghat_t + ((p0 - w0) / BK) * BLOCKED_KSTEP; dp_.kbw = Pw / BK; dp_.wqt = wqt; dp_.rho = rho + p0; dp_.hcoef = hcoef + p0; dp_.targets = a->targets + p0;
+    dp_.wq = wq; dp_.ghat_t = ghat_t + ((p0 - w0) / BK) * BLOCKED_KSTEP; dp_.gexp = gexp + (p0 - w0) / BK; dp_.kbw = Pw / BK; dp_.wqt = wqt; dp_.rho = rho + p0; dp_.hcoef = hcoef + p0; dp_.targets = a->targets + p0;
     dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.ldx = S.ldx; dp_.Np = S.Np; dp_.dq = S.dq; dp_.RT = RTp; dp_.CT = CTd;
     dp_.n_predict = K; dp_.rows_left = (int)(N - p0 > 0 ? N - p0 : 0);
-    dp_.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); dp_.d = (int)d; dp_.V = (int)Vl; dp_.w_s = a->w_s;
+    dp_.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); dp_.d = (int)d; dp_.V = (int)Vl; dp_.w_s = (float)a->w_s;
     dp_.part = (float*)(ws + B.off_dxpart);
     // a panel with fewer than half as many tiles as there are CUs shares each tile's K loop among several workgroups
     const int tiles = RTp * CTd, kpairs = (int)(S.Vp / BK / 2);
@@ -1727,17 +1848,18 @@ extern "C" int sce_backward(const sce_args* a) {
     {
       KernelTimer tm(SCE_K_DX, st);
       const bool f32 = a->dx_dtype == SCE_F32;
+      const int smem_dx = smem_scaled((int)(S.Vp / BK), SMEM_DX);
       dp_.dx = f32 ? (void*)((float*)a->dx + p0 * a->dx_ld) : (void*)((bf16_t*)a->dx + p0 * a->dx_ld);
       if (ksplit == 1) {
-        if (f32) bwd_dx_kernel<float, false><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_DX, st>>>(dp_);
-        else bwd_dx_kernel<bf16_t, false><<<map_tile_grid(RTp, CTd), NTHREADS, SMEM_DX, st>>>(dp_);
+        if (f32) bwd_dx_kernel<float, false><<<map_tile_grid(RTp, CTd), NTHREADS, smem_dx, st>>>(dp_);
+        else bwd_dx_kernel<bf16_t, false><<<map_tile_grid(RTp, CTd), NTHREADS, smem_dx, st>>>(dp_);
       } else if (dp_.rows > 0) {
         const int fgrid = (int)(((int64_t)dp_.rows * (d / 4) + 255) / 256);
         if (f32) {
-          bwd_dx_kernel<float, true><<<map_tile_grid(RTp, CTd * ksplit), NTHREADS, SMEM_DX, st>>>(dp_);
+          bwd_dx_kernel<float, true><<<map_tile_grid(RTp, CTd * ksplit), NTHREADS, smem_dx, st>>>(dp_);
           bwd_dx_finish_kernel<float><<<fgrid, 256, 0, st>>>(dp_);
         } else {
-          bwd_dx_kernel<bf16_t, true><<<map_tile_grid(RTp, CTd * ksplit), NTHREADS, SMEM_DX, st>>>(dp_);
+          bwd_dx_kernel<bf16_t, true><<<map_tile_grid(RTp, CTd * ksplit), NTHREADS, smem_dx, st>>>(dp_);
           bwd_dx_finish_kernel<bf16_t><<<fgrid, 256, 0, st>>>(dp_);
         }
       }
@@ -1747,13 +1869,13 @@ extern "C" int sce_backward(const sce_args* a) {
     if (gathered + P > Pw || p0 + prow >= S.Np) {      // the transposed scratch is full, or this was the last panel
       DwParams wp;
       const int part = launch < nparts ? launch : nparts - 1;
-      wp.xt = xt; wp.ghat_t = ghat_t; wp.dwacc = (float*)((uint8_t*)dwacc + (size_t)part * B.part_stride);
+      wp.xt = xt; wp.ghat_t = ghat_t; wp.gexp = gexp; wp.dwacc = (float*)((uint8_t*)dwacc + (size_t)part * B.part_stride);
       wp.kbn = S.Np / BK; wp.kbw = Pw / BK; wp.kb0 = w0 / BK; wp.Vp = S.Vp;
       wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(gathered / BK);
       {
         KernelTimer tm(SCE_K_DW, st);
-        if (launch >= nparts) bwd_dw_kernel<true><<<map_tile_rr_grid(CTd, CTv), NTHREADS, SMEM_BYTES, st>>>(wp);
-        else bwd_dw_kernel<false><<<map_tile_rr_grid(CTd, CTv), NTHREADS, SMEM_BYTES, st>>>(wp);
+        if (launch >= nparts) bwd_dw_kernel<true><<<map_tile_rr_grid(CTd, CTv), NTHREADS, smem_scaled(wp.KT, 0), st>>>(wp);
+        else bwd_dw_kernel<false><<<map_tile_rr_grid(CTd, CTv), NTHREADS, smem_scaled(wp.KT, 0), st>>>(wp);
       }
       ++launch;
       w0 = p0 + prow;
@@ -1773,10 +1895,10 @@ extern "C" int sce_backward(const sce_args* a) {
   {
     dim3 g((unsigned)((V + 63) / 64), (unsigned)((d + 63) / 64));
     if (a->dw_dtype == SCE_F32)
-      bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, S.dq, a->x_s, (int)d, (int)V,
+      bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, S.dq, (float)a->x_s, (int)d, (int)V,
                                                    (float*)a->dw, a->dw_ld);
     else
-      bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, S.dq, a->x_s, (int)d, (int)V,
+      bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, S.dq, (float)a->x_s, (int)d, (int)V,
                                                     (bf16_t*)a->dw, a->dw_ld);
   }
   HIP_TRY(hipGetLastError());

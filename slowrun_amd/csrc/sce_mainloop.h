@@ -98,11 +98,34 @@ struct NoHook { __device__ __forceinline__ void operator()(int) const {} };
 // does not depend on the accumulators (it runs while the matrix pipe is busy).
 // TRB (see TileLoads): the K blocks of B lie bk1 bytes apart within a pair and bk2 bytes from pair to pair
 // (for TRB = false they are KSTEP and 2 KSTEP and the two arguments are ignored).
-template <bool PREFETCHED = false, class Hook = NoHook, int KSTEP = BK, bool TRB = false>
+//
+// SCALE: the B operand is block-scaled (MX style): its true value is byte * 2^(E - 127) with one E8M0 exponent E per
+// block of 32 B rows x 128 bytes of K or so, applied by v_mfma_scale_f32_32x32x64_f8f6f4 (lane l supplies, in the byte of
+// its scale register that the instruction's op_sel names, the exponent of B row l % 32 for K values [0, 32) of the
+// instruction if l < 32 and [32, 64) otherwise).
+// The exponents of a tile wait in LDS behind the two K slots, one dword per K block for each half (wb) of the B rows:
+//   SCALE = 1: byte b of the dword of K block k belongs to the wave's B rows [32 b, 32 b + 32) (dX: B = dlogits, K = v);
+//   SCALE = 2: byte c of the dword of K block k belongs to K values [32 c, 32 c + 32) of that block, for all of the
+//              wave's 128 B rows (dW: B = dlogits^T, K = i).
+// The A operand goes in with exponent 127 (factor 1).  lds_scale points at the wave's KD dwords.
+template <int OPB>
+__device__ __forceinline__ v16f mfma_fp8_scaled(const v8i& a, const v8i& b, const v16f& c, int sa, int sb) {
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, sa, OPB, sb);
+}
+__device__ __forceinline__ v16f mfma_fp8_scaled_sel(int opb, const v8i& a, const v8i& b, const v16f& c, int sa, int sb) {
+  switch (opb) {       // op_sel is part of the instruction: the callers' loops are unrolled, so this folds
+    case 0: return mfma_fp8_scaled<0>(a, b, c, sa, sb);
+    case 1: return mfma_fp8_scaled<1>(a, b, c, sa, sb);
+    case 2: return mfma_fp8_scaled<2>(a, b, c, sa, sb);
+    default: return mfma_fp8_scaled<3>(a, b, c, sa, sb);
+  }
+}
+
+template <bool PREFETCHED = false, class Hook = NoHook, int KSTEP = BK, bool TRB = false, int SCALE = 0, int FIRST_WAIT = 8>
 __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, int64_t lda,
                                               const uint8_t* __restrict__ Bg, int64_t ldb, int KD,
                                               uint8_t* smem, v16f (&acc)[4][4], int rot_a, int rot_b, int wave, Hook&& hook = NoHook(),
-                                              int64_t bk1_arg = 0, int64_t bk2_arg = 0) {
+                                              int64_t bk1_arg = 0, int64_t bk2_arg = 0, const uint32_t* lds_scale = nullptr) {
   const int lane = lane_id();
   const int wa = wave >> 1, wb = wave & 1;
   const int64_t bk1 = TRB ? bk1_arg : (int64_t)KSTEP, bk2 = TRB ? bk2_arg : (int64_t)(2 * KSTEP);
@@ -131,10 +154,14 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
       fb[b] = f;
       return;
     }
-    const int c0 = ((4 * half + 2 * h) ^ sw) * 16;
+    // Which 32 of the sub-step's 64 K bytes a lane takes does not matter as long as both operands agree -- except
+    // to the block scales: the instruction counts registers 0..3 of lanes l and l + 32 as the first 32 K values (scale
+    // from lane l < 32) and registers 4..7 of both as the second 32 (scale from lane l + 32).  With per-K exponents
+    // (SCALE = 2) the lanes therefore take the 16-byte chunks h and 2 + h, otherwise 2 h and 2 h + 1.
+    const int c0 = ((SCALE == 2 ? 4 * half + h : 4 * half + 2 * h) ^ sw) * 16;
     const uint8_t* s = smem + slot * SLOT_BYTES + ((n < 4) ? abase + n * 32 * BK : bbase + (n - 4) * 32 * BK);
     const v4i lo = *reinterpret_cast<const v4i*>(s + c0);
-    const v4i hi = *reinterpret_cast<const v4i*>(s + (c0 ^ 16));
+    const v4i hi = *reinterpret_cast<const v4i*>(s + (c0 ^ (SCALE == 2 ? 32 : 16)));
     const v8i f = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     if (n < 4) fa[n] = f; else fb[n - 4] = f;
   };
@@ -145,19 +172,33 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
 #pragma unroll
     for (int n = 0; n < 8; ++n) ld.template issue<1>(n, Ag + KSTEP, Bg + bk1);
   }
-  asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+  // FIRST_WAIT: how many of the wave's vector memory operations may still be in flight once K block 0 has landed
+  // (the 8 loads of block 1, plus whatever a caller issued between its prefetch of block 0 and this point)
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(FIRST_WAIT) : "memory");
   v8i fa[2][4], fb[2][4];
 #pragma unroll
   for (int n = 0; n < 8; ++n) rfrag1(0, 0, n, fa[0], fb[0]);
-  auto mm = [&](int cur, int i) {
+  // block scales of the current pair of K blocks and of the next one (read one pair ahead)
+  const __attribute__((address_space(3))) v2i* scp = (const __attribute__((address_space(3))) v2i*)lds_scale;
+  const int sc_shift = (SCALE == 2) ? 8 * (lane >> 5) : 0;      // SCALE = 2: the upper half-wave feeds the odd 32-blocks of K
+  int sc[2] = {0, 0}, scn[2] = {0, 0};
+  auto sc_load = [&](int (&dst)[2]) {
+    const v2i d = *scp++;
+    dst[0] = (int)((uint32_t)d[0] >> sc_shift); dst[1] = (int)((uint32_t)d[1] >> sc_shift);
+  };
+  if (SCALE) sc_load(sc);
+  // blk: which K block of the pair; cur: fragment register set = which 64-byte half of the block
+  auto mm = [&](int blk, int cur, int i) {
     const int a = i >> 2, b = i & 3;
-    acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[cur][a], fb[cur][b], acc[a][b], 0, 0, 0, 0, 0, 0);
+    if (SCALE) acc[a][b] = mfma_fp8_scaled_sel(SCALE == 1 ? b : 2 * cur, fa[cur][a], fb[cur][b], acc[a][b], 127, sc[blk]);
+    else acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[cur][a], fb[cur][b], acc[a][b], 0, 0, 0, 0, 0, 0);
   };
   // the very first MFMA of each accumulator block takes a zero constant instead of the register: nothing clears them
   auto mm0 = [&](int i) {
     const int a = i >> 2, b = i & 3;
     const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[0][a], fb[0][b], zero, 0, 0, 0, 0, 0, 0);
+    if (SCALE) acc[a][b] = mfma_fp8_scaled_sel(SCALE == 1 ? b : 0, fa[0][a], fb[0][b], zero, 127, sc[0]);
+    else acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[0][a], fb[0][b], zero, 0, 0, 0, 0, 0, 0);
   };
   // One K block = two sub-steps of 16 MFMAs; register set 0 feeds the first, set 1 the second.  The
   // loop body handles the blocks in pairs (slot 0, then slot 1) so that every LDS address and every
@@ -175,21 +216,21 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
     // ---- block 2p (slot 0)
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      if (first) mm0(i); else mm(0, i);
+      if (first) mm0(i); else mm(0, 0, i);
       hook(0 + (i & 7));
       ld.template issue<1>(8 + i, ga + KSTEP, gb + bk1);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 8; i < 16; ++i) {
-      if (first) mm0(i); else mm(0, i);
+      if (first) mm0(i); else mm(0, 0, i);
       hook(8 + (i & 7));
       rfrag1(0, 1, i - 8, fa[1], fb[1]);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      mm(1, i);
+      mm(0, 1, i);
       hook(16 + (i & 7));
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -197,30 +238,31 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 8; i < 16; ++i) {
-      mm(1, i);
+      mm(0, 1, i);
       hook(24 + (i & 7));
       rfrag1(1, 0, i - 8, fa[0], fb[0]);
       if (more) ld.template issue<0>(i - 8, ga + 2 * KSTEP, gb + bk2);
       __builtin_amdgcn_sched_barrier(0);
     }
     // ---- block 2p + 1 (slot 1)
+    if (SCALE && more) sc_load(scn);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      mm(0, i);
+      mm(1, 0, i);
       hook(32 + (i & 7));
       if (more) ld.template issue<0>(8 + i, ga + 2 * KSTEP, gb + bk2);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 8; i < 16; ++i) {
-      mm(0, i);
+      mm(1, 0, i);
       hook(40 + (i & 7));
       rfrag1(1, 1, i - 8, fa[1], fb[1]);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      mm(1, i);
+      mm(1, 1, i);
       hook(48 + (i & 7));
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -228,7 +270,7 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 8; i < 16; ++i) {
-      mm(1, i);
+      mm(1, 1, i);
       hook(56 + (i & 7));
       if (more) {
         rfrag1(0, 0, i - 8, fa[0], fb[0]);
@@ -236,6 +278,7 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
       }
       __builtin_amdgcn_sched_barrier(0);
     }
+    if (SCALE && more) { sc[0] = scn[0]; sc[1] = scn[1]; }
   };
   const int P = KD >> 1;
   if (P == 1) {

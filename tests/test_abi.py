@@ -36,7 +36,7 @@ def test_header_functions_are_exported(lib):
 
 
 def test_version(lib):
-    assert lib.sce_version() == _lib.SCE_VERSION == 3
+    assert lib.sce_version() == _lib.SCE_VERSION == 4
 
 
 def test_struct_layout_matches_c(tmp_path):

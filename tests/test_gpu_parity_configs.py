@@ -50,14 +50,15 @@ def test_large_vocab_full():
 def test_irregular_full():
     inp, ours, ref, rep = _run("irregular")
     assert rep["n_ignored"] > 3000
-    # permuting the rows permutes lse and the rows of dX bit for bit (each row is reduced in the same
-    # order wherever it sits) and leaves dW unchanged up to the order of the sum over rows
+    # permuting the rows permutes lse bit for bit (each row is reduced in the same order wherever it sits); the rows
+    # of dX move with it up to the e4m3 rounding of the dlogits, whose exponent a row shares with the 31 rows around
+    # it; dW is unchanged up to that and the order of the sum over rows
     perm = torch.randperm(inp.x.shape[0], generator=torch.Generator().manual_seed(0))
     inp2 = configs.HeadInputs(inp.name, inp.x[perm], inp.w, inp.targets[perm], inp.x_s, inp.w_s, inp.cap)
     ours2 = pu.run_ours(inp2, "mean")
     permd = perm.cuda()
     assert torch.equal(ours2["lse"], ours["lse"][permd])
-    assert torch.equal(ours2["dx"], ours["dx"][permd])
+    assert pu.maxrel(ours2["dx"].float(), ours["dx"][permd].float()) < 2e-2 and pu.cosine(ours2["dx"].float(), ours["dx"][permd].float()) > 0.9999
     assert pu.maxrel(ours2["dw"].float(), ours["dw"].float()) < 1e-2 and pu.cosine(ours2["dw"].float(), ours["dw"].float()) > 0.99999
 
 
