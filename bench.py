@@ -46,6 +46,9 @@ def main():
     ap.add_argument("--workload", default="limited_2p7b")
     ap.add_argument("--rows", type=int, default=None, help="override N (debugging only; the result is then not the headline)")
     ap.add_argument("--panel-rows", type=int, default=0)
+    ap.add_argument("--dlogits", choices=["keep", "recompute"], default="keep",
+                    help="keep: the forward pass emits the dlogits (N x V bytes held until backward, backward is two GEMMs); "
+                         "recompute: backward computes the logit tiles again (nothing N x V is held)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=16384)
     ap.add_argument("--copy-calibration", action="store_true",
@@ -72,11 +75,12 @@ def main():
     w = inp.w.to(dev, torch.bfloat16)
     y = inp.targets.to(dev)
     go = torch.ones((), device=dev)
+    keep = args.dlogits == "keep"
 
     def step():
-        loss, saved, _lse, _am, _nv = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, "mean")
+        loss, saved, _lse, _am, _nv = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, "mean", keep_dlogits=keep)
         dx, dw = ck.ce_backward(saved, y, go, N, d, V, inp.x_s, inp.w_s, inp.cap, 1.0, "mean", torch.bfloat16, torch.bfloat16,
-                                panel_rows=args.panel_rows)
+                                panel_rows=args.panel_rows, keep_dlogits=keep)
         return loss, dx, dw
 
     for _ in range(args.warmup):

@@ -59,6 +59,9 @@ typedef struct sce_sizes {
   size_t bwd_workspace_min_bytes;   /* backward with the smallest row panel (256 rows)       */
   size_t bwd_workspace_bytes;       /* backward with the default row panel                   */
   int64_t bwd_panel_rows;           /* the default row panel                                 */
+  /* with sce_args.dlogits_from_forward: */
+  size_t dlogits_bytes;             /* `saved` grows by this much (N x V bytes and a little)  */
+  size_t bwd_workspace_kept_bytes;  /* and backward needs this workspace, no more             */
 } sce_sizes;
 
 typedef struct sce_args {
@@ -112,7 +115,11 @@ typedef struct sce_args {
                                 normalises inside the quantiser, backward needs x again and returns the
                                 gradient with respect to h in dx                                  */
   float norm_eps;
-  int32_t pad5;
+  int32_t dlogits_from_forward;  /* 0: backward computes the logit tiles again (nothing N x V is kept between the two
+                                calls); non-zero: forward also leaves the dlogits, 8 bits each, at the end of `saved`
+                                (saved_bytes or saved_x_bytes, plus dlogits_bytes) and backward is two GEMMs instead of
+                                three.  Same value in both calls.  The reference keeps bf16 logits and e5m2 dlogits
+                                (tiny/cuda_kernels.py:359-371)                                                       */
 } sce_args;
 
 /* Library / ABI version (SCE_VERSION of the build). */

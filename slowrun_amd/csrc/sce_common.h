@@ -21,6 +21,7 @@ constexpr int BK = 128;          // K bytes per LDS slot row
 constexpr int SLOT_BYTES = (TM + TN) * BK;      // 65536
 constexpr int SMEM_BYTES = 2 * SLOT_BYTES;      // 131072 of the 163840 B a workgroup may hold
 constexpr int NTHREADS = 256;
+constexpr int SMEM_MAX = 160 * 1024;              // LDS a workgroup may hold on gfx950
 
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr int LONG_SEG = 64;     // target columns hit by at least this many rows get their own reduction kernel
@@ -47,9 +48,10 @@ static inline int64_t row_stride(int64_t k) { return k + 128; }
 struct SavedLayout {
   int64_t ldx;                       // row stride in bytes of the [..][dp] e4m3 arrays
   int64_t N, d, V, Np, dp, dq, Vp;   // all padded sizes are multiples of 256 (every K loop runs over an even number of 128-byte blocks); dp = dq
-  size_t off_hdr, off_xq, off_lse, off_umax, off_zy, off_rstd, x_total;
+  size_t off_hdr, off_xq, off_lse, off_umax, off_zy, off_rstd, off_lam, x_total;
   size_t rel_wqt, rel_wq, w_total;   // relative to the start of the W region
   size_t total;                      // x_total + w_total
+  size_t rel_g, rel_gexp, g_total;   // dlogits emitted by the forward pass (optional; behind whatever else `saved` holds)
 };
 // hdr: int32 n_valid, int32 n_bad_targets, float mean loss, float pad
 
@@ -66,18 +68,23 @@ static inline SavedLayout saved_layout(int64_t N, int64_t d, int64_t V, int n_pr
   L.off_umax = take((size_t)L.Np * 4);
   L.off_zy = take((size_t)L.Np * 4 * n_predict);
   L.off_rstd = take((size_t)L.Np * 4);         // 1 / rms of each row when the final norm is part of the call
+  L.off_lam = take((size_t)L.Np * 4);          // per-row exponent boost of the dlogits (an integer in a float)
   L.x_total = o;
   o = 0;
   L.rel_wqt = take((size_t)L.Vp * L.ldx);      // W_q^T [Vp][dp], row stride ldx
   L.rel_wq = take((size_t)L.dq * L.Vp);        // W_q: dq rows, K = Vp, tile by tile (256 rows x 128 B per K block)
   L.w_total = o;
   L.total = L.x_total + L.w_total;
+  o = 0;
+  L.rel_g = take((size_t)L.Vp * L.Np);                          // G^T, Vp rows, K = Np, tile by tile
+  L.rel_gexp = take((size_t)(L.Vp / 128) * (L.Np / 128) * 4);   // its block exponents
+  L.g_total = o;
   return L;
 }
 
 struct BwdLayout {
   int64_t P, Pw;                     // rows per recompute/dX panel and per dW launch (multiples of 256, Pw of P)
-  size_t off_gexp, off_rho, off_hcoef, off_blockmax, off_xi, off_xt, off_dwacc, off_perm, off_keys,
+  size_t off_gexp, off_rho, off_rowinfo, off_hcoef, off_blockmax, off_xi, off_xt, off_dwacc, off_perm, off_keys,
       off_segoff, off_longlist, off_longsum, off_sorttmp, off_dxpart, off_ghat_t, fixed, total;
   size_t sorttmp_bytes, part_stride;   // part_stride: bytes between consecutive fp32 dW partials
   int nparts;

@@ -365,17 +365,170 @@ __global__ __launch_bounds__(256) void transpose_bytes_kernel(const uint8_t* __r
 }
 
 // ------------------------------------------------------------------------------------------
+// dlogits on chip
+// ------------------------------------------------------------------------------------------
+// The softmax part of dlogits, without the factors that belong to a whole row, is
+//   D_iv = (1 - t^2) e^{z - cap} = 4 r (1 - r) e^{z - cap},  r = 1 / (1 + e^{2u/cap}),   0 <= D <= 1,
+// and  du_iv = rho_i D_iv - (one-hot terms),  rho_i = g_i S_i e^{cap - lse_i}.  D is kept in e4m3 with one power-of-two
+// exponent per block of 32 rows i x 128 columns v (MX style: byte * 2^(E - 127), E in an E8M0 byte), taken from the
+// block's own largest logit, so that neither the row's final lse nor its maximum has to be known when the block is
+// formed -- the forward pass can emit it -- and a peak in one place of a row costs the rest of the row nothing.  The
+// dX and dW GEMMs apply the exponents inside the matrix instruction (mfma_mainloop, SCALE).
+// Rows of very different temperature may share a block (a row whose logits saturate the cap next to ordinary ones:
+// D near 0.05 next to D near e^{-cap}), and 8 bits cannot hold both at one exponent.  So each row also has a boost of
+// its own, D_iv 2^{lam_i} is what is stored, with lam_i an integer estimated before the forward pass from a sample of
+// the row's logits (fwd_sample_kernel) and undone exactly in rho_i.  The block exponent is taken after the boost, so
+// a poor estimate costs precision, never range.
+//
+// Layout: G^T, tile by tile ([v tile][K block of 128 rows i][256 v][128 i] bytes): the B operand of dW as it lies,
+// and of dX through the transposing LDS read.  Exponents: one dword per (128 v, 128 i), byte c for rows [32 c, 32 c + 32),
+// as gexp[v / 128][i / 128].
+//
+// One wave turns its 128 (v) x 128 (i) quadrant of a finished logit tile into its quadrant of the staging tile TT
+// ([256 v][STG_PITCH], rows i contiguous) in LDS and returns the dword of exponents of its four 32-row blocks.  The
+// transposition happens in registers: the four lanes of a quad hold four consecutive rows of the same four
+// columns, and two quad-permute + byte-permute steps turn that 4 x 4 byte block around.
+// STATS: the forward pass's row statistics as well (sum of e^{z - cap}, largest raw logit and its column), kept in
+// `stat` (LDS, 12 floats per lane: [sum, max, argmax][4 row blocks], NTHREADS apart).
+constexpr int STG_PITCH = 272;                               // 256 + 16: 16-byte aligned, rows shifted by 4 banks
+constexpr int STG_BYTES = 256 * STG_PITCH;                   // 69632
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// lam (LDS, one float per lane and row block, LAM_STRIDE floats apart): the row's exponent boost (see fwd_sample_kernel).
+template <bool EDGE, bool STATS, int LAM_STRIDE = NTHREADS>
+__device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float k1, float c2, int vlim, int vabs0,
+                                                 uint8_t* TT, int wa, int wb, float* stat, const float* lam) {
+  const int lane = lane_id();
+  const int vloc0 = wa * 128 + 4 * (lane >> 5);       // column (within the tile) of accumulator register 0 of block a = 0
+  const int k = lane & 3;
+  const uint32_t sel1 = (k & 1) ? 0x03070105u : 0x06020400u;
+  const uint32_t sel2 = (k & 2) ? 0x03020706u : 0x05040100u;
+  uint32_t expword = 0;
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int iloc = wb * 128 + b * 32 + (lane & 31);        // row within the tile
+    // the block's largest logit fixes its exponent: D * 2^s <= 2^(lg + s) <= 446 with lg = log2 e^{zmax - cap}
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float x = acc[a][b][r];
+        if (EDGE && vloc0 + a * 32 + 8 * (r >> 2) + (r & 3) >= vlim) x = -INFINITY;
+        tmax = fmaxf(tmax, x);
+      }
+    const float lamb = lam[b * LAM_STRIDE];
+    const float lg = wave_max(fmaf(c2, fast_rcp(1.0f + fast_exp2(tmax * k1)), lamb));      // over the block: log2 of the largest boosted e^{z - cap}
+    const float sb = floorf(8.8f - lg);                       // between -120 and 8 + 2 cap log2(e) <= 124 (cap <= 40, boost <= 120)
+    const float cs = sb + 2.0f + lamb;                        // the 4 of 4 r (1 - r) and the row's boost ride along
+    expword |= (uint32_t)(127 - (int)sb) << (8 * b);
+    float ssum = 0.f;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      // stage by stage over the 16 values of the block: the transcendental unit is pipelined, a chain
+      // of dependent exp2 / rcp / exp2 on one value at a time is not (the scheduler would rebuild the
+      // chains to save registers, hence the barriers)
+      constexpr int NB = 8;        // values per batch: 4, 8 and 16 measure alike
+      float rr[16], gg[16];
+#pragma unroll
+      for (int g0 = 0; g0 < 16; g0 += NB) {
+#pragma unroll
+        for (int m = g0; m < g0 + NB; ++m) rr[m] = fast_exp2(acc[a][b][m] * k1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = g0; m < g0 + NB; ++m) rr[m] = fast_rcp(rr[m] + 1.0f);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = g0; m < g0 + NB; ++m) gg[m] = fast_exp2(fmaf(c2, rr[m], cs));
+        __builtin_amdgcn_sched_barrier(0);
+        if (EDGE) {
+#pragma unroll
+          for (int m = g0; m < g0 + NB; ++m) gg[m] = (vloc0 + a * 32 + 8 * (m >> 2) + (m & 3) >= vlim) ? 0.f : gg[m];
+        }
+        if (STATS) {
+#pragma unroll
+          for (int m = g0; m < g0 + NB; ++m) ssum += gg[m];
+        }
+#pragma unroll
+        for (int m = g0; m < g0 + NB; ++m) gg[m] *= rr[m] - rr[m] * rr[m];
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int vloc = vloc0 + a * 32 + 8 * q;
+        const uint32_t w = cvt4_e4m3(gg[4 * q], gg[4 * q + 1], gg[4 * q + 2], gg[4 * q + 3]);
+        // 4 x 4 byte transpose inside the quad: lane k ends up with column vloc + k, rows (iloc & ~3) .. +3
+        const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xB1, 0xF, 0xF, true);     // lane ^ 1
+        const uint32_t x = __builtin_amdgcn_perm(p1, w, sel1);
+        const uint32_t p2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, true);     // lane ^ 2
+        const uint32_t yv = __builtin_amdgcn_perm(p2, x, sel2);
+        *reinterpret_cast<uint32_t*>(TT + (vloc + k) * STG_PITCH + (iloc & ~3)) = yv;
+      }
+    }
+    if (STATS) {
+      stat[(0 + b) * NTHREADS] += ssum * fast_exp2(-cs);
+      const float amax = stat[(4 + b) * NTHREADS];
+      // the column of the maximum is looked up only when a tile reaches a lane's running maximum (on a tie the lower
+      // column wins: the running one may be a target of this very tile, which take_target_logits has put there)
+      if (__builtin_amdgcn_ballot_w64(tmax >= amax) != 0) {
+        if (tmax >= amax) {
+          int targ = 0x7fffffff;
+#pragma unroll
+          for (int a = 3; a >= 0; --a) {
+#pragma unroll
+            for (int r = 15; r >= 0; --r) {
+              const int vo = a * 32 + 8 * (r >> 2) + (r & 3);
+              if (acc[a][b][r] == tmax && (!EDGE || vloc0 + vo < vlim)) targ = vo;   // descending scan: lowest column wins
+            }
+          }
+          if (tmax > amax || (targ != 0x7fffffff && vabs0 + targ < __float_as_int(stat[(8 + b) * NTHREADS]))) {
+            stat[(4 + b) * NTHREADS] = tmax;
+            stat[(8 + b) * NTHREADS] = __int_as_float(vabs0 + targ);
+          }
+        }
+      }
+    }
+  }
+  return expword;
+}
+
+// The wave's quadrant of the staging tile (128 columns v x 128 rows i) is one contiguous 16 KB run of G^T: out in
+// 16-byte stores.  A wave reads only what it wrote itself, so no barrier is needed between forming and storing.
+__device__ __forceinline__ void store_dlogits_quadrant(const uint8_t* TT, uint8_t* gcol, int wa, int wb) {
+  const int lane = lane_id();
+  const uint8_t* tq = TT + wa * 128 * STG_PITCH + wb * 128;
+#pragma unroll
+  for (int n = 0; n < 16; ++n) {
+    const int cidx = lane + 64 * n, row = cidx >> 3, col = (cidx & 7) * 16;
+    *reinterpret_cast<v4i*>(gcol + row * BK + col) = *reinterpret_cast<const v4i*>(tq + row * STG_PITCH + col);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // forward
 // ------------------------------------------------------------------------------------------
 struct FwdParams {
   const uint8_t* xq;       // [Np][dp]
   const uint8_t* wqt;      // [Vp][dp]
   float4* partials;        // [S][Np]: sum exp(z - cap), max u, argmax u (bits), unused
+  const int64_t* targets;  // (N,)
+  float* s_uy;             // [n_predict][Np]: raw logit u at the target of (offset, row), written by the workgroup that meets it
+  uint8_t* ghat_t;         // EMIT: G^T, all Np rows (K blocks per v tile: kbw)
+  uint32_t* gexp;          // EMIT: its block exponents [Vp / 128][kbw]
+  const float* lam;        // EMIT: exponent boost of every row
+  int64_t ignore_index;
   int64_t dp, ldx;         // K extent and row stride of xq / wqt
-  int N, V, Np, RT, CT, S;
+  int64_t kbw;
+  int N, V, Np, RT, CT, S, n_predict;      // V: columns that take part; CT: column tiles walked (EMIT: all of Vp / 256)
   float sc;                // x_s * w_s
   float k1;                // x_s * w_s * 2 log2(e) / cap : exp2(acc * k1) = e^{2u/cap}
   float ic2;               // 1 / c2, c2 = -2 cap log2(e): e^{z - cap} = exp2(c2 / (1 + e^{2u/cap}))
+  float c2;
 };
 
 // Per 256 x 256 tile and per row a lane owns: add up e^{z - cap} over its 64 columns and keep the
@@ -423,53 +576,204 @@ __device__ __forceinline__ void fwd_epilogue(const v16f (&acc)[4][4], const FwdP
   }
 }
 
-// The row statistics of a workgroup's walk (12 values per lane) wait in LDS behind the two K slots while the
-// main loop runs: kept in registers they are spilled around it, and the reload (a vector memory load) makes
-// the epilogue wait for the tile loads that were just put in flight for the next tile.
-constexpr int SMEM_FWD = SMEM_BYTES + 12 * 4 * NTHREADS;
+__device__ __forceinline__ bool target_valid(const int64_t* __restrict__ targets, int64_t ignore_index, int i, int N, int V) {
+  if (i >= N) return false;
+  const int64_t y = targets[i];
+  return (y != ignore_index) && y >= 0 && y < V;
+}
 
+// The raw logit at a row's targets, taken from the accumulators of the tile that holds the target column, so that z_y
+// and lse come from the same numbers: the fp8 matrix instruction sums with less than fp32 care (about 2e-5 low on a
+// sum of like-signed terms), and a z_y from a separate fp32 dot product would leave that bias in z_y - lse, i.e. in
+// 1 - p_y, where rows the model is sure of cannot afford it.  tgt (LDS): [4 offsets][TGT_STRIDE rows] target column or
+// -1, already at the wave's first row.  A lane looks at its four rows; the 64-way select runs only when some lane of
+// the wave has a hit (a few per cent of the tiles).
+// STORE: the logit goes to s_uy_tile[offset][row] (global).
+// KNOCK: the accumulator of the target is then set to -inf, for the dlogits epilogue that follows: the target takes
+//        no part in the stored dlogits (its column is handled in fp32, see bwd_prep_kernel) and must not set the
+//        exponent of its block either -- a row the model is sure of would push its own other columns, and its
+//        neighbours', out of the 8 bits.
+// STATS: with KNOCK, the row statistics (stat, as in form_dlogits) take the target's share here: e^{z_y - cap} into the
+//        sum, and the running maximum / argmax.
+template <bool STORE, bool KNOCK, bool STATS, int TGT_STRIDE>
+__device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int* tgt, int n_predict, int col0, int rowbase,
+                                                   float sc, float* s_uy_tile, int Np, float* stat, float k1, float ic2) {
+  const int lane = lane_id(), half = lane >> 5;
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int row = b * 32 + (lane & 31);
+    float xk[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < n_predict; ++k) {
+      const int y = tgt[k * TGT_STRIDE + row];
+      const int rel = y - col0;                        // column within the wave's 128
+      const bool hit = (unsigned)rel < 128u && ((rel >> 2) & 1) == half;
+      if (__builtin_amdgcn_ballot_w64(hit) != 0) {
+        if (hit) {
+          const int idx = (rel >> 5) * 16 + ((rel >> 3) & 3) * 4 + (rel & 3);
+          float x = 0.f;
+          bool again = false;                          // an earlier offset of this row has the same target
+          if (KNOCK) {
+            for (int k2 = 0; k2 < k; ++k2)
+              if (tgt[k2 * TGT_STRIDE + row] == y) { again = true; x = xk[k2]; }
+          }
+          if (!again) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+              for (int r = 0; r < 16; ++r) {
+                x = (idx == a * 16 + r) ? acc[a][b][r] : x;
+                if (KNOCK) acc[a][b][r] = (idx == a * 16 + r) ? -INFINITY : acc[a][b][r];
+              }
+            if (KNOCK && STATS) {
+              // (the -inf left behind reads as z = -cap to the epilogue that follows, which will add e^{-2 cap} for it)
+              stat[(0 + b) * NTHREADS] += fast_exp2(fast_rcp(fmaf(fast_exp2(x * k1), ic2, ic2))) - fast_exp2(fast_rcp(ic2));
+              const float amax = stat[(4 + b) * NTHREADS];
+              if (x > amax || (x == amax && y < __float_as_int(stat[(8 + b) * NTHREADS]))) {
+                stat[(4 + b) * NTHREADS] = x;
+                stat[(8 + b) * NTHREADS] = __int_as_float(y);
+              }
+            }
+          }
+          xk[k] = x;
+          if (STORE) s_uy_tile[(int64_t)k * Np + rowbase + row] = x * sc;
+        }
+      }
+    }
+  }
+}
+
+// The exponent boost of every row, from one tile of its logits (256 columns from the middle of the vocabulary):
+// lam_i = floor(-log2 m_i), m_i the smallest of the means of e^{z - cap} over 16 groups of 16 columns -- the smallest,
+// so that a few peaks inside the sample (a target, say) do not pass for the level of the row.  One workgroup per row tile.
+__global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p, int ct, float* __restrict__ lam_out) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int rt = blockIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wa = wave >> 1, wb = wave & 1;
+  v16f acc[4][4];
+  mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 0, 0, wave);
+  const int lane = lane_id();
+  const int vlim = p.V - ct * 256, vloc0 = wa * 128 + 4 * (lane >> 5);
+  float gmin[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    gmin[b] = INFINITY;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      float sum = 0.f, cnt = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float pt = fast_exp2(fast_rcp(fmaf(fast_exp2(acc[a][b][r] * p.k1), p.ic2, p.ic2)));
+        const bool live = vloc0 + a * 32 + 8 * (r >> 2) + (r & 3) < vlim;
+        sum += live ? pt : 0.f;
+        cnt += live ? 1.f : 0.f;
+      }
+      if (cnt > 0.f) gmin[b] = fminf(gmin[b], sum / cnt);
+    }
+    gmin[b] = fminf(gmin[b], __shfl_xor(gmin[b], 32));
+  }
+  float* red = reinterpret_cast<float*>(smem);          // free: the main loop has ended in every wave
+  if (wa == 1 && lane < 32) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) red[wb * 128 + b * 32 + lane] = gmin[b];
+  }
+  __syncthreads();
+  if (wa == 0 && lane < 32) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const float m = fminf(gmin[b], red[wb * 128 + b * 32 + lane]);
+      float l = floorf(-log2f(m));
+      l = l > 0.f ? (l < 120.f ? l : 120.f) : 0.f;           // also: NaN -> 0
+      lam_out[rt * 256 + wb * 128 + b * 32 + lane] = l;
+    }
+  }
+}
+
+// LDS of the forward kernel: the two K slots; with EMIT the staging tile of the dlogits in the second slot (reaching
+// 4 KB beyond it); the row statistics of the workgroup's walk (12 values per lane, and the boosts of its rows: kept in registers they are spilled
+// around the main loop, and the reload -- a vector memory load -- makes the epilogue wait for the tile loads that were
+// just put in flight for the next tile); the targets of the workgroup's 256 rows.
+constexpr int FWD_STAGE_OFF = SLOT_BYTES;
+constexpr int FWD_STAT_OFF = SMEM_MAX - 4096 - 16 * 4 * NTHREADS;      // 12 statistics and the boosts of the lane's 4 rows
+constexpr int FWD_TGT_OFF = SMEM_MAX - 4096;
+constexpr int SMEM_FWD = SMEM_MAX;
+static_assert(FWD_STAGE_OFF + STG_BYTES <= FWD_STAT_OFF, "staging tile and row statistics overlap");
+
+// EMIT: the epilogue also leaves the block-scaled dlogits of the tile in G^T (see form_dlogits), for a backward pass
+// that does not compute the logits again.
+template <bool EMIT>
 __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   int rt, s;
   if (!map_tile(blockIdx.x, p.RT, p.S, rt, s)) return;
   const int ct0 = (int)((int64_t)p.CT * s / p.S), ct1 = (int)((int64_t)p.CT * (s + 1) / p.S);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wa = wave >> 1, wb = wave & 1;
-  float* stat = reinterpret_cast<float*>(smem + SMEM_BYTES) + wave * 64 + lane_id();   // [12][256]: sum, amax, uarg of the 4 row blocks
+  {
+    float* stat = reinterpret_cast<float*>(smem + FWD_STAT_OFF) + wave * 64 + lane_id();   // [12][256]: sum, amax, uarg of the 4 row blocks
 #pragma unroll
-  for (int b = 0; b < 4; ++b) {
-    stat[(0 + b) * NTHREADS] = 0.f;
-    stat[(4 + b) * NTHREADS] = -INFINITY;
-    stat[(8 + b) * NTHREADS] = __int_as_float(0x7fffffff);
+    for (int b = 0; b < 4; ++b) {
+      stat[(0 + b) * NTHREADS] = 0.f;
+      stat[(4 + b) * NTHREADS] = -INFINITY;
+      stat[(8 + b) * NTHREADS] = __int_as_float(0x7fffffff);
+      if (EMIT) stat[(12 + b) * NTHREADS] = p.lam[rt * 256 + wb * 128 + b * 32 + (lane_id() & 31)];
+    }
+    int* tgt = reinterpret_cast<int*>(smem + FWD_TGT_OFF);
+    for (int e = threadIdx.x; e < p.n_predict * 256; e += NTHREADS) {
+      const int i = rt * 256 + (e & 255) + (e >> 8);
+      tgt[e] = ((e & 255) + rt * 256 < p.N && target_valid(p.targets, p.ignore_index, i, p.N, p.V)) ? (int)p.targets[i] : -1;
+    }
   }
+  __syncthreads();
   v16f acc[4][4];
   const uint8_t* Bg = p.xq + (int64_t)rt * 256 * p.ldx;
   const int KT = (int)(p.dp / BK);
   // of the workgroups that start together on this XCD, those with the same split share the W tiles, those with the same rt the X rows
   const int rot_a = 2 * (rt & 3), rot_b = s & 7;
-  // the first K blocks of the next tile travel while the epilogue of this one runs (it does not touch the K slots)
+  // the first K blocks of the next tile travel while the epilogue of this one runs (it does not touch the K slots;
+  // with EMIT it uses the second one, so only the first block travels and the rest follows after the epilogue)
   if (ct0 < ct1) mfma_prefetch(p.wqt + (int64_t)ct0 * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
   for (int ct = ct0; ct < ct1; ++ct) {
-    mfma_mainloop<true>(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, Bg, p.ldx, KT, smem, acc, rot_a, rot_b, wave);
-    if (ct + 1 < ct1) mfma_prefetch(p.wqt + (int64_t)(ct + 1) * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
-    float sum[4], amax[4];
-    int uarg[4];
-    float* stat = reinterpret_cast<float*>(smem + SMEM_BYTES) + wave * 64 + lane_id();
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      sum[b] = stat[(0 + b) * NTHREADS]; amax[b] = stat[(4 + b) * NTHREADS]; uarg[b] = __float_as_int(stat[(8 + b) * NTHREADS]);
-    }
+    mfma_mainloop<true>(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, Bg, p.ldx, KT, smem, acc, rot_a, rot_b, wave, NoHook(), 0, 0, nullptr,
+                        EMIT && ct > ct0);
+    const uint8_t* Anext = p.wqt + (int64_t)(ct + 1) * 256 * p.ldx;
+    if (ct + 1 < ct1) mfma_prefetch<EMIT ? 1 : 3>(Anext, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
+    float* stat = reinterpret_cast<float*>(smem + FWD_STAT_OFF) + wave * 64 + lane_id();
     const int vbase = ct * 256 + wa * 128 + 4 * (lane_id() >> 5);
-    if (ct * 256 + 256 > p.V) fwd_epilogue<true>(acc, p, vbase, sum, amax, uarg);
-    else fwd_epilogue<false>(acc, p, vbase, sum, amax, uarg);
+    const int* tgt = reinterpret_cast<const int*>(smem + FWD_TGT_OFF) + wb * 128;
+    if (EMIT) {
+      take_target_logits<true, true, true, 256>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2);
+      const int vlim = p.V - ct * 256;
+      uint8_t* TT = smem + FWD_STAGE_OFF;
+      uint32_t ew;
+      if (vlim < 256) ew = form_dlogits<true, true>(acc, p.k1, p.c2, vlim, vbase, TT, wa, wb, stat, stat + 12 * NTHREADS);
+      else ew = form_dlogits<false, true>(acc, p.k1, p.c2, vlim, vbase, TT, wa, wb, stat, stat + 12 * NTHREADS);
+      store_dlogits_quadrant(TT, p.ghat_t + ((int64_t)ct * p.kbw + 2 * rt + wb) * BLOCKED_KSTEP + wa * 128 * BK, wa, wb);
+      if (lane_id() == 0) p.gexp[(int64_t)(2 * ct + wa) * p.kbw + 2 * rt + wb] = ew;
+    } else {
+      float sum[4], amax[4];
+      int uarg[4];
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      stat[(0 + b) * NTHREADS] = sum[b]; stat[(4 + b) * NTHREADS] = amax[b]; stat[(8 + b) * NTHREADS] = __int_as_float(uarg[b]);
+      for (int b = 0; b < 4; ++b) {
+        sum[b] = stat[(0 + b) * NTHREADS]; amax[b] = stat[(4 + b) * NTHREADS]; uarg[b] = __float_as_int(stat[(8 + b) * NTHREADS]);
+      }
+      if (ct * 256 + 256 > p.V) fwd_epilogue<true>(acc, p, vbase, sum, amax, uarg);
+      else fwd_epilogue<false>(acc, p, vbase, sum, amax, uarg);
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        stat[(0 + b) * NTHREADS] = sum[b]; stat[(4 + b) * NTHREADS] = amax[b]; stat[(8 + b) * NTHREADS] = __int_as_float(uarg[b]);
+      }
+    }
+    if (!EMIT) take_target_logits<true, false, false, 256>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, nullptr, 0.f, 0.f);
+    if (EMIT && ct + 1 < ct1) {
+      // every wave has read its part of the staging tile (its stores have their data) before the second K slot fills again
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      mfma_prefetch<2>(Anext, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
     }
   }
+  if (EMIT) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");     // the staging tile gives way to the reduction below
   float sum[4], amax[4];
   int uarg[4];
   const int lane = lane_id();
-  stat = reinterpret_cast<float*>(smem + SMEM_BYTES) + wave * 64 + lane;
+  float* stat = reinterpret_cast<float*>(smem + FWD_STAT_OFF) + wave * 64 + lane;
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
     sum[b] = stat[(0 + b) * NTHREADS]; amax[b] = stat[(4 + b) * NTHREADS]; uarg[b] = __float_as_int(stat[(8 + b) * NTHREADS]);
@@ -502,47 +806,6 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p) {
   }
 }
 
-// z at the targets: one wavefront per (row i, offset k) takes the dot product of X_q[i, :] with
-// W_q^T[y_{i+k}, :] (both contiguous) and applies the softcap.  Offsets index the flattened target
-// vector, as in the reference kernel (tiny/cuda_kernels.py:229).  Pairs that take no part get 0.
-__global__ __launch_bounds__(256) void fwd_target_logit_kernel(const uint8_t* __restrict__ xq, const uint8_t* __restrict__ wqt,
-                                                              int64_t dp, int64_t ldx, const int64_t* __restrict__ targets,
-                                                              int64_t ignore_index, int N, int Np, int V, float sc, float cap,
-                                                              float* __restrict__ s_zy) {
-  const int lane = threadIdx.x & 63;
-  const int i = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int k = blockIdx.y;
-  if (i >= N) return;
-  const int64_t y = (i + k < N) ? targets[i + k] : ignore_index;
-  const bool valid = (y != ignore_index) && y >= 0 && y < V;
-  float acc = 0.f;
-  if (valid) {
-    const uint8_t* xr = xq + (int64_t)i * ldx;
-    const uint8_t* wr = wqt + y * ldx;
-    for (int64_t c = lane * 16; c < dp; c += 64 * 16) {
-      const v4i xa = *reinterpret_cast<const v4i*>(xr + c);
-      const v4i wa = *reinterpret_cast<const v4i*>(wr + c);
-#pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        const uint32_t xw = (uint32_t)xa[m], ww = (uint32_t)wa[m];
-        acc = fmaf(e4m3_to_float<0>(xw), e4m3_to_float<0>(ww), acc);
-        acc = fmaf(e4m3_to_float<1>(xw), e4m3_to_float<1>(ww), acc);
-        acc = fmaf(e4m3_to_float<2>(xw), e4m3_to_float<2>(ww), acc);
-        acc = fmaf(e4m3_to_float<3>(xw), e4m3_to_float<3>(ww), acc);
-      }
-    }
-  }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
-  if (lane == 0) s_zy[(int64_t)k * Np + i] = valid ? cap * tanhf(acc * sc / cap) : 0.f;
-}
-
-__device__ __forceinline__ bool target_valid(const int64_t* __restrict__ targets, int64_t ignore_index, int i, int N, int V) {
-  if (i >= N) return false;
-  const int64_t y = targets[i];
-  return (y != ignore_index) && y >= 0 && y < V;
-}
-
 // What a block of 256 rows contributes to the mean loss: left by fwd_combine_kernel in the first 16 bytes of the
 // block's own rows of the partial records (which it has consumed by then), summed by fwd_reduce_kernel.
 struct BlockLoss {
@@ -557,7 +820,7 @@ __global__ __launch_bounds__(256) void fwd_combine_kernel(float4* __restrict__ p
                                                          const int64_t* __restrict__ targets, int64_t ignore_index, float cap,
                                                          const float* __restrict__ mtp_weights, int n_predict,
                                                          float* __restrict__ s_lse, float* __restrict__ s_umax,
-                                                         const float* __restrict__ s_zy, float* __restrict__ losses,
+                                                         float* __restrict__ s_zy, float* __restrict__ losses,
                                                          float* __restrict__ lse_out, int32_t* __restrict__ argmax_out) {
   __shared__ double ssum[256];
   __shared__ int scnt[256], sbad[256];
@@ -566,6 +829,7 @@ __global__ __launch_bounds__(256) void fwd_combine_kernel(float4* __restrict__ p
   int cnt = 0, bad = 0;
   if (i >= N) {
     s_lse[i] = 0.f; s_umax[i] = 0.f;
+    for (int k = 0; k < n_predict; ++k) s_zy[(int64_t)k * Np + i] = 0.f;
   } else {
     float sum = 0.f, umax = -INFINITY;
     int uarg = 0x7fffffff;
@@ -577,14 +841,18 @@ __global__ __launch_bounds__(256) void fwd_combine_kernel(float4* __restrict__ p
     }
     const float lse = cap + logf(sum);
     s_lse[i] = lse; s_umax[i] = umax;
-    if (losses) {
-      // loss_i = sum_k w_k (lse_i - z[i, y_{i+k}]) over the offsets that take part (tiny/cuda_kernels.py:226-240)
-      float l = 0.f;
-      for (int k = 0; k < n_predict; ++k)
-        if (target_valid(targets, ignore_index, i + k, N, V))
-          l += (mtp_weights ? mtp_weights[k] : 1.0f) * (lse - s_zy[(int64_t)k * Np + i]);
-      losses[i] = l;
+    // the forward kernel left the raw logit at each target that takes part: z_y = cap tanh(u_y / cap) replaces it (0 for the others);
+    // loss_i = sum_k w_k (lse_i - z[i, y_{i+k}]) over the offsets that take part (tiny/cuda_kernels.py:226-240)
+    float l = 0.f;
+    for (int k = 0; k < n_predict; ++k) {
+      float zy = 0.f;
+      if (target_valid(targets, ignore_index, i + k, N, V)) {
+        zy = cap * tanhf(s_zy[(int64_t)k * Np + i] / cap);
+        l += (mtp_weights ? mtp_weights[k] : 1.0f) * (lse - zy);
+      }
+      s_zy[(int64_t)k * Np + i] = zy;
     }
+    if (losses) losses[i] = l;
     if (lse_out) lse_out[i] = lse;
     if (argmax_out) argmax_out[i] = (uarg == 0x7fffffff) ? 0 : uarg;
     const int64_t y = targets[i];
@@ -639,8 +907,8 @@ __global__ __launch_bounds__(1024) void fwd_reduce_kernel(const float4* __restri
 // ------------------------------------------------------------------------------------------
 // per row: rho (row factor of the block-scaled dlogits) and h_k (one-hot coefficients).
 //   dz_iv = g_i ( S_i p_iv - sum_k w_k [v = y_{i+k}] ),  S_i = sum of w_k over the offsets that take part,
-//   S_i p_iv (1 - t^2) = rho_i D_iv  with  rho_i = g_i S_i e^{cap - lse_i}.
-// The target columns take no part in D (bwd_zero_targets_kernel clears them): their S_i p_iy goes into the
+//   S_i p_iv (1 - t^2) = rho_i (D_iv 2^{lam_i})  with  rho_i = g_i S_i e^{cap - lse_i} 2^{-lam_i}.
+// The target columns take no part in D (take_target_logits knocks them out where D is formed): their S_i p_iy goes into the
 // one-hot coefficient instead, h_ik = g_i (1 - t_y^2) (w_k - S_i p_iy), formed here in fp32 from lse and z_y.
 // Through e4m3 the difference S_i p_iy - w_k would carry the rounding error of p_iy alone, a relative
 // error of eps p / (1 - p) that grows without bound on rows the model is sure of.  When two offsets of a row
@@ -650,13 +918,18 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__
                                                       int64_t ignore_index, const int32_t* __restrict__ hdr,
                                                       const float* __restrict__ grad_output, int per_row, float grad_scale,
                                                       const float* __restrict__ mtp_weights, int n_predict,
-                                                      float cap, int N, int Np, int V,
+                                                      float cap, int N, int Np, int V, const float* __restrict__ lam,
                                                       float* __restrict__ rho, float* __restrict__ hcoef,
-                                                      float* __restrict__ blockmax) {
+                                                      float* __restrict__ blockmax, int32_t* __restrict__ rowinfo) {
   __shared__ float smax[256];
   const int i = blockIdx.x * 256 + threadIdx.x;
   float r = 0.f;
   float h[4] = {0.f, 0.f, 0.f, 0.f};
+  if (rowinfo && i < Np) {          // what the recompute kernel wants to know of a row: its boost and its target columns
+    rowinfo[i] = __float_as_int(i < N ? lam[i] : 0.f);
+    for (int k = 0; k < 4; ++k)
+      rowinfo[(int64_t)(1 + k) * Np + i] = (k < n_predict && i < N && target_valid(targets, ignore_index, i + k, N, V)) ? (int)targets[i + k] : -1;
+  }
   if (i < N) {
     const float g = (per_row ? grad_output[i] : grad_output[0] / (float)hdr[0]) * grad_scale;
     float sw = 0.f;
@@ -679,7 +952,7 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__
         for (int k2 = 0; k2 < k; ++k2) first = first && !(ok[k2] && yk[k2] == yk[k]);
         h[k] = g * (1.0f - ty * ty) * (wk - (first ? sw * expf(zy - lse) : 0.f));
       }
-      r = g * sw * expf(cap - lse);
+      r = ldexpf(g * sw * expf(cap - lse), -(int)lam[i]);      // the stored dlogits carry the row's boost 2^lam
     }
   }
   if (i < Np) {
@@ -693,18 +966,6 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__
     __syncthreads();
   }
   if (threadIdx.x == 0) blockmax[blockIdx.x] = smax[0];
-}
-
-// Clears the target columns of the rows [i0, i0 + rows) in G^T (blocked; `g` points at the K block of row i0):
-// one thread per (offset, row) pair, one byte each.  Runs between the kernel that forms G and its readers.
-__global__ __launch_bounds__(256) void bwd_zero_targets_kernel(const int64_t* __restrict__ targets, int64_t ignore_index,
-                                                              int i0, int rows, int N, int V, int n_predict,
-                                                              uint8_t* __restrict__ g, int64_t kbw) {
-  const int e = blockIdx.x * 256 + threadIdx.x;
-  if (e >= rows * n_predict) return;
-  const int k = e / rows, il = e - k * rows;
-  if (!target_valid(targets, ignore_index, i0 + il + k, N, V)) return;
-  g[blocked_offset(targets[i0 + il + k], il, kbw)] = 0;
 }
 
 __global__ __launch_bounds__(1024) void bwd_xi_kernel(const float* __restrict__ blockmax, int n, float* __restrict__ xi) {
@@ -752,147 +1013,14 @@ __global__ __launch_bounds__(256) void bwd_xt_kernel(const uint8_t* __restrict__
   *reinterpret_cast<v4i*>(xt + blocked_offset(j0 + jr, i0 + ic, kbn)) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
 }
 
-// ------------------------------------------------------------------------------------------
-// dlogits on chip
-// ------------------------------------------------------------------------------------------
-// The softmax part of dlogits, without the factors that belong to a whole row, is
-//   D_iv = (1 - t^2) e^{z - cap} = 4 r (1 - r) e^{z - cap},  r = 1 / (1 + e^{2u/cap}),   0 <= D <= 1,
-// and  du_iv = rho_i D_iv - (one-hot terms),  rho_i = g_i S_i e^{cap - lse_i}.  D is kept in e4m3 with one power-of-two
-// exponent per block of 32 rows i x 128 columns v (MX style: byte * 2^(E - 127), E in an E8M0 byte), taken from the
-// block's own largest logit, so that neither the row's final lse nor its maximum has to be known when the block is
-// formed -- the forward pass can emit it -- and a peak in one place of a row costs the rest of the row nothing.  The
-// dX and dW GEMMs apply the exponents inside the matrix instruction (mfma_mainloop, SCALE).
-//
-// Layout: G^T, tile by tile ([v tile][K block of 128 rows i][256 v][128 i] bytes): the B operand of dW as it lies,
-// and of dX through the transposing LDS read.  Exponents: one dword per (128 v, 128 i), byte c for rows [32 c, 32 c + 32),
-// as gexp[v / 128][i / 128].
-//
-// One wave turns its 128 (v) x 128 (i) quadrant of a finished logit tile into its quadrant of the staging tile TT
-// ([256 v][STG_PITCH], rows i contiguous) in LDS and returns the dword of exponents of its four 32-row blocks.  The
-// transposition happens in registers: the four lanes of a quad hold four consecutive rows of the same four
-// columns, and two quad-permute + byte-permute steps turn that 4 x 4 byte block around.
-// STATS: the forward pass's row statistics as well (sum of e^{z - cap}, largest raw logit and its column), kept in
-// `stat` (LDS, 12 floats per lane: [sum, max, argmax][4 row blocks], NTHREADS apart).
-constexpr int STG_PITCH = 272;                               // 256 + 16: 16-byte aligned, rows shifted by 4 banks
-constexpr int STG_BYTES = 256 * STG_PITCH;                   // 69632
-
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
-}
-
-template <bool EDGE, bool STATS>
-__device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float k1, float c2, int vlim, int vabs0,
-                                                 uint8_t* TT, int wa, int wb, float* stat) {
-  const int lane = lane_id();
-  const int vloc0 = wa * 128 + 4 * (lane >> 5);       // column (within the tile) of accumulator register 0 of block a = 0
-  const int k = lane & 3;
-  const uint32_t sel1 = (k & 1) ? 0x03070105u : 0x06020400u;
-  const uint32_t sel2 = (k & 2) ? 0x03020706u : 0x05040100u;
-  uint32_t expword = 0;
-#pragma unroll
-  for (int b = 0; b < 4; ++b) {
-    const int iloc = wb * 128 + b * 32 + (lane & 31);        // row within the tile
-    // the block's largest logit fixes its exponent: D * 2^s <= 2^(lg + s) <= 446 with lg = log2 e^{zmax - cap}
-    float tmax = -INFINITY;
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float x = acc[a][b][r];
-        if (EDGE && vloc0 + a * 32 + 8 * (r >> 2) + (r & 3) >= vlim) x = -INFINITY;
-        tmax = fmaxf(tmax, x);
-      }
-    const float bmax = wave_max(tmax);
-    const float lg = c2 * fast_rcp(1.0f + fast_exp2(bmax * k1));
-    const float sb = floorf(8.8f - lg);                       // 8 .. 8 + 2 cap log2(e): at most 124 for cap <= 40
-    const float cs = sb + 2.0f;                               // the 4 of 4 r (1 - r) rides along
-    expword |= (uint32_t)(127 - (int)sb) << (8 * b);
-    float ssum = 0.f;
-#pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      // stage by stage over the 16 values of the block: the transcendental unit is pipelined, a chain
-      // of dependent exp2 / rcp / exp2 on one value at a time is not (the scheduler would rebuild the
-      // chains to save registers, hence the barriers)
-      constexpr int NB = 8;        // values per batch: 4, 8 and 16 measure alike
-      float rr[16], gg[16];
-#pragma unroll
-      for (int g0 = 0; g0 < 16; g0 += NB) {
-#pragma unroll
-        for (int m = g0; m < g0 + NB; ++m) rr[m] = fast_exp2(acc[a][b][m] * k1);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int m = g0; m < g0 + NB; ++m) rr[m] = fast_rcp(rr[m] + 1.0f);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int m = g0; m < g0 + NB; ++m) gg[m] = fast_exp2(fmaf(c2, rr[m], cs));
-        __builtin_amdgcn_sched_barrier(0);
-        if (EDGE) {
-#pragma unroll
-          for (int m = g0; m < g0 + NB; ++m) gg[m] = (vloc0 + a * 32 + 8 * (m >> 2) + (m & 3) >= vlim) ? 0.f : gg[m];
-        }
-        if (STATS) {
-#pragma unroll
-          for (int m = g0; m < g0 + NB; ++m) ssum += gg[m];
-        }
-#pragma unroll
-        for (int m = g0; m < g0 + NB; ++m) gg[m] *= rr[m] - rr[m] * rr[m];
-        __builtin_amdgcn_sched_barrier(0);
-      }
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int vloc = vloc0 + a * 32 + 8 * q;
-        const uint32_t w = cvt4_e4m3(gg[4 * q], gg[4 * q + 1], gg[4 * q + 2], gg[4 * q + 3]);
-        // 4 x 4 byte transpose inside the quad: lane k ends up with column vloc + k, rows (iloc & ~3) .. +3
-        const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xB1, 0xF, 0xF, true);     // lane ^ 1
-        const uint32_t x = __builtin_amdgcn_perm(p1, w, sel1);
-        const uint32_t p2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, true);     // lane ^ 2
-        const uint32_t yv = __builtin_amdgcn_perm(p2, x, sel2);
-        *reinterpret_cast<uint32_t*>(TT + (vloc + k) * STG_PITCH + (iloc & ~3)) = yv;
-      }
-    }
-    if (STATS) {
-      stat[(0 + b) * NTHREADS] += ssum * fast_exp2(-cs);
-      const float amax = stat[(4 + b) * NTHREADS];
-      // the column of the maximum is looked up only when a tile raises a lane's running maximum
-      if (__builtin_amdgcn_ballot_w64(tmax > amax) != 0) {
-        if (tmax > amax) {
-          int targ = 0x7fffffff;
-#pragma unroll
-          for (int a = 3; a >= 0; --a) {
-#pragma unroll
-            for (int r = 15; r >= 0; --r) {
-              const int vo = a * 32 + 8 * (r >> 2) + (r & 3);
-              if (acc[a][b][r] == tmax && (!EDGE || vloc0 + vo < vlim)) targ = vo;   // descending scan: lowest column wins
-            }
-          }
-          stat[(4 + b) * NTHREADS] = tmax;
-          stat[(8 + b) * NTHREADS] = __int_as_float(vabs0 + targ);
-        }
-      }
-    }
-  }
-  return expword;
-}
-
-// The wave's quadrant of the staging tile (128 columns v x 128 rows i) is one contiguous 16 KB run of G^T: out in
-// 16-byte stores.  A wave reads only what it wrote itself, so no barrier is needed between forming and storing.
-__device__ __forceinline__ void store_dlogits_quadrant(const uint8_t* TT, uint8_t* gcol, int wa, int wb) {
-  const int lane = lane_id();
-  const uint8_t* tq = TT + wa * 128 * STG_PITCH + wb * 128;
-#pragma unroll
-  for (int n = 0; n < 16; ++n) {
-    const int cidx = lane + 64 * n, row = cidx >> 3, col = (cidx & 7) * 16;
-    *reinterpret_cast<v4i*>(gcol + row * BK + col) = *reinterpret_cast<const v4i*>(tq + row * STG_PITCH + col);
-  }
-}
-
 struct RecomputeParams {
   const uint8_t* xq;     // [Np][dp], already offset to the panel's first row
   const uint8_t* wqt;    // [Vp][dp]
   uint8_t* ghat_t;       // Vp rows, K = 128 * kbw, blocked
   uint32_t* gexp;        // [Vp / 128][kbw]
+  const int32_t* rowinfo;      // [ROWINFO_PLANES][Np], offset to the panel's first row: boosts and targets (bwd_prep_kernel)
+  int64_t Np;
+  int n_predict;
   int64_t dp, ldx;             // K extent and row stride of xq / wqt
   int64_t kbw, kb0;            // ghat_t (blocked): K blocks per tile, K block of this panel's first row
   int RT, CT, V;
@@ -901,7 +1029,9 @@ struct RecomputeParams {
 
 // Recompute a 256 x 256 logit tile and leave its block-scaled dlogits in G^T.  The tile is assembled in LDS (free
 // once the main loop is done) and leaves the chip as 64 KB of consecutive 16-byte stores.
-constexpr int SMEM_RECOMPUTE = SMEM_BYTES > STG_BYTES ? SMEM_BYTES : STG_BYTES;
+constexpr int ROWINFO_PLANES = 5;                      // per row: exponent boost (a float), then the target column of each of 4 offsets (or -1)
+constexpr int SMEM_RECOMPUTE = SMEM_BYTES + 4 * ROWINFO_PLANES * 512;      // two K slots (the staging tile reuses them) + the row data of 128 rows per wave
+static_assert(STG_BYTES <= SMEM_BYTES, "the staging tile must fit the K slots");
 
 __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -912,12 +1042,29 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   // still in the memory-side cache.
   ct = p.CT - 1 - ct;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wa = wave >> 1, wb = wave & 1;
+  // The boosts and targets of the wave's 128 rows go straight to LDS, behind the two slots: requested before the K
+  // loop (whose waits for its own, younger loads cover them), read after it, no register held in between.
+  {
+    const uint32_t dst = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)(smem + SMEM_BYTES)) + wave * (ROWINFO_PLANES * 512);
+    const int voff = lane_id() * 4;
+#pragma unroll
+    for (int q = 0; q < ROWINFO_PLANES; ++q) {
+      const int32_t* src = p.rowinfo + (int64_t)q * p.Np + rt * 256 + wb * 128;
+      // the instruction's offset moves the memory address and the LDS address alike: the second half of the rows
+      asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %2, %3\n\t"
+                   "global_load_lds_dword %2, %3 offset:256"
+                   ::"s"(dst), "n"(q * 512), "v"(voff), "s"(src) : "memory", "scc");
+    }
+  }
   v16f acc[4][4];
   mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 2 * (rt & 3), ct & 7, wave);
   const int vlim = p.V - ct * 256;           // columns >= vlim of this tile do not exist
+  const float* lam = reinterpret_cast<const float*>(smem + SMEM_BYTES) + wave * (ROWINFO_PLANES * 128) + (lane_id() & 31);     // row block b: 32 floats on
+  const int* tgt = reinterpret_cast<const int*>(smem + SMEM_BYTES) + wave * (ROWINFO_PLANES * 128) + 128;
+  take_target_logits<false, true, false, 128>(acc, tgt, p.n_predict, ct * 256 + wa * 128, 0, 0.f, nullptr, 0, nullptr, 0.f, 0.f);
   uint32_t ew;
-  if (vlim < 256) ew = form_dlogits<true, false>(acc, p.k1, p.c2, vlim, 0, smem, wa, wb, nullptr);
-  else ew = form_dlogits<false, false>(acc, p.k1, p.c2, vlim, 0, smem, wa, wb, nullptr);
+  if (vlim < 256) ew = form_dlogits<true, false, 32>(acc, p.k1, p.c2, vlim, 0, smem, wa, wb, nullptr, lam);
+  else ew = form_dlogits<false, false, 32>(acc, p.k1, p.c2, vlim, 0, smem, wa, wb, nullptr, lam);
   store_dlogits_quadrant(smem, p.ghat_t + ((int64_t)ct * p.kbw + p.kb0 + 2 * rt + wb) * BLOCKED_KSTEP + wa * 128 * BK, wa, wb);
   if (lane_id() == 0) p.gexp[(int64_t)(2 * ct + wa) * p.kbw + p.kb0 + 2 * rt + wb] = ew;
 }
@@ -946,7 +1093,6 @@ struct DxParams {
 constexpr int DX_STAGE_BYTES = 128 * (64 * 4 + 16);
 constexpr int SMEM_DX = 4 * DX_STAGE_BYTES > SMEM_BYTES ? 4 * DX_STAGE_BYTES : SMEM_BYTES;
 // ... or the two K slots and, behind them, the block exponents of the K loop (one dword per K block and half of the rows)
-constexpr int SMEM_MAX = 160 * 1024;
 constexpr int MAX_SCALE_KBLOCKS = (SMEM_MAX - SMEM_BYTES) / 8;      // K blocks of one scaled main loop: 4096
 static inline int smem_scaled(int kblocks, int at_least) { const int n = SMEM_BYTES + 8 * kblocks; return n > at_least ? n : at_least; }
 
@@ -1435,7 +1581,9 @@ static int check_device(int dev) {
     g_cus[dev] = prop.multiProcessorCount;
     if (g_arch_ok[dev] == 1) {
       // the MFMA kernels hold two 64 KB K-slots in LDS
-      HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
+      HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
+      HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
+      HIP_TRY(hipFuncSetAttribute((const void*)fwd_sample_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_recompute_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_RECOMPUTE));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
@@ -1474,12 +1622,14 @@ static size_t sort_tmp_bytes(int64_t N, int64_t V) {
 // fp32 partial sums of a K-split dX panel: at most 256 tiles of 256 x 256
 constexpr size_t DX_PART_BYTES = (size_t)256 * 256 * 256 * 4;
 
-static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int nparts, int K) {
+// kept: the dlogits come with `saved` (the forward pass emitted them): no panel scratch here
+static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int nparts, int K, bool kept = false) {
   BwdLayout B;
   B.P = P; B.Pw = Pw; B.nparts = nparts;
   size_t o = 0;
   auto take = [&](size_t bytes) { size_t r = o; o += (bytes + 255) / 256 * 256; return r; };
   B.off_rho = take((size_t)S.Np * 4);
+  B.off_rowinfo = take((size_t)S.Np * 4 * ROWINFO_PLANES);
   B.off_hcoef = take((size_t)S.Np * 4 * K);
   B.off_blockmax = take((size_t)(S.Np / 256) * 4);
   B.off_xi = take(256);
@@ -1493,8 +1643,8 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int npa
   B.off_sorttmp = take(B.sorttmp_bytes);
   B.off_dxpart = take(DX_PART_BYTES);
   B.fixed = o;
-  B.off_ghat_t = take((size_t)S.Vp * Pw);
-  B.off_gexp = take((size_t)(S.Vp / 128) * (Pw / 128) * 4);      // block exponents of the dlogits
+  B.off_ghat_t = take(kept ? 0 : (size_t)S.Vp * Pw);
+  B.off_gexp = take(kept ? 0 : (size_t)(S.Vp / 128) * (Pw / 128) * 4);      // block exponents of the dlogits
   B.part_stride = ((size_t)S.dq * S.Vp * 4 + 255) / 256 * 256;
   B.off_dwacc = take(B.part_stride * (size_t)nparts);     // fp32 dW partials, one per dW launch
   B.total = o;
@@ -1586,6 +1736,8 @@ extern "C" int sce_sizes_for(const sce_shape* shape, sce_sizes* out) {
   {
     const int64_t Pw = default_dw_panel(S, out->bwd_panel_rows);
     out->bwd_workspace_bytes = bwd_layout(S, out->bwd_panel_rows, Pw, dw_launches(S, Pw), shape->n_predict).total;
+    out->dlogits_bytes = S.g_total;
+    out->bwd_workspace_kept_bytes = bwd_layout(S, out->bwd_panel_rows, Pw, dw_launches(S, Pw), shape->n_predict, true).total;
   }
   return SCE_OK;
 }
@@ -1657,9 +1809,8 @@ extern "C" int sce_forward(const sce_args* a) {
   if (a->wcache && a->wcache_bytes < S.w_total) return fail(SCE_EINVAL, "weight cache too small: %zu < %zu", a->wcache_bytes, S.w_total);
   const int64_t Vl = a->vocab_limit > 0 ? a->vocab_limit : V;       // columns that take part
   const int RT = (int)(S.Np / 256), CT = (int)((Vl + 255) / 256);
-  const int nsplit = fwd_splits(RT, CT, device_cus_or_default(a->device));
-  const size_t need_ws = (size_t)nsplit * S.Np * 16;
-  if (!a->workspace || a->workspace_bytes < need_ws) return fail(SCE_EINVAL, "forward workspace too small: %zu < %zu", a->workspace_bytes, need_ws);
+  const size_t gneed = need_saved + (a->dlogits_from_forward ? S.g_total : 0);
+  if (a->saved_bytes < gneed) return fail(SCE_EINVAL, "saved buffer too small for the dlogits: %zu < %zu", a->saved_bytes, gneed);
   DeviceGuard guard(a->device);
   if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", a->device);
   hipStream_t st = (hipStream_t)a->stream;
@@ -1668,6 +1819,7 @@ extern "C" int sce_forward(const sce_args* a) {
   uint8_t* wbase = a->wcache ? (uint8_t*)a->wcache : sv + S.x_total;
   uint8_t* wqt = wbase + S.rel_wqt;
   uint8_t* wq = wbase + S.rel_wq;
+  uint8_t* gbase = sv + need_saved;       // dlogits, when the forward pass emits them
 
   {
     KernelTimer tm(SCE_K_QUANT, st);
@@ -1692,21 +1844,34 @@ extern "C" int sce_forward(const sce_args* a) {
       quantize_w_kernel<bf16_t><<<gw, 256, 0, st>>>((const bf16_t*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.Vp / BK, (float)(1.0 / a->w_s));
     else return fail(SCE_EINVAL, "unsupported w dtype %d", a->w_dtype);
   }
+  const bool emit = a->dlogits_from_forward != 0;
+  const int CTw = emit ? (int)(S.Vp / 256) : CT;       // with the dlogits every tile is visited: the masked ones must read as zero later
+  const int nsplit = fwd_splits(RT, CTw, device_cus_or_default(a->device));
+  const size_t need_ws = (size_t)nsplit * S.Np * 16;
+  if (!a->workspace || a->workspace_bytes < need_ws) return fail(SCE_EINVAL, "forward workspace too small: %zu < %zu", a->workspace_bytes, need_ws);
   FwdParams p;
   p.xq = xq; p.wqt = wqt; p.partials = (float4*)a->workspace;
-  p.dp = S.dp; p.ldx = S.ldx; p.N = (int)N; p.V = (int)Vl; p.Np = (int)S.Np; p.RT = RT; p.CT = CT; p.S = nsplit;
-  p.sc = (float)a->x_s * (float)a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.ic2 = 1.0f / (-2.0f * a->cap * LOG2E);
+  p.targets = a->targets; p.ignore_index = a->ignore_index; p.n_predict = a->shape.n_predict; p.s_uy = (float*)(sv + S.off_zy);
+  p.ghat_t = emit ? gbase + S.rel_g : nullptr; p.gexp = emit ? (uint32_t*)(gbase + S.rel_gexp) : nullptr; p.kbw = S.Np / BK;
+  p.dp = S.dp; p.ldx = S.ldx; p.N = (int)N; p.V = (int)Vl; p.Np = (int)S.Np; p.RT = RT; p.CT = CTw; p.S = nsplit;
+  p.sc = (float)a->x_s * (float)a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.c2 = -2.0f * a->cap * LOG2E; p.ic2 = 1.0f / p.c2;
   const int grid = 8 * nsplit * ((RT + 7) / 8);
   {
+    // the exponent boosts of the rows, from the tile in the middle of the vocabulary (kept for backward in either mode)
+    KernelTimer tm(SCE_K_QUANT, st);
+    float* lam = (float*)(sv + S.off_lam);
+    p.lam = lam;
+    fwd_sample_kernel<<<RT, NTHREADS, SMEM_BYTES, st>>>(p, CT / 2, lam);
+  }
+  {
     KernelTimer tm(SCE_K_FWD, st);
-    fwd_kernel<<<grid, NTHREADS, SMEM_FWD, st>>>(p);
+    if (emit) fwd_kernel<true><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
+    else fwd_kernel<false><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
   }
   KernelTimer tm_red(SCE_K_FWD_REDUCE, st);
   float* s_lse = (float*)(sv + S.off_lse);
   float* s_umax = (float*)(sv + S.off_umax);
   float* s_zy = (float*)(sv + S.off_zy);
-  fwd_target_logit_kernel<<<dim3((unsigned)((N + 3) / 4), (unsigned)a->shape.n_predict), 256, 0, st>>>(
-      xq, wqt, S.dp, S.ldx, a->targets, a->ignore_index, (int)N, (int)S.Np, (int)Vl, (float)a->x_s * (float)a->w_s, a->cap, s_zy);
   fwd_combine_kernel<<<(int)(S.Np / 256), 256, 0, st>>>(p.partials, nsplit, (int)N, (int)S.Np, (int)Vl, a->targets, a->ignore_index,
                                                        a->cap, a->mtp_weights, a->shape.n_predict, s_lse, s_umax, s_zy, a->losses, a->lse,
                                                        a->argmax);
@@ -1736,31 +1901,46 @@ extern "C" int sce_backward(const sce_args* a) {
   const int64_t Vl = a->vocab_limit > 0 ? a->vocab_limit : V;       // columns that take part
   if (!a->workspace) return fail(SCE_EINVAL, "workspace is NULL");
   const int K = a->shape.n_predict;
-  const BwdLayout Bmin = bwd_layout(S, 256, 256, 1, K);
+  const bool kept = a->dlogits_from_forward != 0;        // the dlogits came with `saved`
+  if (kept && a->saved_bytes < need_saved + S.g_total)
+    return fail(SCE_EINVAL, "saved buffer too small for the dlogits: %zu < %zu", a->saved_bytes, need_saved + S.g_total);
+  const BwdLayout Bmin = bwd_layout(S, 256, 256, 1, K, kept);
   if (a->workspace_bytes < Bmin.total) return fail(SCE_EINVAL, "backward workspace too small: %zu < %zu", a->workspace_bytes, Bmin.total);
+  if (a->panel_rows % 256) return fail(SCE_EINVAL, "panel_rows must be a multiple of 256");
   // panel sizes from what the caller gave: P rows per recompute/dX panel, Pw = m * P rows per dW launch
-  // bytes left for the e4m3 dlogits: Vp rows of Pw bytes
-  const int64_t room = (int64_t)(a->workspace_bytes - Bmin.fixed - Bmin.part_stride);
-  int64_t P = default_panel(S);
-  if (a->panel_rows > 0) {
-    if (a->panel_rows % 256) return fail(SCE_EINVAL, "panel_rows must be a multiple of 256");
-    P = a->panel_rows < S.Np ? a->panel_rows : S.Np;
-    if (P > 131072) P = 131072;          // a dW launch covers at least one panel and at most MAX_SCALE_KBLOCKS K blocks
+  int64_t P, Pw;
+  int nparts;
+  if (kept) {
+    // no producer to stay close to: dX takes all rows at once (as many as one dW launch may contract over)
+    P = a->panel_rows > 0 ? a->panel_rows : S.Np;
+    if (P > S.Np) P = S.Np;
+    if (P > 131072) P = 131072;
+    Pw = default_dw_panel(S, P);
+    nparts = dw_launches(S, Pw);
+    while (nparts > 1 && bwd_layout(S, P, Pw, nparts, K, true).total > a->workspace_bytes) --nparts;
+  } else {
+    // bytes left for the e4m3 dlogits: Vp rows of Pw bytes
+    const int64_t room = (int64_t)(a->workspace_bytes - Bmin.fixed - Bmin.part_stride);
+    P = default_panel(S);
+    if (a->panel_rows > 0) {
+      P = a->panel_rows < S.Np ? a->panel_rows : S.Np;
+      if (P > 131072) P = 131072;          // a dW launch covers at least one panel and at most MAX_SCALE_KBLOCKS K blocks
+    }
+    if (P * S.Vp > room) P = room / S.Vp / 256 * 256;
+    if (P < 256) P = 256;                                  // Bmin fits, as checked above
+    Pw = default_dw_panel(S, P);
+    if (Pw * S.Vp > room) Pw = room / S.Vp / P * P;
+    if (Pw < P) Pw = P;
+    nparts = dw_launches(S, Pw);
+    // the estimate above ignores the 256-byte alignment of each region: settle on a layout that fits
+    while (bwd_layout(S, P, Pw, nparts, K).total > a->workspace_bytes) {
+      if (nparts > 1) --nparts;
+      else if (Pw > P) Pw -= P;
+      else if (P > 256) { P -= 256; Pw = P; }
+      else return fail(SCE_EINVAL, "internal: panel layout exceeds workspace");
+    }
   }
-  if (P * S.Vp > room) P = room / S.Vp / 256 * 256;
-  if (P < 256) P = 256;                                  // Bmin fits, as checked above
-  int64_t Pw = default_dw_panel(S, P);
-  if (Pw * S.Vp > room) Pw = room / S.Vp / P * P;
-  if (Pw < P) Pw = P;
-  int nparts = dw_launches(S, Pw);
-  // the estimate above ignores the 256-byte alignment of each region: settle on a layout that fits
-  while (bwd_layout(S, P, Pw, nparts, K).total > a->workspace_bytes) {
-    if (nparts > 1) --nparts;
-    else if (Pw > P) Pw -= P;
-    else if (P > 256) { P -= 256; Pw = P; }
-    else return fail(SCE_EINVAL, "internal: panel layout exceeds workspace");
-  }
-  const BwdLayout B = bwd_layout(S, P, Pw, nparts, K);
+  const BwdLayout B = bwd_layout(S, P, Pw, nparts, K, kept);
   DeviceGuard guard(a->device);
   if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", a->device);
   hipStream_t st = (hipStream_t)a->stream;
@@ -1773,8 +1953,10 @@ extern "C" int sce_backward(const sce_args* a) {
   const float* s_lse = (const float*)(sv + S.off_lse);
   const float* s_zy = (const float*)(sv + S.off_zy);
   const int32_t* hdr = (const int32_t*)(sv + S.off_hdr);
-  uint32_t* gexp = (uint32_t*)(ws + B.off_gexp);
+  uint8_t* gkept = sv + need_saved;
+  uint32_t* gexp = kept ? (uint32_t*)(gkept + S.rel_gexp) : (uint32_t*)(ws + B.off_gexp);
   float* rho = (float*)(ws + B.off_rho);
+  int32_t* rowinfo = (int32_t*)(ws + B.off_rowinfo);
   float* hcoef = (float*)(ws + B.off_hcoef);
   float* blockmax = (float*)(ws + B.off_blockmax);
   float* xi = (float*)(ws + B.off_xi);
@@ -1788,13 +1970,14 @@ extern "C" int sce_backward(const sce_args* a) {
   int32_t* segoff = (int32_t*)(ws + B.off_segoff);
   int32_t* longlist = (int32_t*)(ws + B.off_longlist);
   float* longsum = (float*)(ws + B.off_longsum);
-  uint8_t* ghat_t = ws + B.off_ghat_t;
+  uint8_t* ghat_t = kept ? gkept + S.rel_g : ws + B.off_ghat_t;
+  const int64_t gkb = kept ? S.Np / BK : Pw / BK;      // K blocks per v tile of the dlogits buffer
 
   const int nblk = (int)(S.Np / 256);
   KernelTimer* tm_prep = new KernelTimer(SCE_K_BWD_PREP, st);
   bwd_prep_kernel<<<nblk, 256, 0, st>>>(s_lse, s_zy, a->targets, a->ignore_index, hdr, a->grad_output,
                                         a->reduction == SCE_REDUCE_NONE ? 1 : 0, a->grad_scale, a->mtp_weights, K, a->cap, (int)N,
-                                        (int)S.Np, (int)Vl, rho, hcoef, blockmax);
+                                        (int)S.Np, (int)Vl, (const float*)(sv + S.off_lam), rho, hcoef, blockmax, kept ? nullptr : rowinfo);
   bwd_xi_kernel<<<1, 1024, 0, st>>>(blockmax, nblk, xi);
   {
     dim3 g((unsigned)(S.Np / 64), (unsigned)(S.dq / 64));
@@ -1819,22 +2002,19 @@ extern "C" int sce_backward(const sce_args* a) {
   for (int64_t p0 = 0; p0 < S.Np; p0 += P) {
     const int64_t prow = (S.Np - p0 < P) ? (S.Np - p0) : P;     // multiple of 256
     const int RTp = (int)(prow / 256);
-    RecomputeParams rp;
-    rp.xq = xq + p0 * S.ldx; rp.wqt = wqt; rp.ghat_t = ghat_t; rp.gexp = gexp;
-    rp.dp = S.dp; rp.ldx = S.ldx; rp.kbw = Pw / BK; rp.kb0 = (p0 - w0) / BK; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2;
-    {
-      KernelTimer tm(SCE_K_RECOMPUTE, st);
-      bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_RECOMPUTE, st>>>(rp);
-    }
-    if (p0 < N) {      // the target columns leave G: their part of dlogits is in the one-hot coefficients
-      KernelTimer tm(SCE_K_BWD_PREP, st);
-      const int rows = (int)(N - p0 < prow ? N - p0 : prow);
-      bwd_zero_targets_kernel<<<(rows * K + 255) / 256, 256, 0, st>>>(a->targets, a->ignore_index, (int)p0, rows, (int)N, (int)Vl, K,
-                                                                    ghat_t + ((p0 - w0) / BK) * BLOCKED_KSTEP, Pw / BK);
+    const int64_t gorg = kept ? 0 : w0;                         // the row that K block 0 of the dlogits buffer stands for
+    if (!kept) {
+      RecomputeParams rp;
+      rp.xq = xq + p0 * S.ldx; rp.wqt = wqt; rp.ghat_t = ghat_t; rp.gexp = gexp; rp.rowinfo = rowinfo + p0; rp.Np = S.Np; rp.n_predict = K;
+      rp.dp = S.dp; rp.ldx = S.ldx; rp.kbw = gkb; rp.kb0 = (p0 - gorg) / BK; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2;
+      {
+        KernelTimer tm(SCE_K_RECOMPUTE, st);
+        bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_RECOMPUTE, st>>>(rp);
+      }
     }
 
     DxParams dp_;
-    dp_.wq = wq; dp_.ghat_t = ghat_t + ((p0 - w0) / BK) * BLOCKED_KSTEP; dp_.gexp = gexp + (p0 - w0) / BK; dp_.kbw = Pw / BK; dp_.wqt = wqt; dp_.rho = rho + p0; dp_.hcoef = hcoef + p0; dp_.targets = a->targets + p0;
+    dp_.wq = wq; dp_.ghat_t = ghat_t + ((p0 - gorg) / BK) * BLOCKED_KSTEP; dp_.gexp = gexp + (p0 - gorg) / BK; dp_.kbw = gkb; dp_.wqt = wqt; dp_.rho = rho + p0; dp_.hcoef = hcoef + p0; dp_.targets = a->targets + p0;
     dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.ldx = S.ldx; dp_.Np = S.Np; dp_.dq = S.dq; dp_.RT = RTp; dp_.CT = CTd;
     dp_.n_predict = K; dp_.rows_left = (int)(N - p0 > 0 ? N - p0 : 0);
     dp_.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); dp_.d = (int)d; dp_.V = (int)Vl; dp_.w_s = (float)a->w_s;
@@ -1869,8 +2049,8 @@ extern "C" int sce_backward(const sce_args* a) {
     if (gathered + P > Pw || p0 + prow >= S.Np) {      // the transposed scratch is full, or this was the last panel
       DwParams wp;
       const int part = launch < nparts ? launch : nparts - 1;
-      wp.xt = xt; wp.ghat_t = ghat_t; wp.gexp = gexp; wp.dwacc = (float*)((uint8_t*)dwacc + (size_t)part * B.part_stride);
-      wp.kbn = S.Np / BK; wp.kbw = Pw / BK; wp.kb0 = w0 / BK; wp.Vp = S.Vp;
+      wp.xt = xt; wp.ghat_t = ghat_t + ((w0 - gorg) / BK) * BLOCKED_KSTEP; wp.gexp = gexp + (w0 - gorg) / BK; wp.dwacc = (float*)((uint8_t*)dwacc + (size_t)part * B.part_stride);
+      wp.kbn = S.Np / BK; wp.kbw = gkb; wp.kb0 = w0 / BK; wp.Vp = S.Vp;
       wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(gathered / BK);
       {
         KernelTimer tm(SCE_K_DW, st);

@@ -27,7 +27,10 @@ namespace sce {
 // vmcnt(0).  Completion is tracked by hand with s_waitcnt vmcnt before the barrier that
 // publishes the data.  LDS_CONST is an immediate, so that the only scalar work per load is the one
 // addition that forms M0.  (The instruction's own offset field is of no use for stepping through
-// K: the hardware adds it to the LDS address as well as to the memory address.)
+// K: the hardware adds it to the LDS address as well as to the memory address.)  M0 is written and consumed inside the
+// one asm statement; it cannot be named as a clobber (the compiler treats it as reserved and says that a clobber of
+// it is not honoured), so this relies on the compiler not keeping a value of its own in M0 across the statement --
+// it loads M0 immediately before each instruction of its own that reads it.
 template <int LDS_CONST>
 __device__ __forceinline__ void lds_direct_16(uint32_t lds_addr, uint32_t voff, const uint8_t* sbase) {
   asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
@@ -121,11 +124,15 @@ __device__ __forceinline__ v16f mfma_fp8_scaled_sel(int opb, const v8i& a, const
   }
 }
 
-template <bool PREFETCHED = false, class Hook = NoHook, int KSTEP = BK, bool TRB = false, int SCALE = 0, int FIRST_WAIT = 8>
+// stores_between (PREFETCHED only, uniform): the caller issued at least 16 vector memory stores between its prefetch of
+// K block 0 and its 8 loads of K block 1 (mfma_prefetch<1>, the stores, mfma_prefetch<2>); they are younger than
+// block 0, so the first wait may leave them in flight.
+template <bool PREFETCHED = false, class Hook = NoHook, int KSTEP = BK, bool TRB = false, int SCALE = 0>
 __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, int64_t lda,
                                               const uint8_t* __restrict__ Bg, int64_t ldb, int KD,
                                               uint8_t* smem, v16f (&acc)[4][4], int rot_a, int rot_b, int wave, Hook&& hook = NoHook(),
-                                              int64_t bk1_arg = 0, int64_t bk2_arg = 0, const uint32_t* lds_scale = nullptr) {
+                                              int64_t bk1_arg = 0, int64_t bk2_arg = 0, const uint32_t* lds_scale = nullptr,
+                                              bool stores_between = false) {
   const int lane = lane_id();
   const int wa = wave >> 1, wb = wave & 1;
   const int64_t bk1 = TRB ? bk1_arg : (int64_t)KSTEP, bk2 = TRB ? bk2_arg : (int64_t)(2 * KSTEP);
@@ -172,9 +179,9 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
 #pragma unroll
     for (int n = 0; n < 8; ++n) ld.template issue<1>(n, Ag + KSTEP, Bg + bk1);
   }
-  // FIRST_WAIT: how many of the wave's vector memory operations may still be in flight once K block 0 has landed
-  // (the 8 loads of block 1, plus whatever a caller issued between its prefetch of block 0 and this point)
-  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(FIRST_WAIT) : "memory");
+  // K block 0 has landed once at most the 8 loads of block 1 (and the stores a caller put between the two) are in flight
+  if (PREFETCHED && stores_between) asm volatile("s_waitcnt vmcnt(24)\n\ts_barrier" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
   v8i fa[2][4], fb[2][4];
 #pragma unroll
   for (int n = 0; n < 8; ++n) rfrag1(0, 0, n, fa[0], fb[0]);

@@ -36,6 +36,12 @@ from ._lib import SceArgs, SceShape
 CE_KERNEL_VOCAB_SIZE = 50304          # tiny/cuda_kernels.py:82
 IGNORE_INDEX = -1                     # tiny/train.py:743
 
+# How backward gets the dlogits when a call does not say (keep_dlogits=None):
+#   True   forward leaves them in the saved state, 8 bits per logit (N x V bytes held until backward; the reference
+#          holds 3 N x V bytes, tiny/cuda_kernels.py:359-371); backward is two GEMMs
+#   False  backward computes the logit tiles again: nothing N x V is held, backward is three GEMMs
+KEEP_DLOGITS = True
+
 _DTYPES = {torch.float32: _lib.SCE_F32, torch.bfloat16: _lib.SCE_BF16}
 
 
@@ -115,8 +121,10 @@ class WeightCache:
 
 
 def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_weights=None, vocab_size=None,
-               weight_cache=None, norm_eps=None):
+               weight_cache=None, norm_eps=None, keep_dlogits=False):
     """One call of sce_forward.  Returns (out, saved, lse, argmax, n_valid).
+
+    keep_dlogits: the forward pass also leaves the dlogits in ``saved`` (pass the same value to ce_backward).
 
     norm_eps: when given, ``x`` is the hidden state before the trunk's final ``F.rms_norm(x, (d,))``
     (tiny/train.py:397-398,734) and the norm is applied inside the quantiser."""
@@ -131,7 +139,8 @@ def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_w
     V = w.shape[1]
     dev = x.device
     sz = _lib.sizes_for(N, d, V, n_predict)
-    saved = torch.empty(sz.saved_x_bytes if weight_cache is not None else sz.saved_bytes, dtype=torch.uint8, device=dev)
+    saved = torch.empty((sz.saved_x_bytes if weight_cache is not None else sz.saved_bytes) + (sz.dlogits_bytes if keep_dlogits else 0),
+                        dtype=torch.uint8, device=dev)
     ws = torch.empty(sz.fwd_workspace_bytes, dtype=torch.uint8, device=dev)
     losses = torch.empty(N, dtype=torch.float32, device=dev)
     lse = torch.empty(N, dtype=torch.float32, device=dev)
@@ -146,6 +155,7 @@ def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_w
     a.saved, a.saved_bytes = saved.data_ptr(), saved.numel()
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
     a.vocab_limit = 0 if vocab_size is None else int(vocab_size)
+    a.dlogits_from_forward = int(bool(keep_dlogits))
     if norm_eps is not None:
         a.norm, a.norm_eps = 1, float(norm_eps)
     if weight_cache is not None:
@@ -158,7 +168,7 @@ def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_w
 
 def ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale, reduction, x_dtype, w_dtype,
                 panel_rows=0, workspace_bytes=None, mtp_weights=None, vocab_size=None, weight_cache=None,
-                hidden=None, norm_eps=None):
+                hidden=None, norm_eps=None, keep_dlogits=False):
     """One call of sce_backward.  Returns (dx (N,d) in x_dtype, dw (d,V) in w_dtype).
 
     hidden, norm_eps: the pre-norm hidden state and eps given to ce_forward(norm_eps=...); dx is then the
@@ -166,7 +176,7 @@ def ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale,
     dev = saved.device
     n_predict, mtp_w = _mtp(mtp_weights, dev)
     sz = _lib.sizes_for(N, d, V, n_predict)
-    nbytes = sz.bwd_workspace_bytes if workspace_bytes is None else workspace_bytes
+    nbytes = (sz.bwd_workspace_kept_bytes if keep_dlogits else sz.bwd_workspace_bytes) if workspace_bytes is None else workspace_bytes
     ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     dx = torch.empty(N, d, dtype=x_dtype, device=dev)
     dw = torch.empty(d, V, dtype=w_dtype, device=dev)
@@ -184,6 +194,7 @@ def ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale,
     a.dw, a.dw_dtype, a.dw_ld = dw.data_ptr(), _DTYPES[w_dtype], V
     a.panel_rows = panel_rows
     a.vocab_limit = 0 if vocab_size is None else int(vocab_size)
+    a.dlogits_from_forward = int(bool(keep_dlogits))
     if norm_eps is not None:
         if hidden is None or tuple(hidden.shape) != (N, d) or hidden.device != dev:
             raise ValueError("backward through the fused norm needs the (N, d) hidden state given to forward")
@@ -203,59 +214,61 @@ def ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale,
 # ---------------------------------------------------------------------------------------------
 @torch.library.custom_op("slowrun_amd::ce_forward", mutates_args=())
 def ce_forward_op(x: torch.Tensor, w: torch.Tensor, targets: torch.Tensor, mtp_weights: Optional[torch.Tensor],
-                  x_s: float, w_s: float, cap: float, mean: bool) -> Tuple[torch.Tensor, torch.Tensor]:
-    out, saved, _lse, _am, _nv = ce_forward(x, w, targets, x_s, w_s, cap, "mean" if mean else "none", mtp_weights=mtp_weights)
+                  x_s: float, w_s: float, cap: float, mean: bool, keep: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    out, saved, _lse, _am, _nv = ce_forward(x, w, targets, x_s, w_s, cap, "mean" if mean else "none", mtp_weights=mtp_weights,
+                                            keep_dlogits=keep)
     return out, saved
 
 
 @ce_forward_op.register_fake
-def _ce_forward_fake(x, w, targets, mtp_weights, x_s, w_s, cap, mean):
+def _ce_forward_fake(x, w, targets, mtp_weights, x_s, w_s, cap, mean, keep):
     N, d = x.shape
     V = w.shape[1]
     n_predict = 1 if mtp_weights is None else mtp_weights.numel()
     sz = _lib.sizes_for(N, d, V, n_predict)
     out = x.new_empty((), dtype=torch.float32) if mean else x.new_empty((N,), dtype=torch.float32)
-    return out, x.new_empty((sz.saved_bytes,), dtype=torch.uint8)
+    return out, x.new_empty((sz.saved_bytes + (sz.dlogits_bytes if keep else 0),), dtype=torch.uint8)
 
 
 @torch.library.custom_op("slowrun_amd::ce_backward", mutates_args=())
 def ce_backward_op(saved: torch.Tensor, targets: torch.Tensor, grad_output: torch.Tensor, mtp_weights: Optional[torch.Tensor],
                    N: int, d: int, V: int, x_s: float, w_s: float, cap: float, grad_scale: float, mean: bool,
-                   x_bf16: bool, w_bf16: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+                   x_bf16: bool, w_bf16: bool, keep: bool) -> Tuple[torch.Tensor, torch.Tensor]:
     return ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale, "mean" if mean else "none",
                        torch.bfloat16 if x_bf16 else torch.float32, torch.bfloat16 if w_bf16 else torch.float32,
-                       mtp_weights=mtp_weights)
+                       mtp_weights=mtp_weights, keep_dlogits=keep)
 
 
 @ce_backward_op.register_fake
-def _ce_backward_fake(saved, targets, grad_output, mtp_weights, N, d, V, x_s, w_s, cap, grad_scale, mean, x_bf16, w_bf16):
+def _ce_backward_fake(saved, targets, grad_output, mtp_weights, N, d, V, x_s, w_s, cap, grad_scale, mean, x_bf16, w_bf16, keep):
     return (saved.new_empty((N, d), dtype=torch.bfloat16 if x_bf16 else torch.float32),
             saved.new_empty((d, V), dtype=torch.bfloat16 if w_bf16 else torch.float32))
 
 
 @torch.library.custom_op("slowrun_amd::norm_ce_forward", mutates_args=())
 def norm_ce_forward_op(h: torch.Tensor, w: torch.Tensor, targets: torch.Tensor, mtp_weights: Optional[torch.Tensor],
-                       x_s: float, w_s: float, cap: float, mean: bool, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+                       x_s: float, w_s: float, cap: float, mean: bool, eps: float, keep: bool) -> Tuple[torch.Tensor, torch.Tensor]:
     out, saved, _lse, _am, _nv = ce_forward(h, w, targets, x_s, w_s, cap, "mean" if mean else "none", mtp_weights=mtp_weights,
-                                            norm_eps=eps)
+                                            norm_eps=eps, keep_dlogits=keep)
     return out, saved
 
 
-norm_ce_forward_op.register_fake(lambda h, w, targets, mtp_weights, x_s, w_s, cap, mean, eps:
-                                 _ce_forward_fake(h, w, targets, mtp_weights, x_s, w_s, cap, mean))
+norm_ce_forward_op.register_fake(lambda h, w, targets, mtp_weights, x_s, w_s, cap, mean, eps, keep:
+                                 _ce_forward_fake(h, w, targets, mtp_weights, x_s, w_s, cap, mean, keep))
 
 
 @torch.library.custom_op("slowrun_amd::norm_ce_backward", mutates_args=())
 def norm_ce_backward_op(saved: torch.Tensor, h: torch.Tensor, targets: torch.Tensor, grad_output: torch.Tensor,
                         mtp_weights: Optional[torch.Tensor], V: int, x_s: float, w_s: float, cap: float, grad_scale: float,
-                        mean: bool, w_bf16: bool, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+                        mean: bool, w_bf16: bool, eps: float, keep: bool) -> Tuple[torch.Tensor, torch.Tensor]:
     N, d = h.shape
     return ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale, "mean" if mean else "none",
-                       h.dtype, torch.bfloat16 if w_bf16 else torch.float32, mtp_weights=mtp_weights, hidden=h, norm_eps=eps)
+                       h.dtype, torch.bfloat16 if w_bf16 else torch.float32, mtp_weights=mtp_weights, hidden=h, norm_eps=eps,
+                       keep_dlogits=keep)
 
 
 @norm_ce_backward_op.register_fake
-def _norm_ce_backward_fake(saved, h, targets, grad_output, mtp_weights, V, x_s, w_s, cap, grad_scale, mean, w_bf16, eps):
+def _norm_ce_backward_fake(saved, h, targets, grad_output, mtp_weights, V, x_s, w_s, cap, grad_scale, mean, w_bf16, eps, keep):
     return torch.empty_like(h), h.new_empty((h.shape[1], V), dtype=torch.bfloat16 if w_bf16 else torch.float32)
 
 
@@ -263,27 +276,29 @@ class FusedSoftcappedCrossEntropy(torch.autograd.Function):
     """Same call as tiny/cuda_kernels.py:336-414; see the module docstring."""
 
     @staticmethod
-    def forward(ctx, x, targets, mtp_weights, lm_head_weight, x_s, w_s, grad_s, grad_scale, cap=15.0, reduction="none"):
+    def forward(ctx, x, targets, mtp_weights, lm_head_weight, x_s, w_s, grad_s, grad_scale, cap=15.0, reduction="none",
+                keep_dlogits=None):
         if reduction not in ("none", "mean"):
             raise ValueError("reduction must be 'none' or 'mean'")
         _dtype_code(x, "x")
         _dtype_code(lm_head_weight, "lm_head_weight")
         xs, ws_ = _scale_value(x_s, x), _scale_value(w_s, lm_head_weight)
+        keep = bool(KEEP_DLOGITS if keep_dlogits is None else keep_dlogits)
         out, saved = ce_forward_op(x.detach(), lm_head_weight.detach(), targets, mtp_weights, xs, ws_, float(cap),
-                                   reduction == "mean")
+                                   reduction == "mean", keep)
         ctx.save_for_backward(saved, targets, mtp_weights if mtp_weights is not None else torch.empty(0, device=x.device))
         ctx.params = (x.shape[0], x.shape[1], lm_head_weight.shape[1], xs, ws_, float(cap), float(grad_scale),
                       reduction == "mean", x.dtype == torch.bfloat16, lm_head_weight.dtype == torch.bfloat16,
-                      mtp_weights is not None)
+                      mtp_weights is not None, keep)
         return out
 
     @staticmethod
     def backward(ctx, grad_output):
         saved, targets, mtp_w = ctx.saved_tensors
-        N, d, V, xs, ws_, cap, gscale, mean, x_bf16, w_bf16, has_mtp = ctx.params
+        N, d, V, xs, ws_, cap, gscale, mean, x_bf16, w_bf16, has_mtp, keep = ctx.params
         dx, dw = ce_backward_op(saved, targets, grad_output.contiguous(), mtp_w if has_mtp else None, N, d, V, xs, ws_, cap,
-                                gscale, mean, x_bf16, w_bf16)
-        return dx, None, None, dw, None, None, None, None, None, None
+                                gscale, mean, x_bf16, w_bf16, keep)
+        return dx, None, None, dw, None, None, None, None, None, None, None
 
 
 class FusedNormSoftcappedCrossEntropy(torch.autograd.Function):
@@ -294,7 +309,7 @@ class FusedNormSoftcappedCrossEntropy(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, h, targets, mtp_weights, lm_head_weight, x_s, w_s, grad_s, grad_scale, cap=15.0, reduction="none",
-                eps=None):
+                eps=None, keep_dlogits=None):
         if reduction not in ("none", "mean"):
             raise ValueError("reduction must be 'none' or 'mean'")
         _dtype_code(h, "h")
@@ -302,20 +317,21 @@ class FusedNormSoftcappedCrossEntropy(torch.autograd.Function):
         eps = float(torch.finfo(torch.float32).eps if eps is None else eps)
         xs, ws_ = _scale_value(x_s, h), _scale_value(w_s, lm_head_weight)
         hd = h.detach()
+        keep = bool(KEEP_DLOGITS if keep_dlogits is None else keep_dlogits)
         out, saved = norm_ce_forward_op(hd, lm_head_weight.detach(), targets, mtp_weights, xs, ws_, float(cap),
-                                        reduction == "mean", eps)
+                                        reduction == "mean", eps, keep)
         ctx.save_for_backward(saved, hd, targets, mtp_weights if mtp_weights is not None else torch.empty(0, device=h.device))
         ctx.params = (lm_head_weight.shape[1], xs, ws_, float(cap), float(grad_scale), reduction == "mean",
-                      lm_head_weight.dtype == torch.bfloat16, mtp_weights is not None, eps)
+                      lm_head_weight.dtype == torch.bfloat16, mtp_weights is not None, eps, keep)
         return out
 
     @staticmethod
     def backward(ctx, grad_output):
         saved, h, targets, mtp_w = ctx.saved_tensors
-        V, xs, ws_, cap, gscale, mean, w_bf16, has_mtp, eps = ctx.params
+        V, xs, ws_, cap, gscale, mean, w_bf16, has_mtp, eps, keep = ctx.params
         dh, dw = norm_ce_backward_op(saved, h, targets, grad_output.contiguous(), mtp_w if has_mtp else None, V, xs, ws_, cap,
-                                     gscale, mean, w_bf16, eps)
-        return dh, None, None, dw, None, None, None, None, None, None, None
+                                     gscale, mean, w_bf16, eps, keep)
+        return dh, None, None, dw, None, None, None, None, None, None, None, None
 
 
 def softcapped_cross_entropy(x, lm_head_weight, targets, x_s, w_s, cap=15.0, vocab_size=None, reduction="mean",

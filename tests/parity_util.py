@@ -19,18 +19,20 @@ def cosine(a, b):
 
 
 def run_ours(inp, reduction="mean", x_dtype=torch.bfloat16, w_dtype=torch.bfloat16, grad_output=None, device="cuda",
-             want_argmax=True, panel_rows=0):
+             want_argmax=True, panel_rows=0, keep_dlogits=False):
+    """keep_dlogits: the forward pass emits the dlogits and backward reads them, instead of computing the logits again."""
     from slowrun_amd import cuda_kernels as ck
     x = inp.x.to(device=device, dtype=x_dtype)
     w = inp.w.to(device=device, dtype=w_dtype)
     y = inp.targets.to(device)
     N, d = x.shape
     V = w.shape[1]
-    out, saved, lse, argmax, n_valid = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, reduction, want_argmax=want_argmax)
+    out, saved, lse, argmax, n_valid = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, reduction, want_argmax=want_argmax,
+                                                     keep_dlogits=keep_dlogits)
     if grad_output is None:
         grad_output = torch.ones((), device=device) if reduction == "mean" else torch.full((N,), 1.0 / N, device=device)
     dx, dw = ck.ce_backward(saved, y, grad_output, N, d, V, inp.x_s, inp.w_s, inp.cap, 1.0, reduction, x_dtype, w_dtype,
-                            panel_rows=panel_rows)
+                            panel_rows=panel_rows, keep_dlogits=keep_dlogits)
     torch.cuda.synchronize()
     return dict(loss=out, lse=lse, argmax=argmax, n_valid=n_valid, dx=dx, dw=dw, x=x, w=w, y=y, x_s=inp.x_s, w_s=inp.w_s)
 

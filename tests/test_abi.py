@@ -108,16 +108,17 @@ def test_custom_ops_have_fake_implementations():
     w = torch.empty(128, 1024, dtype=torch.bfloat16, device="meta")
     y = torch.empty(512, dtype=torch.int64, device="meta")
     mw = torch.empty(3, dtype=torch.float32, device="meta")
-    out, saved = ck.ce_forward_op(x, w, y, mw, 0.1, 0.1, 15.0, False)
+    out, saved = ck.ce_forward_op(x, w, y, mw, 0.1, 0.1, 15.0, False, False)
     assert out.shape == (512,) and out.dtype == torch.float32
-    assert saved.dtype == torch.uint8 and saved.numel() == _lib.sizes_for(512, 128, 1024, 3).saved_bytes
-    out2, _ = ck.ce_forward_op(x, w, y, None, 0.1, 0.1, 15.0, True)
-    assert out2.shape == ()
-    dx, dw = ck.ce_backward_op(saved, y, out, mw, 512, 128, 1024, 0.1, 0.1, 15.0, 1.0, False, True, False)
+    sz3 = _lib.sizes_for(512, 128, 1024, 3)
+    assert saved.dtype == torch.uint8 and saved.numel() == sz3.saved_bytes
+    out2, saved2 = ck.ce_forward_op(x, w, y, mw, 0.1, 0.1, 15.0, True, True)         # the dlogits travel in `saved`
+    assert out2.shape == () and saved2.numel() == sz3.saved_bytes + sz3.dlogits_bytes and sz3.dlogits_bytes >= 512 * 1024
+    dx, dw = ck.ce_backward_op(saved, y, out, mw, 512, 128, 1024, 0.1, 0.1, 15.0, 1.0, False, True, False, False)
     assert dx.shape == (512, 128) and dx.dtype == torch.bfloat16 and dw.shape == (128, 1024) and dw.dtype == torch.float32
-    out3, saved3 = ck.norm_ce_forward_op(x, w, y, None, 0.1, 0.1, 15.0, True, 1e-6)
+    out3, saved3 = ck.norm_ce_forward_op(x, w, y, None, 0.1, 0.1, 15.0, True, 1e-6, False)
     assert out3.shape == () and saved3.numel() == _lib.sizes_for(512, 128, 1024, 1).saved_bytes
-    dh, dw2 = ck.norm_ce_backward_op(saved3, x, y, out3, None, 1024, 0.1, 0.1, 15.0, 1.0, True, True, 1e-6)
+    dh, dw2 = ck.norm_ce_backward_op(saved3, x, y, out3, None, 1024, 0.1, 0.1, 15.0, 1.0, True, True, 1e-6, False)
     assert dh.shape == (512, 128) and dh.dtype == torch.bfloat16 and dw2.shape == (128, 1024) and dw2.dtype == torch.bfloat16
 
 

@@ -35,9 +35,10 @@ def test_transpose_copy():
 
 @pytest.mark.parametrize("N,d,V", [(256, 128, 256), (300, 128, 1000), (1000, 80, 777), (513, 272, 2049), (64, 16, 50304)])
 @pytest.mark.parametrize("reduction", ["mean", "none"])
-def test_small_shapes(N, d, V, reduction):
+@pytest.mark.parametrize("keep", [False, True])
+def test_small_shapes(N, d, V, reduction, keep):
     inp = _small("tiny_track", N, d, V)
-    ours = pu.run_ours(inp, reduction)
+    ours = pu.run_ours(inp, reduction, keep_dlogits=keep)
     ref = pu.run_oracle(inp, ours, reduction)
     print(pu.check_parity(ours, ref, reduction))
 
@@ -119,7 +120,9 @@ def test_multi_token_prediction(weights):
         assert pu.maxrel(got.float(), want) <= pu.GRAD_MAXREL and pu.cosine(got.float(), want) > pu.GRAD_COS
     if weights == [1.0, 0.0, 0.0]:
         plain = FusedSoftcappedCrossEntropy.apply(x.detach(), y, None, w.detach(), inp.x_s, inp.w_s, 0.75 / 448, 1.0, inp.cap)
-        assert torch.equal(plain, losses.detach())
+        # the same up to the order of the fp32 sum over the columns (the targets of the zero-weight offsets take their
+        # own way into the row sums)
+        assert torch.allclose(plain, losses.detach(), rtol=2e-6, atol=2e-6)
 
 
 def test_traced_by_torch_compile():
@@ -376,12 +379,13 @@ def _random_shapes(seed, count):
 
 
 @pytest.mark.parametrize("N,d,V", [(1, 16, 2), (2, 16, 257), (255, 32, 255), (257, 48, 513)] + _random_shapes(1234, 10))
-def test_ragged_and_tiny_shapes(N, d, V):
+@pytest.mark.parametrize("keep", [False, True])
+def test_ragged_and_tiny_shapes(N, d, V, keep):
     """Sizes on both sides of every tile boundary, down to one row, 16 hidden units and two columns: ignored rows
     included, panels of the smallest size and of the default size must agree with the oracle and with each other."""
     inp = _small("irregular", N, d, V)
     reduction = "none" if (N + d + V) % 2 else "mean"
-    ours = pu.run_ours(inp, reduction)
+    ours = pu.run_ours(inp, reduction, keep_dlogits=keep)
     ref = pu.run_oracle(inp, ours, reduction)
     # The stated gradient tolerance is for sums over many rows and columns.  The part of dlogits that is not the
     # one-hot term passes through e4m3 (three mantissa bits: steps of up to 6.25 %, the reference's e5m2 has twice
@@ -389,7 +393,7 @@ def test_ragged_and_tiny_shapes(N, d, V):
     tiny = N < 64 or V < 64
     rep = pu.check_parity(ours, ref, reduction, grad_maxrel=7e-2 if tiny else pu.GRAD_MAXREL,
                           grad_cos=0.999 if tiny else pu.GRAD_COS)
-    small = pu.run_ours(inp, reduction, panel_rows=256)
+    small = pu.run_ours(inp, reduction, panel_rows=256, keep_dlogits=keep)
     assert torch.equal(small["dx"], ours["dx"])
     assert pu.maxrel(small["dw"].float(), ours["dw"].float()) < 1e-2
     print(N, d, V, reduction, rep)
