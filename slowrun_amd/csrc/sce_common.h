@@ -85,7 +85,7 @@ static inline SavedLayout saved_layout(int64_t N, int64_t d, int64_t V, int n_pr
 struct BwdLayout {
   int64_t P, Pw;                     // rows per recompute/dX panel and per dW launch (multiples of 256, Pw of P)
   size_t off_gexp, off_rho, off_rowinfo, off_hcoef, off_blockmax, off_xi, off_xt, off_dwacc, off_perm, off_keys,
-      off_segoff, off_longlist, off_longsum, off_sorttmp, off_dxpart, off_ghat_t, fixed, total;
+      off_segoff, off_longlist, off_longbase, off_longsum, off_sorttmp, off_dxpart, off_ghat_t, fixed, total;
   size_t sorttmp_bytes, part_stride;   // part_stride: bytes between consecutive fp32 dW partials
   int nparts;
 };

@@ -1365,17 +1365,18 @@ __global__ __launch_bounds__(256) void bwd_segoff_kernel(const int32_t* __restri
 
 
 // A column that is the target of at least LONG_SEG rows has its segment of the sorted list cut into
-// nch = ceil(L / LONG_CHUNK) equal chunks of at least LONG_SEG rows each; chunk c starts at sorted
-// position s0 + c * ceil(L / nch).  Distinct chunks start at least LONG_SEG positions apart, so
-// (start / LONG_SEG) is a slot of its own in the array of chunk sums.
+// nch = ceil(L / LONG_CHUNK) equal chunks (the last one may be shorter); chunk c starts at sorted
+// position s0 + c * ceil(L / nch).
 __device__ __forceinline__ void long_chunks(int L, int& nch, int& len) {
   nch = (L + LONG_CHUNK - 1) / LONG_CHUNK;
   len = (L + nch - 1) / nch;
 }
 
 // List of (column, chunk) pairs of the long columns (order irrelevant: each pair is handled on its
-// own).  longlist[0] is the count, then two ints per pair.
-__global__ __launch_bounds__(256) void bwd_longlist_kernel(const int32_t* __restrict__ segoff, int V, int32_t* __restrict__ longlist) {
+// own).  longlist[0] is the count, then two ints per pair; the position of a pair in the list is the slot of its
+// chunk sum, and longbase[v] is the position of column v's first pair.
+__global__ __launch_bounds__(256) void bwd_longlist_kernel(const int32_t* __restrict__ segoff, int V, int32_t* __restrict__ longlist,
+                                                          int32_t* __restrict__ longbase) {
   const int v = blockIdx.x * 256 + threadIdx.x;
   if (v >= V) return;
   const int L = segoff[v + 1] - segoff[v];
@@ -1383,6 +1384,7 @@ __global__ __launch_bounds__(256) void bwd_longlist_kernel(const int32_t* __rest
   int nch, len;
   long_chunks(L, nch, len);
   const int at = atomicAdd(&longlist[0], nch);
+  longbase[v] = at;
   for (int c = 0; c < nch; ++c) { longlist[1 + 2 * (at + c)] = v; longlist[2 + 2 * (at + c)] = c; }
 }
 
@@ -1437,7 +1439,7 @@ __global__ __launch_bounds__(256) void bwd_dw_long_kernel(const int32_t* __restr
   float sfold = 0.f;
 #pragma unroll
   for (int k = 0; k < 16; ++k) sfold += red[k][t];
-  longsum[(int64_t)(s0 / LONG_SEG) * dq + jb + t] = sfold;
+  longsum[(int64_t)blockIdx.x * dq + jb + t] = sfold;
 }
 
 // dW = x_s * ( xi * (sum of the dW partials) - sum over the target segment of h_i X_q[i, :] ), cast to the output
@@ -1447,7 +1449,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restrict__ dwacc, int nparts, int64_t part_stride, int64_t Vp, const int32_t* __restrict__ segoff,
                                                           const int32_t* __restrict__ perm, const float* __restrict__ hcoef,
                                                           const uint8_t* __restrict__ xq, int64_t ldx, int Np, const float* __restrict__ xi,
-                                                          const float* __restrict__ longsum, int64_t dq,
+                                                          const float* __restrict__ longsum, const int32_t* __restrict__ longbase, int64_t dq,
                                                           float x_s, int d, int V, T* __restrict__ dw, int64_t dw_ld) {
   const int t = threadIdx.x;
   const int v = blockIdx.x * 64 + (t & 63);
@@ -1466,7 +1468,7 @@ __global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restri
     int nch, len;
     long_chunks(L, nch, len);
     for (int c = 0; c < nch; ++c) {                       // fixed order
-      const float* ls = longsum + (int64_t)((s0 + c * len) / LONG_SEG) * dq + j0;
+      const float* ls = longsum + (int64_t)(longbase[v] + c) * dq + j0;
 #pragma unroll
       for (int m = 0; m < 16; ++m) o[m] -= ls[m] * x_s;
     }
@@ -1571,16 +1573,20 @@ struct KernelTimer {   // records an event pair around the launches made while i
   }
 };
 
+// First use of a device: its architecture, and the kernels' LDS limits, set with that device current.  A device
+// counts as known only once every step has succeeded, so a failure here is tried again on the next call.
 static int check_device(int dev) {
   if (dev < 0 || dev >= 64) return fail(SCE_EINVAL, "device %d out of range", dev);
   std::lock_guard<std::mutex> lk(g_mu);
   if (g_arch_ok[dev] == 0) {
+    DeviceGuard guard(dev);
+    if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", dev);
     hipDeviceProp_t prop;
     HIP_TRY(hipGetDeviceProperties(&prop, dev));
-    g_arch_ok[dev] = strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : -1;
-    g_cus[dev] = prop.multiProcessorCount;
-    if (g_arch_ok[dev] == 1) {
-      // the MFMA kernels hold two 64 KB K-slots in LDS
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+      g_arch_ok[dev] = -1;
+    } else {
+      // the MFMA kernels hold two 64 KB K-slots in LDS, and more behind them
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_sample_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
@@ -1591,6 +1597,8 @@ static int check_device(int dev) {
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
+      g_cus[dev] = prop.multiProcessorCount;
+      g_arch_ok[dev] = 1;
     }
   }
   if (g_arch_ok[dev] != 1) return fail(SCE_EARCH, "device %d is not gfx950", dev);
@@ -1638,7 +1646,8 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int npa
   B.off_keys = take((size_t)S.N * K * 4 * 2);  // sorted keys + unsorted keys
   B.off_segoff = take((size_t)(S.V + 2) * 4);
   B.off_longlist = take((size_t)(2 * (S.N * K / LONG_SEG + 1) + 2) * 4);   // (column, chunk) pairs: at most one per LONG_SEG entries
-  B.off_longsum = take((size_t)(S.N * K / LONG_SEG + 1) * S.dq * 4);      // chunk sums, one slot per LONG_SEG sorted positions
+  B.off_longbase = take((size_t)S.V * 4);                                  // first slot of each long column
+  B.off_longsum = take((size_t)(S.N * K / LONG_SEG + 1) * S.dq * 4);      // chunk sums: a long column has at most one chunk per LONG_SEG of its entries
   B.sorttmp_bytes = sort_tmp_bytes(S.N * K, S.V);
   B.off_sorttmp = take(B.sorttmp_bytes);
   B.off_dxpart = take(DX_PART_BYTES);
@@ -1813,6 +1822,7 @@ extern "C" int sce_forward(const sce_args* a) {
   if (a->saved_bytes < gneed) return fail(SCE_EINVAL, "saved buffer too small for the dlogits: %zu < %zu", a->saved_bytes, gneed);
   DeviceGuard guard(a->device);
   if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", a->device);
+  (void)hipGetLastError();          // an error left by some earlier, unrelated call is not this call's
   hipStream_t st = (hipStream_t)a->stream;
   uint8_t* sv = (uint8_t*)a->saved;
   uint8_t* xq = sv + S.off_xq;
@@ -1943,6 +1953,7 @@ extern "C" int sce_backward(const sce_args* a) {
   const BwdLayout B = bwd_layout(S, P, Pw, nparts, K, kept);
   DeviceGuard guard(a->device);
   if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", a->device);
+  (void)hipGetLastError();          // an error left by some earlier, unrelated call is not this call's
   hipStream_t st = (hipStream_t)a->stream;
   uint8_t* sv = (uint8_t*)a->saved;
   uint8_t* ws = (uint8_t*)a->workspace;
@@ -1970,6 +1981,7 @@ extern "C" int sce_backward(const sce_args* a) {
   int32_t* segoff = (int32_t*)(ws + B.off_segoff);
   int32_t* longlist = (int32_t*)(ws + B.off_longlist);
   float* longsum = (float*)(ws + B.off_longsum);
+  int32_t* longbase = (int32_t*)(ws + B.off_longbase);
   uint8_t* ghat_t = kept ? gkept + S.rel_g : ws + B.off_ghat_t;
   const int64_t gkb = kept ? S.Np / BK : Pw / BK;      // K blocks per v tile of the dlogits buffer
 
@@ -1992,7 +2004,7 @@ extern "C" int sce_backward(const sce_args* a) {
     if (sce::sort_pairs(ws + B.off_sorttmp, &tmp, keys_in, skeys, vals_in, perm, (size_t)NE, bits, st) != 0)
     { delete tm_prep; return fail(SCE_EHIP, "radix sort of the targets failed"); }
     bwd_segoff_kernel<<<(int)((NE + 256) / 256), 256, 0, st>>>(skeys, (int)NE, (int)V, segoff);
-    bwd_longlist_kernel<<<(int)((V + 255) / 256), 256, 0, st>>>(segoff, (int)V, longlist);
+    bwd_longlist_kernel<<<(int)((V + 255) / 256), 256, 0, st>>>(segoff, (int)V, longlist, longbase);
   }
   delete tm_prep;
   const float k1 = (float)a->x_s * (float)a->w_s * 2.0f * LOG2E / a->cap, c2 = -2.0f * a->cap * LOG2E;
@@ -2075,10 +2087,10 @@ extern "C" int sce_backward(const sce_args* a) {
   {
     dim3 g((unsigned)((V + 63) / 64), (unsigned)((d + 63) / 64));
     if (a->dw_dtype == SCE_F32)
-      bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, S.dq, (float)a->x_s, (int)d, (int)V,
+      bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, longbase, S.dq, (float)a->x_s, (int)d, (int)V,
                                                    (float*)a->dw, a->dw_ld);
     else
-      bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, S.dq, (float)a->x_s, (int)d, (int)V,
+      bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, longbase, S.dq, (float)a->x_s, (int)d, (int)V,
                                                     (bf16_t*)a->dw, a->dw_ld);
   }
   HIP_TRY(hipGetLastError());

@@ -102,11 +102,22 @@ class WeightCache:
 
     The reference re-quantises and re-lays-out W on every micro-step (tiny/cuda_kernels.py:341-343) although W
     only changes at optimizer.step().  With a WeightCache the forward quantises W only when the tensor (storage,
-    version counter, scale) differs from the one the cache was filled from.
+    version counter, shape, dtype, scale) differs from the one the cache was filled from.
+
+    The version counter does not see everything: writes through ``w.data`` (the reference broadcasts parameters
+    that way, tiny/train.py:1586), a checkpoint loaded with ``copy_`` into ``.data``, or a new tensor that happens
+    to be allocated at the old address.  Call ``invalidate()`` after anything of that kind -- after
+    ``optimizer.step()`` is always right.  ``generation`` counts the fills; ce_forward hands it out with the saved
+    state and ce_backward refuses a cache that has been refilled since, instead of using another W's bytes.
     """
 
     def __init__(self):
         self.buf = None
+        self.key = None
+        self.generation = 0
+
+    def invalidate(self):
+        """The next forward quantises W again, whatever the tensor's version counter says."""
         self.key = None
 
     def prepare(self, w, w_s, nbytes):
@@ -116,6 +127,8 @@ class WeightCache:
             self.buf = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
             self.key = None
         valid = self.key == key
+        if not valid:
+            self.generation += 1
         self.key = key
         return self.buf, valid
 
@@ -168,11 +181,12 @@ def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_w
 
 def ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale, reduction, x_dtype, w_dtype,
                 panel_rows=0, workspace_bytes=None, mtp_weights=None, vocab_size=None, weight_cache=None,
-                hidden=None, norm_eps=None, keep_dlogits=False):
+                hidden=None, norm_eps=None, keep_dlogits=False, cache_generation=None):
     """One call of sce_backward.  Returns (dx (N,d) in x_dtype, dw (d,V) in w_dtype).
 
     hidden, norm_eps: the pre-norm hidden state and eps given to ce_forward(norm_eps=...); dx is then the
-    gradient with respect to that hidden state."""
+    gradient with respect to that hidden state.
+    cache_generation: ``weight_cache.generation`` as it was right after the matching ce_forward; checked."""
     dev = saved.device
     n_predict, mtp_w = _mtp(mtp_weights, dev)
     sz = _lib.sizes_for(N, d, V, n_predict)
@@ -202,6 +216,9 @@ def ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale,
         a.norm, a.norm_eps = 1, float(norm_eps)
         a.x, a.x_dtype, a.x_ld = hidden.data_ptr(), _dtype_code(hidden, "hidden"), hidden.stride(0)
     if weight_cache is not None:
+        if cache_generation is not None and cache_generation != weight_cache.generation:
+            raise RuntimeError("the weight cache has been refilled since the forward pass this backward belongs to "
+                               f"(generation {weight_cache.generation}, forward saw {cache_generation})")
         a.wcache, a.wcache_bytes, a.wcache_valid = weight_cache.buf.data_ptr(), weight_cache.buf.numel(), 1
     _lib.check(_lib.lib().sce_backward(C.byref(a)), "sce_backward")
     return dx, dw

@@ -206,6 +206,20 @@ def test_vocabulary_slice_backward_and_weight_cache():
     loss3, *_ = ck.ce_forward(x, w2, y, inp.x_s, inp.w_s, inp.cap, "mean", vocab_size=vocab, weight_cache=cache)
     loss3_nocache, *_ = ck.ce_forward(x, w2, y, inp.x_s, inp.w_s, inp.cap, "mean", vocab_size=vocab)
     assert torch.equal(loss3, loss3_nocache)
+    # a write through .data is invisible to the version counter (tiny/train.py:1586 broadcasts parameters that way):
+    # the cache has to be told
+    w2.data.mul_(2.0)
+    gen = cache.generation
+    stale, *_ = ck.ce_forward(x, w2, y, inp.x_s, inp.w_s, inp.cap, "mean", vocab_size=vocab, weight_cache=cache)
+    assert torch.equal(stale, loss3) and cache.generation == gen
+    cache.invalidate()
+    loss4, saved4, *_ = ck.ce_forward(x, w2, y, inp.x_s, inp.w_s, inp.cap, "mean", vocab_size=vocab, weight_cache=cache)
+    loss4_nocache, *_ = ck.ce_forward(x, w2, y, inp.x_s, inp.w_s, inp.cap, "mean", vocab_size=vocab)
+    assert torch.equal(loss4, loss4_nocache) and cache.generation == gen + 1
+    # a backward that belongs to an older fill of the cache is refused
+    with pytest.raises(RuntimeError, match="refilled"):
+        ck.ce_backward(saved4, y, go, 520, 128, 1024, inp.x_s, inp.w_s, inp.cap, 1.0, "mean", torch.bfloat16, torch.bfloat16,
+                       vocab_size=vocab, weight_cache=cache, cache_generation=gen)
 
 
 def test_minimum_workspace_and_strided_rows():
