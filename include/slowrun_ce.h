@@ -154,6 +154,16 @@ int sce_transpose_bytes(const void* src, void* dst, int64_t rows, int64_t cols,
  * (fwd_workspace_bytes) and fills args->saved. */
 int sce_forward(const sce_args* args);
 
+/* sce_forward without a workspace: the scratch that sce_forward takes from args->workspace (the partial row
+ * statistics of the vocabulary splits) lives in a static device array of the library, 8 MiB on every GPU the
+ * library has run on, until the process ends.  No counterpart in the reference; it is for callers that cannot
+ * allocate: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The call allocates
+ * nothing and frees nothing; args->workspace and args->workspace_bytes are ignored, every other field means what it
+ * means to sce_forward, and the results are the same bits.  Limit: ceil(N / 256) * 256 * S <= 524288, S the number of
+ * vocabulary splits (8 to 16; 8 at N = 65536, V = 50304), else SCE_EINVAL with a message.  All calls on one device
+ * share the one array: calls that overlap in time on the same device (two streams, two threads) race. */
+int sce_forward_noalloc(const sce_args* args);
+
 /* Backward: recompute logit tiles from the saved fp8 operands, form dlogits on chip,
  * dX = dlogits * W_q^T, dW = X_q^T * dlogits.  Replaces
  * FusedSoftcappedCrossEntropy.backward (tiny/cuda_kernels.py:375-414) and the dlogits half

@@ -14,7 +14,7 @@ SCE_REDUCE_NONE, SCE_REDUCE_MEAN = 0, 1
 SCE_VERSION = 4
 
 EXPORTS = ("sce_version", "sce_last_error", "sce_sizes_for", "sce_quantize_e4m3", "sce_transpose_bytes",
-           "sce_forward", "sce_backward", "sce_timing_enable", "sce_timing_read")
+           "sce_forward", "sce_forward_noalloc", "sce_backward", "sce_timing_enable", "sce_timing_read")
 
 KERNEL_KINDS = ("quantize", "fwd", "fwd_reduce", "bwd_prep", "recompute", "dx", "dw", "dw_final")
 
@@ -71,6 +71,7 @@ def lib():
         L.sce_quantize_e4m3.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_double, C.c_size_t, C.c_int32, C.c_void_p]
         L.sce_transpose_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int32, C.c_void_p]
         L.sce_forward.argtypes = [C.POINTER(SceArgs)]
+        L.sce_forward_noalloc.argtypes = [C.POINTER(SceArgs)]
         L.sce_backward.argtypes = [C.POINTER(SceArgs)]
         L.sce_timing_enable.argtypes = [C.c_int]
         L.sce_timing_read.argtypes = [C.POINTER(SceTiming)]

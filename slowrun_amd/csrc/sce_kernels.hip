@@ -1530,8 +1530,15 @@ struct DeviceGuard {
   ~DeviceGuard() { if (prev >= 0) (void)hipSetDevice(prev); }
 };
 
+// Scratch of sce_forward_noalloc: the V-split partial records of the forward kernel (what sce_forward takes from the
+// caller's workspace).  Every GPU the library runs on holds its own copy until the process ends; in host code the
+// array's name is only a handle, the address on a device comes from hipGetSymbolAddress (g_scratch, below).
+constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)8 << 20;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+
 static std::mutex g_mu;
 static int g_arch_ok[64];   // 0 unknown, 1 gfx950, -1 other
+static void* g_scratch[64]; // device address of `scratch` on each device, filled with g_arch_ok
 static int g_cus[64];       // compute units, filled with g_arch_ok
 static inline int device_cus_or_default(int dev) { return (dev >= 0 && dev < 64 && g_cus[dev] > 0) ? g_cus[dev] : 256; }
 
@@ -1597,6 +1604,9 @@ static int check_device(int dev) {
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
+      void* sp = nullptr;
+      HIP_TRY(hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)));       // this device's copy of the array
+      g_scratch[dev] = sp;
       g_cus[dev] = prop.multiProcessorCount;
       g_arch_ok[dev] = 1;
     }
@@ -1803,8 +1813,8 @@ static int check_common(const sce_args* a) {
   return check_device(a->device);
 }
 
-extern "C" int sce_forward(const sce_args* a) {
-  if (int rc = check_common(a)) return rc;
+// ws: the partial records of the V-splits (the caller's workspace, or the library's static scratch)
+static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char* ws_name) {
   const int64_t N = a->shape.N, d = a->shape.d, V = a->shape.V;
   if (!a->x || !a->w) return fail(SCE_EINVAL, "x or w is NULL");
   if (a->x_ld < d || a->w_ld < V) return fail(SCE_EINVAL, "row strides smaller than the row length");
@@ -1858,9 +1868,9 @@ extern "C" int sce_forward(const sce_args* a) {
   const int CTw = emit ? (int)(S.Vp / 256) : CT;       // with the dlogits every tile is visited: the masked ones must read as zero later
   const int nsplit = fwd_splits(RT, CTw, device_cus_or_default(a->device));
   const size_t need_ws = (size_t)nsplit * S.Np * 16;
-  if (!a->workspace || a->workspace_bytes < need_ws) return fail(SCE_EINVAL, "forward workspace too small: %zu < %zu", a->workspace_bytes, need_ws);
+  if (!ws || ws_bytes < need_ws) return fail(SCE_EINVAL, "%s too small: %zu < %zu", ws_name, ws_bytes, need_ws);
   FwdParams p;
-  p.xq = xq; p.wqt = wqt; p.partials = (float4*)a->workspace;
+  p.xq = xq; p.wqt = wqt; p.partials = (float4*)ws;
   p.targets = a->targets; p.ignore_index = a->ignore_index; p.n_predict = a->shape.n_predict; p.s_uy = (float*)(sv + S.off_zy);
   p.ghat_t = emit ? gbase + S.rel_g : nullptr; p.gexp = emit ? (uint32_t*)(gbase + S.rel_gexp) : nullptr; p.kbw = S.Np / BK;
   p.dp = S.dp; p.ldx = S.ldx; p.N = (int)N; p.V = (int)Vl; p.Np = (int)S.Np; p.RT = RT; p.CT = CTw; p.S = nsplit;
@@ -1889,6 +1899,24 @@ extern "C" int sce_forward(const sce_args* a) {
                                         a->reduction == SCE_REDUCE_MEAN ? a->loss : nullptr, a->n_valid);
   HIP_TRY(hipGetLastError());
   return SCE_OK;
+}
+
+extern "C" int sce_forward(const sce_args* a) {
+  if (int rc = check_common(a)) return rc;
+  return forward_impl(a, a->workspace, a->workspace_bytes, "forward workspace");
+}
+
+// The same launches as sce_forward with the partial records in the library's static device array instead of a
+// caller's workspace: no allocation, by the caller for this call or by the library ever.  Calls on one device share
+// the array; nothing in it has to start at zero (the forward kernel writes every record that the combine kernel
+// reads), so nothing is cleared, but two calls in flight on one device at a time would overwrite each other's records.
+extern "C" int sce_forward_noalloc(const sce_args* a) {
+  if (int rc = check_common(a)) return rc;
+  void* sp = g_scratch[a->device];              // set by check_device (inside check_common) for this very device
+  if (!sp) return fail(SCE_EHIP, "no static scratch on device %d", a->device);
+  return forward_impl(a, sp, NOALLOC_SCRATCH_BYTES,
+                      "the static scratch of sce_forward_noalloc (8 MiB: N rounded up to 256 times the number of V-splits, 8 to 16, "
+                      "may not exceed 524288; use sce_forward with a workspace)");
 }
 
 extern "C" int sce_backward(const sce_args* a) {

@@ -134,8 +134,11 @@ class WeightCache:
 
 
 def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_weights=None, vocab_size=None,
-               weight_cache=None, norm_eps=None, keep_dlogits=False):
+               weight_cache=None, norm_eps=None, keep_dlogits=False, no_alloc=False):
     """One call of sce_forward.  Returns (out, saved, lse, argmax, n_valid).
+
+    no_alloc: call sce_forward_noalloc instead, which keeps its scratch in a static device array of the library (this
+    wrapper still allocates the outputs with torch; a caller that may not allocate passes buffers of its own to the C ABI).
 
     keep_dlogits: the forward pass also leaves the dlogits in ``saved`` (pass the same value to ce_backward).
 
@@ -154,7 +157,7 @@ def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_w
     sz = _lib.sizes_for(N, d, V, n_predict)
     saved = torch.empty((sz.saved_x_bytes if weight_cache is not None else sz.saved_bytes) + (sz.dlogits_bytes if keep_dlogits else 0),
                         dtype=torch.uint8, device=dev)
-    ws = torch.empty(sz.fwd_workspace_bytes, dtype=torch.uint8, device=dev)
+    ws = None if no_alloc else torch.empty(sz.fwd_workspace_bytes, dtype=torch.uint8, device=dev)
     losses = torch.empty(N, dtype=torch.float32, device=dev)
     lse = torch.empty(N, dtype=torch.float32, device=dev)
     loss = torch.empty(1, dtype=torch.float32, device=dev)
@@ -166,7 +169,8 @@ def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_w
     a.loss, a.losses, a.lse, a.n_valid = loss.data_ptr(), losses.data_ptr(), lse.data_ptr(), n_valid.data_ptr()
     a.argmax = argmax.data_ptr() if want_argmax else None
     a.saved, a.saved_bytes = saved.data_ptr(), saved.numel()
-    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    if ws is not None:
+        a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
     a.vocab_limit = 0 if vocab_size is None else int(vocab_size)
     a.dlogits_from_forward = int(bool(keep_dlogits))
     if norm_eps is not None:
@@ -174,7 +178,10 @@ def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_w
     if weight_cache is not None:
         wbuf, valid = weight_cache.prepare(w, w_s, sz.wcache_bytes)
         a.wcache, a.wcache_bytes, a.wcache_valid = wbuf.data_ptr(), wbuf.numel(), int(valid)
-    _lib.check(_lib.lib().sce_forward(C.byref(a)), "sce_forward")
+    if no_alloc:
+        _lib.check(_lib.lib().sce_forward_noalloc(C.byref(a)), "sce_forward_noalloc")
+    else:
+        _lib.check(_lib.lib().sce_forward(C.byref(a)), "sce_forward")
     out = loss.reshape(()) if reduction == "mean" else losses
     return out, saved, lse, argmax, n_valid
 
