@@ -17,10 +17,39 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP8_TFLOPS = 5000.0        # MI355X dense fp8 MFMA, published
 
-# HBM-side bytes per launch (fetched + written) of the MFMA kernels at the full limited_2p7b shape, from
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB device copy (factors 2.0 / 1.0); the
-# summary is profiles/bench_limited_2p7b_pmc.txt.  None for any other workload.
-MEASURED_TRAFFIC_GIB = {"fwd": 16.645 + 0.008, "recompute": 1.487 + 0.284, "dx": 1.331 + 0.031, "dw": 13.540 + 0.481}
+PROFILE_KERNEL = {"fwd": "fwd_kernel", "recompute": "bwd_recompute_kernel", "dx": "bwd_dx_kernel<bf16_t, false>",
+                  "dw": "bwd_dw_kernel<false>"}
+
+
+def measured_traffic(workload, mode, kind):
+    """HBM-side bytes per launch (fetched + written) of one kind of kernel, read from the committed rocprofv3
+    counter summary of this very workload and mode (profiles/bench_<workload>_<mode>_pmc.txt: FETCH_SIZE / WRITE_SIZE
+    scaled by a 1 GiB device copy), or None if there is none.  bench.py does not measure it itself: the counters need
+    the profiler."""
+    path = os.path.join(ROOT, "profiles", f"bench_{workload}_{mode}_pmc.txt")
+    try:
+        lines = open(path).read().splitlines()
+    except OSError:
+        return None
+    name = PROFILE_KERNEL.get(kind)
+    for ln in lines:
+        if name and ln.startswith(name + " "):
+            cols = ln[len(name):].split()
+            try:
+                return round((float(cols[1]) + float(cols[2])) * 2 ** 30)        # launches, fetched GiB/launch, written GiB/launch
+            except (IndexError, ValueError):
+                return None
+    return None
+
+
+def cpu_model():
+    try:
+        for ln in open("/proc/cpuinfo"):
+            if ln.startswith("model name"):
+                return ln.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def cpu_baseline(inp, rows, threads):
@@ -28,7 +57,6 @@ def cpu_baseline(inp, rows, threads):
     on the first `rows` rows against the full W."""
     import torch
     from oracle import eager
-    torch.set_num_threads(threads)
     x = inp.x[:rows].bfloat16()
     w = inp.w.bfloat16()
     y = inp.targets[:rows]
@@ -129,8 +157,7 @@ def main():
     roofline = {
         "bound": "mfma", "kernel": dom, "achieved": kernels[dom]["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
         "frac": round(kernels[dom]["tflops"] / PEAK_FP8_TFLOPS, 4),
-        "traffic": (round(MEASURED_TRAFFIC_GIB[dom] * 2 ** 30) if (args.workload == "limited_2p7b" and args.rows is None
-                                                                   and args.panel_rows == 0) else None),
+        "traffic": (measured_traffic(args.workload, args.dlogits, dom) if (args.rows is None and args.panel_rows == 0) else None),
         "avg_launch_ms": kernels[dom]["avg_launch_ms"],
     }
     result = {
@@ -138,21 +165,26 @@ def main():
         "value": round(tokens_per_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp8_e4m3", "data": "synthetic",
-        "config": {"workload": f"{inp.name}: N={N}, d={d}, V={V}, cap={inp.cap}, fp8 e4m3 amax scales, bf16 dX/dW, mean reduction"},
+        "config": {"workload": f"{inp.name}: N={N}, d={d}, V={V}, cap={inp.cap}, fp8 e4m3 amax scales, bf16 dX/dW, mean reduction",
+                   "dlogits": ("kept from the forward pass (8 bits per logit held until backward)" if keep
+                               else "recomputed in backward (nothing N x V held)")},
         "algorithmic_tflops": round(flops_step / (ms_per_step * 1e-3) * 1e-12, 1),
         "frac_fp8_mfma_peak": round(flops_step / (ms_per_step * 1e-3) * 1e-12 / PEAK_FP8_TFLOPS, 4),
-        "hardware_flops_per_step": 8.0 * N * d * V,
+        "hardware_flops_per_step": (6.0 if keep else 8.0) * N * d * V,
         "loss": loss,
         "wall_s_timed_region": round(wall, 3),
         "roofline": roofline,
         "kernels": kernels,
     }
     if not args.no_cpu_baseline:
-        threads = min(16, os.cpu_count() or 1)
+        # every core this process has been given: torch's default thread count follows the OMP_NUM_THREADS the box sets
+        # (its share of the host), not os.cpu_count(), which shows the whole machine
+        threads = torch.get_num_threads()
         rows = min(args.cpu_rows, N)
         tps, dt = cpu_baseline(inp, rows, threads)
         result["cpu_baseline"] = {
             "value": round(tps, 1), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "host_cpus": os.cpu_count(), "cpu_model": cpu_model(), "torch_threads": threads,
             "sample": f"eager fp8-quantise + fp32 matmul + softcap + F.cross_entropy fwd+bwd on the first {rows} rows "
                       f"against the full (d,V) weight, {dt:.1f} s, torch {torch.__version__} with {threads} threads",
         }

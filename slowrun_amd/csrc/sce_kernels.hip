@@ -393,14 +393,19 @@ __global__ __launch_bounds__(256) void transpose_bytes_kernel(const uint8_t* __r
 constexpr int STG_PITCH = 272;                               // 256 + 16: 16-byte aligned, rows shifted by 4 banks
 constexpr int STG_BYTES = 256 * STG_PITCH;                   // 69632
 
+// Maximum over the 64 lanes, in every lane.  The lane exchanges are LDS-crossbar swizzles with the pattern in the
+// instruction (xor 1 .. 16 within a half-wave), and one ds_bpermute across the halves whose address comes from
+// lane_id(): __shfl_xor would keep its own copy of the lane index alive across the main loop, where it is spilled.
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
+#define SCE_SWZ_MAX(X) v = fmaxf(v, __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), ((X) << 10) | 0x1f)))
+  SCE_SWZ_MAX(1); SCE_SWZ_MAX(2); SCE_SWZ_MAX(4); SCE_SWZ_MAX(8); SCE_SWZ_MAX(16);
+#undef SCE_SWZ_MAX
+  return fmaxf(v, __int_as_float(__builtin_amdgcn_ds_bpermute((lane_id() ^ 32) << 2, __float_as_int(v))));
 }
 
-// lam (LDS, one float per lane and row block, LAM_STRIDE floats apart): the row's exponent boost (see fwd_sample_kernel).
-template <bool EDGE, bool STATS, int LAM_STRIDE = NTHREADS>
+// lam (LDS, wave-uniform base; per row block LAM_STRIDE floats apart, one float for each of LAM_LANES lanes): the row's
+// exponent boost (see fwd_sample_kernel).
+template <bool EDGE, bool STATS, int LAM_STRIDE = NTHREADS, int LAM_LANES = 64>
 __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float k1, float c2, int vlim, int vabs0,
                                                  uint8_t* TT, int wa, int wb, float* stat, const float* lam) {
   const int lane = lane_id();
@@ -422,7 +427,7 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
         if (EDGE && vloc0 + a * 32 + 8 * (r >> 2) + (r & 3) >= vlim) x = -INFINITY;
         tmax = fmaxf(tmax, x);
       }
-    const float lamb = lam[b * LAM_STRIDE];
+    const float lamb = lam[b * LAM_STRIDE + (lane_id() & (LAM_LANES - 1))];      // (index taken anew: see lane_id)
     const float lg = wave_max(fmaf(c2, fast_rcp(1.0f + fast_exp2(tmax * k1)), lamb));      // over the block: log2 of the largest boosted e^{z - cap}
     const float sb = floorf(8.8f - lg);                       // between -120 and 8 + 2 cap log2(e) <= 124 (cap <= 40, boost <= 120)
     const float cs = sb + 2.0f + lamb;                        // the 4 of 4 r (1 - r) and the row's boost ride along
@@ -635,7 +640,8 @@ __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int*
             }
           }
           xk[k] = x;
-          if (STORE) s_uy_tile[(int64_t)k * Np + rowbase + row] = x * sc;
+          // (the lane index is taken anew: an address kept from outside the branch stays live across the main loop and is spilled)
+          if (STORE) s_uy_tile[(int64_t)k * Np + rowbase + b * 32 + (lane_id() & 31)] = x * sc;
         }
       }
     }
@@ -744,8 +750,9 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p) {
       const int vlim = p.V - ct * 256;
       uint8_t* TT = smem + FWD_STAGE_OFF;
       uint32_t ew;
-      if (vlim < 256) ew = form_dlogits<true, true>(acc, p.k1, p.c2, vlim, vbase, TT, wa, wb, stat, stat + 12 * NTHREADS);
-      else ew = form_dlogits<false, true>(acc, p.k1, p.c2, vlim, vbase, TT, wa, wb, stat, stat + 12 * NTHREADS);
+      const float* lam = reinterpret_cast<const float*>(smem + FWD_STAT_OFF) + 12 * NTHREADS + wave * 64;
+      if (vlim < 256) ew = form_dlogits<true, true>(acc, p.k1, p.c2, vlim, vbase, TT, wa, wb, stat, lam);
+      else ew = form_dlogits<false, true>(acc, p.k1, p.c2, vlim, vbase, TT, wa, wb, stat, lam);
       store_dlogits_quadrant(TT, p.ghat_t + ((int64_t)ct * p.kbw + 2 * rt + wb) * BLOCKED_KSTEP + wa * 128 * BK, wa, wb);
       if (lane_id() == 0) p.gexp[(int64_t)(2 * ct + wa) * p.kbw + 2 * rt + wb] = ew;
     } else {
@@ -1059,12 +1066,12 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
   v16f acc[4][4];
   mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 2 * (rt & 3), ct & 7, wave);
   const int vlim = p.V - ct * 256;           // columns >= vlim of this tile do not exist
-  const float* lam = reinterpret_cast<const float*>(smem + SMEM_BYTES) + wave * (ROWINFO_PLANES * 128) + (lane_id() & 31);     // row block b: 32 floats on
+  const float* lam = reinterpret_cast<const float*>(smem + SMEM_BYTES) + wave * (ROWINFO_PLANES * 128);     // row block b: 32 floats on
   const int* tgt = reinterpret_cast<const int*>(smem + SMEM_BYTES) + wave * (ROWINFO_PLANES * 128) + 128;
   take_target_logits<false, true, false, 128>(acc, tgt, p.n_predict, ct * 256 + wa * 128, 0, 0.f, nullptr, 0, nullptr, 0.f, 0.f);
   uint32_t ew;
-  if (vlim < 256) ew = form_dlogits<true, false, 32>(acc, p.k1, p.c2, vlim, 0, smem, wa, wb, nullptr, lam);
-  else ew = form_dlogits<false, false, 32>(acc, p.k1, p.c2, vlim, 0, smem, wa, wb, nullptr, lam);
+  if (vlim < 256) ew = form_dlogits<true, false, 32, 32>(acc, p.k1, p.c2, vlim, 0, smem, wa, wb, nullptr, lam);
+  else ew = form_dlogits<false, false, 32, 32>(acc, p.k1, p.c2, vlim, 0, smem, wa, wb, nullptr, lam);
   store_dlogits_quadrant(smem, p.ghat_t + ((int64_t)ct * p.kbw + p.kb0 + 2 * rt + wb) * BLOCKED_KSTEP + wa * 128 * BK, wa, wb);
   if (lane_id() == 0) p.gexp[(int64_t)(2 * ct + wa) * p.kbw + p.kb0 + 2 * rt + wb] = ew;
 }
@@ -1949,8 +1956,8 @@ extern "C" int sce_backward(const sce_args* a) {
   int64_t P, Pw;
   int nparts;
   if (kept) {
-    // no producer to stay close to: dX takes all rows at once (as many as one dW launch may contract over)
-    P = a->panel_rows > 0 ? a->panel_rows : S.Np;
+    // dX still goes panel by panel, one round of tiles each: a launch with several rounds was measured 2 % slower
+    P = a->panel_rows > 0 ? a->panel_rows : default_panel(S);
     if (P > S.Np) P = S.Np;
     if (P > 131072) P = 131072;
     Pw = default_dw_panel(S, P);
