@@ -120,6 +120,12 @@ typedef struct sce_args {
                                 (saved_bytes or saved_x_bytes, plus dlogits_bytes) and backward is two GEMMs instead of
                                 three.  Same value in both calls.  The reference keeps bf16 logits and e5m2 dlogits
                                 (tiny/cuda_kernels.py:359-371)                                                       */
+  const float* x_s_dev;      /* NULL, or a device float that holds the scale of X: read when the kernels run, not when the
+                                call is made, so it may be the result of earlier work on the stream (an amax pass, see
+                                sce_amax_scale) and may change between replays of a captured graph; x_s is then ignored.
+                                The quantiser then divides (x / s) as torch does for a tensor divisor.  Same in forward
+                                and backward (backward reads the value forward used from `saved`)                       */
+  const float* w_s_dev;      /* the same for W                                                                           */
 } sce_args;
 
 /* Library / ABI version (SCE_VERSION of the build). */
@@ -141,6 +147,16 @@ int sce_sizes_for(const sce_shape* shape, sce_sizes* out);
  * x.div(x_s).to(torch.float8_e4m3fn) (tiny/cuda_kernels.py:340-341), which runs on the GPU. */
 int sce_quantize_e4m3(const void* src, int32_t src_dtype, void* dst, double scale, size_t n,
                       int32_t device, void* stream);
+
+/* The same with the scale in device memory (a 0-dim tensor): dst[i] = e4m3_rne(src[i] / *scale_dev), a true
+ * division, which is what torch computes for a tensor divisor; nothing is read on the host. */
+int sce_quantize_e4m3_dev(const void* src, int32_t src_dtype, void* dst, const float* scale_dev, size_t n,
+                          int32_t device, void* stream);
+
+/* *scale_out (a device float) = max |src[i]| / 448, the per-tensor "amax" scale of the fp8 cast, for
+ * x_s_dev / w_s_dev; NaN if any element is NaN.  Replaces a host-side `float(t.abs().max()) / 448` (the reference's
+ * scales are constants, tiny/train.py:188-189; a trainer that rescales per step does this). */
+int sce_amax_scale(const void* src, int32_t src_dtype, size_t n, float* scale_out, int32_t device, void* stream);
 
 /* dst (cols, rows) = transpose of src (rows, cols), one byte per element.  Replaces
  * transpose_copy (tiny/cuda_kernels.py:56-78) for callers that still want it; the fused

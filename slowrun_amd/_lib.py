@@ -13,7 +13,8 @@ SCE_F32, SCE_BF16 = 0, 1
 SCE_REDUCE_NONE, SCE_REDUCE_MEAN = 0, 1
 SCE_VERSION = 4
 
-EXPORTS = ("sce_version", "sce_last_error", "sce_sizes_for", "sce_quantize_e4m3", "sce_transpose_bytes",
+EXPORTS = ("sce_version", "sce_last_error", "sce_sizes_for", "sce_quantize_e4m3", "sce_quantize_e4m3_dev", "sce_amax_scale",
+           "sce_transpose_bytes",
            "sce_forward", "sce_forward_noalloc", "sce_backward", "sce_timing_enable", "sce_timing_read")
 
 KERNEL_KINDS = ("quantize", "fwd", "fwd_reduce", "bwd_prep", "recompute", "dx", "dw", "dw_final")
@@ -46,6 +47,7 @@ class SceArgs(C.Structure):
         ("panel_rows", C.c_int64),
         ("vocab_limit", C.c_int64), ("wcache", C.c_void_p), ("wcache_bytes", C.c_size_t),
         ("wcache_valid", C.c_int32), ("norm", C.c_int32), ("norm_eps", C.c_float), ("dlogits_from_forward", C.c_int32),
+        ("x_s_dev", C.c_void_p), ("w_s_dev", C.c_void_p),
     ]
 
 
@@ -69,6 +71,8 @@ def lib():
         L.sce_last_error.restype = C.c_char_p
         L.sce_sizes_for.argtypes = [C.POINTER(SceShape), C.POINTER(SceSizes)]
         L.sce_quantize_e4m3.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_double, C.c_size_t, C.c_int32, C.c_void_p]
+        L.sce_quantize_e4m3_dev.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int32, C.c_void_p]
+        L.sce_amax_scale.argtypes = [C.c_void_p, C.c_int32, C.c_size_t, C.c_void_p, C.c_int32, C.c_void_p]
         L.sce_transpose_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int32, C.c_void_p]
         L.sce_forward.argtypes = [C.POINTER(SceArgs)]
         L.sce_forward_noalloc.argtypes = [C.POINTER(SceArgs)]

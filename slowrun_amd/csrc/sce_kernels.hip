@@ -65,6 +65,8 @@ template <> struct Elem<float> {
   // x.div(s) with a host scalar s as torch's GPU kernels compute it: x * (1 / s), the reciprocal taken once in fp32
   // (the CPU kernels divide; the two differ in the last bit now and then, which moves an fp8 tie)
   static __device__ __forceinline__ float div_round(float x, float inv_s) { return x * inv_s; }
+  // x.div(s) with s a device scalar (a 0-dim tensor): a true division, on the GPU too
+  static __device__ __forceinline__ float div_true(float x, float s) { return x / s; }
 };
 struct bf16_t { uint16_t bits; };
 template <> struct Elem<bf16_t> {
@@ -72,7 +74,40 @@ template <> struct Elem<bf16_t> {
   static __device__ __forceinline__ void store(bf16_t* p, float v) { p->bits = float_to_bf16_bits(v); }
   // torch scales a bf16 tensor in fp32 and rounds the result back to bf16 before the fp8 cast
   static __device__ __forceinline__ float div_round(float x, float inv_s) { return round_to_bf16(x * inv_s); }
+  static __device__ __forceinline__ float div_true(float x, float s) { return round_to_bf16(x / s); }
 };
+
+// How the quantisers apply the fp8 scale: `by` is 1 / s (host scalar: multiplied in) or, with `divide`, s itself read
+// from device memory (true division), in both cases what torch's GPU kernels do for that kind of divisor.
+struct Scaler {
+  float by;
+  bool divide;
+  template <typename T>
+  __device__ __forceinline__ float apply(float x) const { return divide ? Elem<T>::div_true(x, by) : Elem<T>::div_round(x, by); }
+};
+// scale_dev != NULL: the scale lives on the device.  torch brings a 0-dim tensor divisor to the dtype of the tensor it
+// divides before it divides (a bf16 tensor is divided by the scale rounded to bf16); a Python-float divisor is not.
+template <typename T>
+__device__ __forceinline__ Scaler make_scaler(float inv_host, const float* scale_dev) {
+  Scaler sc;
+  sc.divide = scale_dev != nullptr;
+  sc.by = sc.divide ? (sizeof(T) == 2 ? round_to_bf16(*scale_dev) : *scale_dev) : inv_host;
+  return sc;
+}
+
+// Scale-derived constants when a scale lives on the device (sce_args.x_s_dev / w_s_dev): written by dev_consts_kernel
+// into the header of the saved state, read by every kernel that needs them in place of its by-value copies.
+struct DevConsts {
+  float x_s, w_s, sc, k1;      // sc = x_s w_s; k1 = sc 2 log2(e) / cap
+};
+__global__ void dev_consts_kernel(const float* xs_dev, const float* ws_dev, float xs_host, float ws_host, float cap, DevConsts* out) {
+  DevConsts c;
+  c.x_s = xs_dev ? *xs_dev : xs_host;
+  c.w_s = ws_dev ? *ws_dev : ws_host;
+  c.sc = c.x_s * c.w_s;
+  c.k1 = c.sc * 2.0f * LOG2E / cap;
+  *out = c;
+}
 
 // XCD-aware tile order.  Consecutive workgroup ids go round-robin to the 8 XCDs, each with its
 // own L2.  The tiles are put in a locality-preserving order (groups of 8 columns, walked row by
@@ -114,40 +149,42 @@ static inline int map_tile_rr_grid(int RT, int CT) { return 256 * ((RT * CT + 25
 // ------------------------------------------------------------------------------------------
 // quantisation
 // ------------------------------------------------------------------------------------------
-// 16 consecutive elements starting at p as floats after the scaling by 1 / s; elements at or beyond
+// 16 consecutive elements starting at p as floats after the scaling; elements at or beyond
 // `valid` are 0.  One or two 16/32-byte vector loads when the run is complete and 16-byte aligned.
 template <typename T>
-__device__ __forceinline__ void load16_scaled(const T* __restrict__ p, int64_t valid, float scale, float (&v)[16]) {     // scale: 1 / s
+__device__ __forceinline__ void load16_scaled(const T* __restrict__ p, int64_t valid, const Scaler scale, float (&v)[16]) {
   if (valid >= 16 && (((uintptr_t)p) & 15) == 0) {
     if constexpr (sizeof(T) == 2) {
       const v4i r0 = *reinterpret_cast<const v4i*>(p), r1 = *reinterpret_cast<const v4i*>(p + 8);
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
-        v[2 * m] = Elem<T>::div_round(__uint_as_float((uint32_t)r0[m] << 16), scale);
-        v[2 * m + 1] = Elem<T>::div_round(__uint_as_float((uint32_t)r0[m] & 0xffff0000u), scale);
-        v[8 + 2 * m] = Elem<T>::div_round(__uint_as_float((uint32_t)r1[m] << 16), scale);
-        v[8 + 2 * m + 1] = Elem<T>::div_round(__uint_as_float((uint32_t)r1[m] & 0xffff0000u), scale);
+        v[2 * m] = scale.apply<T>(__uint_as_float((uint32_t)r0[m] << 16));
+        v[2 * m + 1] = scale.apply<T>(__uint_as_float((uint32_t)r0[m] & 0xffff0000u));
+        v[8 + 2 * m] = scale.apply<T>(__uint_as_float((uint32_t)r1[m] << 16));
+        v[8 + 2 * m + 1] = scale.apply<T>(__uint_as_float((uint32_t)r1[m] & 0xffff0000u));
       }
     } else {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const v4f r = *reinterpret_cast<const v4f*>(p + 4 * q);
 #pragma unroll
-        for (int m = 0; m < 4; ++m) v[4 * q + m] = Elem<T>::div_round(r[m], scale);
+        for (int m = 0; m < 4; ++m) v[4 * q + m] = scale.apply<T>(r[m]);
       }
     }
   } else {
 #pragma unroll
-    for (int m = 0; m < 16; ++m) v[m] = (m < valid) ? Elem<T>::div_round(Elem<T>::load(p + m), scale) : 0.f;
+    for (int m = 0; m < 16; ++m) v[m] = (m < valid) ? scale.apply<T>(Elem<T>::load(p + m)) : 0.f;
   }
 }
 
-// dst [rows_p][cols_p] e4m3 = src [rows][cols] * scale, zero outside; 16 outputs per thread.  In all the
-// quantising kernels `scale` is the reciprocal 1 / s of the fp8 scale s, taken once on the host.
+// dst [rows_p][cols_p] e4m3 = src [rows][cols] / s, zero outside; 16 outputs per thread.  In all the quantising
+// kernels inv_scale is the reciprocal 1 / s taken once on the host, or, with scale_dev, s is read from the device.
 template <typename T>
 __global__ __launch_bounds__(256) void quantize_pad_kernel(const T* __restrict__ src, int64_t ld, int64_t rows,
                                                           int64_t cols, uint8_t* __restrict__ dst,
-                                                          int64_t rows_p, int64_t cols_p, int64_t dst_ld, float scale) {
+                                                          int64_t rows_p, int64_t cols_p, int64_t dst_ld, float inv_scale,
+                                                          const float* __restrict__ scale_dev) {
+  const Scaler scale = make_scaler<T>(inv_scale, scale_dev);
   const int64_t chunks_per_row = cols_p / 16;
   const int64_t total = rows_p * chunks_per_row;
   for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < total; q += (int64_t)gridDim.x * blockDim.x) {
@@ -175,8 +212,9 @@ __device__ __forceinline__ float wave_sum(float v) {
 template <typename T>
 __global__ __launch_bounds__(256) void rmsnorm_quantize_kernel(const T* __restrict__ src, int64_t ld, int64_t rows,
                                                               int64_t cols, float eps, uint8_t* __restrict__ dst,
-                                                              int64_t rows_p, int64_t cols_p, int64_t dst_ld, float scale,
-                                                              float* __restrict__ rstd_out) {
+                                                              int64_t rows_p, int64_t cols_p, int64_t dst_ld, float inv_scale,
+                                                              const float* __restrict__ scale_dev, float* __restrict__ rstd_out) {
+  const Scaler scale = make_scaler<T>(inv_scale, scale_dev), one = {1.0f, false};
   const int lane = threadIdx.x & 63;
   const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= rows_p) return;
@@ -190,7 +228,7 @@ __global__ __launch_bounds__(256) void rmsnorm_quantize_kernel(const T* __restri
   float ss = 0.f;
   for (int64_t c = lane; c * 16 < cols; c += 64) {
     float v[16];
-    load16_scaled<T>(row + c * 16, cols - c * 16, 1.0f, v);      // scaling by 1 is exact: the values themselves
+    load16_scaled<T>(row + c * 16, cols - c * 16, one, v);      // scaling by 1 is exact: the values themselves
 #pragma unroll
     for (int m = 0; m < 16; ++m) ss = fmaf(v[m], v[m], ss);
   }
@@ -201,12 +239,12 @@ __global__ __launch_bounds__(256) void rmsnorm_quantize_kernel(const T* __restri
     uint32_t out[4] = {0, 0, 0, 0};
     if (c * 16 < cols) {
       float v[16];
-      load16_scaled<T>(row + c * 16, cols - c * 16, 1.0f, v);
+      load16_scaled<T>(row + c * 16, cols - c * 16, one, v);
 #pragma unroll
       for (int m = 0; m < 16; ++m) {
         float y = v[m] * rstd;
         if constexpr (sizeof(T) == 2) y = round_to_bf16(y);
-        v[m] = Elem<T>::div_round(y, scale);
+        v[m] = scale.apply<T>(y);
       }
 #pragma unroll
       for (int m = 0; m < 4; ++m) out[m] = cvt4_e4m3(v[4 * m], v[4 * m + 1], v[4 * m + 2], v[4 * m + 3]);
@@ -299,7 +337,9 @@ constexpr int BLOCKED_KSTEP = 256 * BK;     // bytes from one K block of a tile 
 template <typename T>
 __global__ __launch_bounds__(256) void quantize_w_kernel(const T* __restrict__ w, int64_t ld, int64_t d, int64_t V,
                                                         uint8_t* __restrict__ wq, uint8_t* __restrict__ wqt,
-                                                        int64_t dp, int64_t ldx, int64_t kbv, float scale) {
+                                                        int64_t dp, int64_t ldx, int64_t kbv, float inv_scale,
+                                                        const float* __restrict__ scale_dev) {
+  const Scaler scale = make_scaler<T>(inv_scale, scale_dev);
   __shared__ uint8_t tile[64][68];
   const int t = threadIdx.x;
   const int64_t j0 = (int64_t)blockIdx.y * 64, v0 = (int64_t)blockIdx.x * 64;
@@ -333,11 +373,12 @@ __global__ __launch_bounds__(256) void quantize_w_kernel(const T* __restrict__ w
 // flat cast, for the standalone sce_quantize_e4m3 entry point
 template <typename T>
 __global__ __launch_bounds__(256) void quantize_flat_kernel(const T* __restrict__ src, uint8_t* __restrict__ dst,
-                                                           size_t n, float scale) {
+                                                           size_t n, float inv_scale, const float* __restrict__ scale_dev) {
+  const Scaler scale = make_scaler<T>(inv_scale, scale_dev);
   for (size_t q = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; q < n; q += (size_t)gridDim.x * blockDim.x * 4) {
     float v[4];
 #pragma unroll
-    for (int m = 0; m < 4; ++m) v[m] = (q + m < n) ? Elem<T>::div_round(Elem<T>::load(src + q + m), scale) : 0.f;
+    for (int m = 0; m < 4; ++m) v[m] = (q + m < n) ? scale.apply<T>(Elem<T>::load(src + q + m)) : 0.f;
     const uint32_t w = cvt4_e4m3(v[0], v[1], v[2], v[3]);
     if (q + 4 <= n && (((uintptr_t)(dst + q)) & 3) == 0) {
       *reinterpret_cast<uint32_t*>(dst + q) = w;
@@ -346,6 +387,27 @@ __global__ __launch_bounds__(256) void quantize_flat_kernel(const T* __restrict_
     }
   }
 }
+
+// max |src| over n elements, as the bits of a non-negative float (they order like unsigned integers, NaN above
+// everything); *bits starts at 0 (amax_begin_kernel) and ends as max / 448 (amax_end_kernel).
+__global__ void amax_begin_kernel(uint32_t* bits) { *bits = 0u; }
+template <typename T>
+__global__ __launch_bounds__(256) void amax_kernel(const T* __restrict__ src, size_t n, uint32_t* __restrict__ bits) {
+  __shared__ uint32_t smax[256];
+  uint32_t m = 0u;
+  for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < n; q += (size_t)gridDim.x * blockDim.x) {
+    const uint32_t b = __float_as_uint(Elem<T>::load(src + q)) & 0x7fffffffu;
+    m = b > m ? b : m;
+  }
+  smax[threadIdx.x] = m;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if (threadIdx.x < w) smax[threadIdx.x] = smax[threadIdx.x] > smax[threadIdx.x + w] ? smax[threadIdx.x] : smax[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) atomicMax(bits, smax[0]);
+}
+__global__ void amax_end_kernel(uint32_t* bits) { *reinterpret_cast<float*>(bits) = __uint_as_float(*bits) / 448.0f; }
 
 // dst (cols, rows) = src (rows, cols)^T, bytes.
 __global__ __launch_bounds__(256) void transpose_bytes_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
@@ -534,6 +596,7 @@ struct FwdParams {
   float k1;                // x_s * w_s * 2 log2(e) / cap : exp2(acc * k1) = e^{2u/cap}
   float ic2;               // 1 / c2, c2 = -2 cap log2(e): e^{z - cap} = exp2(c2 / (1 + e^{2u/cap}))
   float c2;
+  const DevConsts* dc;     // non-NULL: sc and k1 come from here (a scale lives on the device)
 };
 
 // Per 256 x 256 tile and per row a lane owns: add up e^{z - cap} over its 64 columns and keep the
@@ -651,8 +714,10 @@ __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int*
 // The exponent boost of every row, from one tile of its logits (256 columns from the middle of the vocabulary):
 // lam_i = floor(-log2 m_i), m_i the smallest of the means of e^{z - cap} over 16 groups of 16 columns -- the smallest,
 // so that a few peaks inside the sample (a target, say) do not pass for the level of the row.  One workgroup per row tile.
-__global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p, int ct, float* __restrict__ lam_out) {
+__global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct, float* __restrict__ lam_out) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  FwdParams p = p_in;
+  if (p.dc) { p.sc = p.dc->sc; p.k1 = p.dc->k1; }
   const int rt = blockIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wa = wave >> 1, wb = wave & 1;
   v16f acc[4][4];
@@ -707,8 +772,10 @@ static_assert(FWD_STAGE_OFF + STG_BYTES <= FWD_STAT_OFF, "staging tile and row s
 // EMIT: the epilogue also leaves the block-scaled dlogits of the tile in G^T (see form_dlogits), for a backward pass
 // that does not compute the logits again.
 template <bool EMIT>
-__global__ __launch_bounds__(256) void fwd_kernel(FwdParams p) {
+__global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  FwdParams p = p_in;
+  if (p.dc) { p.sc = p.dc->sc; p.k1 = p.dc->k1; }
   int rt, s;
   if (!map_tile(blockIdx.x, p.RT, p.S, rt, s)) return;
   const int ct0 = (int)((int64_t)p.CT * s / p.S), ct1 = (int)((int64_t)p.CT * (s + 1) / p.S);
@@ -1032,6 +1099,7 @@ struct RecomputeParams {
   int64_t kbw, kb0;            // ghat_t (blocked): K blocks per tile, K block of this panel's first row
   int RT, CT, V;
   float k1, c2;          // as in FwdParams
+  const DevConsts* dc;   // non-NULL: k1 comes from here
 };
 
 // Recompute a 256 x 256 logit tile and leave its block-scaled dlogits in G^T.  The tile is assembled in LDS (free
@@ -1040,8 +1108,10 @@ constexpr int ROWINFO_PLANES = 5;                      // per row: exponent boos
 constexpr int SMEM_RECOMPUTE = SMEM_BYTES + 4 * ROWINFO_PLANES * 512;      // two K slots (the staging tile reuses them) + the row data of 128 rows per wave
 static_assert(STG_BYTES <= SMEM_BYTES, "the staging tile must fit the K slots");
 
-__global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p) {
+__global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p_in) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  RecomputeParams p = p_in;
+  if (p.dc) p.k1 = p.dc->k1;
   int rt, ct;
   if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
   // The tile order goes through the columns in groups of 8, and it does so from the last group to the first:
@@ -1092,6 +1162,7 @@ struct DxParams {
   int n_predict, rows_left; // rows_left: N - (first row of the panel), bounds the target look-ahead
   int ksplit;              // the K loop (V) is cut into this many parts, one workgroup each
   float w_s;
+  const DevConsts* dc;     // non-NULL: w_s comes from here
 };
 
 // Row scale and one-hot term of four consecutive dX columns j..j+3 of panel row il:
@@ -1140,8 +1211,10 @@ struct DxRowTerms {
 // SPLIT = true : a panel with too few tiles to fill the chip; each tile's K loop is shared by ksplit
 //                workgroups that store raw fp32 partial sums, and bwd_dx_finish_kernel adds them up.
 template <typename T, bool SPLIT>
-__global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p) {
+__global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p_in) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  DxParams p = p_in;
+  if (p.dc) p.w_s = p.dc->w_s;
   int rt, ct, ks = 0;
   if (!map_tile(blockIdx.x, p.RT, SPLIT ? p.CT * p.ksplit : p.CT, rt, ct)) return;
   int64_t k0 = 0;
@@ -1291,7 +1364,9 @@ __global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p) {
 
 // sum of the K-split partials, row scale, one-hot term, cast: a thread per (row, four columns)
 template <typename T>
-__global__ __launch_bounds__(256) void bwd_dx_finish_kernel(DxParams p) {
+__global__ __launch_bounds__(256) void bwd_dx_finish_kernel(DxParams p_in) {
+  DxParams p = p_in;
+  if (p.dc) p.w_s = p.dc->w_s;
   const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int per_row = p.d / 4;
   const int il = (int)(q / per_row), j = (int)(q - (int64_t)il * per_row) * 4;
@@ -1457,7 +1532,8 @@ __global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restri
                                                           const int32_t* __restrict__ perm, const float* __restrict__ hcoef,
                                                           const uint8_t* __restrict__ xq, int64_t ldx, int Np, const float* __restrict__ xi,
                                                           const float* __restrict__ longsum, const int32_t* __restrict__ longbase, int64_t dq,
-                                                          float x_s, int d, int V, T* __restrict__ dw, int64_t dw_ld) {
+                                                          float x_s_host, const DevConsts* __restrict__ dc, int d, int V, T* __restrict__ dw, int64_t dw_ld) {
+  const float x_s = dc ? dc->x_s : x_s_host;
   const int t = threadIdx.x;
   const int v = blockIdx.x * 64 + (t & 63);
   const int j0 = blockIdx.y * 64 + (t >> 6) * 16;
@@ -1775,19 +1851,49 @@ static int grid_for(size_t work_items, int per_block) {
   return (int)g;
 }
 
-extern "C" int sce_quantize_e4m3(const void* src, int32_t src_dtype, void* dst, double scale, size_t n, int32_t device,
-                                 void* stream) {
+static int quantize_impl(const void* src, int32_t src_dtype, void* dst, float inv_scale, const float* scale_dev, size_t n, int32_t device,
+                         void* stream) {
   if (!src || !dst) return fail(SCE_EINVAL, "src/dst is NULL");
-  if (!(scale > 0.0)) return fail(SCE_EINVAL, "scale must be positive");
   if (int rc = check_device(device)) return rc;
   if (n == 0) return SCE_OK;
   DeviceGuard guard(device);
   if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", device);
   hipStream_t st = (hipStream_t)stream;
   const int grid = grid_for((n + 3) / 4, 256);
-  if (src_dtype == SCE_F32) quantize_flat_kernel<float><<<grid, 256, 0, st>>>((const float*)src, (uint8_t*)dst, n, (float)(1.0 / scale));
-  else if (src_dtype == SCE_BF16) quantize_flat_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)src, (uint8_t*)dst, n, (float)(1.0 / scale));
+  if (src_dtype == SCE_F32) quantize_flat_kernel<float><<<grid, 256, 0, st>>>((const float*)src, (uint8_t*)dst, n, inv_scale, scale_dev);
+  else if (src_dtype == SCE_BF16) quantize_flat_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)src, (uint8_t*)dst, n, inv_scale, scale_dev);
   else return fail(SCE_EINVAL, "unsupported dtype %d", src_dtype);
+  HIP_TRY(hipGetLastError());
+  return SCE_OK;
+}
+
+extern "C" int sce_quantize_e4m3(const void* src, int32_t src_dtype, void* dst, double scale, size_t n, int32_t device,
+                                 void* stream) {
+  if (!(scale > 0.0)) return fail(SCE_EINVAL, "scale must be positive");
+  return quantize_impl(src, src_dtype, dst, (float)(1.0 / scale), nullptr, n, device, stream);
+}
+
+extern "C" int sce_quantize_e4m3_dev(const void* src, int32_t src_dtype, void* dst, const float* scale_dev, size_t n, int32_t device,
+                                     void* stream) {
+  if (!scale_dev) return fail(SCE_EINVAL, "scale_dev is NULL");
+  return quantize_impl(src, src_dtype, dst, 0.f, scale_dev, n, device, stream);
+}
+
+extern "C" int sce_amax_scale(const void* src, int32_t src_dtype, size_t n, float* scale_out, int32_t device, void* stream) {
+  if (!src || !scale_out) return fail(SCE_EINVAL, "src/scale_out is NULL");
+  if (n == 0) return fail(SCE_EINVAL, "n must be positive");
+  if (src_dtype != SCE_F32 && src_dtype != SCE_BF16) return fail(SCE_EINVAL, "unsupported dtype %d", src_dtype);
+  if (int rc = check_device(device)) return rc;
+  DeviceGuard guard(device);
+  if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", device);
+  hipStream_t st = (hipStream_t)stream;
+  uint32_t* bits = reinterpret_cast<uint32_t*>(scale_out);
+  int grid = grid_for(n, 256 * 16);
+  if (grid > 4096) grid = 4096;
+  amax_begin_kernel<<<1, 1, 0, st>>>(bits);
+  if (src_dtype == SCE_F32) amax_kernel<float><<<grid, 256, 0, st>>>((const float*)src, n, bits);
+  else amax_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)src, n, bits);
+  amax_end_kernel<<<1, 1, 0, st>>>(bits);
   HIP_TRY(hipGetLastError());
   return SCE_OK;
 }
@@ -1811,7 +1917,7 @@ static int check_common(const sce_args* a) {
   if (int rc = check_shape(&a->shape)) return rc;
   if (!a->targets) return fail(SCE_EINVAL, "targets is NULL");
   if (!(a->cap > 0.f) || a->cap > 40.f) return fail(SCE_EINVAL, "cap = %g must be in (0, 40]", (double)a->cap);
-  if (!(a->x_s > 0.0) || !(a->w_s > 0.0)) return fail(SCE_EINVAL, "x_s and w_s must be positive");
+  if ((!a->x_s_dev && !(a->x_s > 0.0)) || (!a->w_s_dev && !(a->w_s > 0.0))) return fail(SCE_EINVAL, "x_s and w_s must be positive");
   if (a->reduction != SCE_REDUCE_NONE && a->reduction != SCE_REDUCE_MEAN) return fail(SCE_EINVAL, "bad reduction %d", a->reduction);
   if (!a->saved) return fail(SCE_EINVAL, "saved is NULL");
   if (((uintptr_t)a->saved & 255) || ((uintptr_t)a->workspace & 255) || ((uintptr_t)a->wcache & 255))
@@ -1848,27 +1954,33 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
   uint8_t* wq = wbase + S.rel_wq;
   uint8_t* gbase = sv + need_saved;       // dlogits, when the forward pass emits them
 
+  // a scale that lives on the device: its value and what follows from it go into the header of `saved`, for the
+  // kernels of this call and of the matching backward
+  const bool devsc = a->x_s_dev || a->w_s_dev;
+  DevConsts* dcp = devsc ? (DevConsts*)(sv + S.off_hdr + 32) : nullptr;
+  const float inv_xs = a->x_s_dev ? 0.f : (float)(1.0 / a->x_s), inv_ws = a->w_s_dev ? 0.f : (float)(1.0 / a->w_s);
   {
     KernelTimer tm(SCE_K_QUANT, st);
+    if (devsc) dev_consts_kernel<<<1, 1, 0, st>>>(a->x_s_dev, a->w_s_dev, (float)a->x_s, (float)a->w_s, a->cap, dcp);
     const int grid = grid_for((size_t)S.Np * (S.dp / 16), 256);
     float* rstd = (float*)(sv + S.off_rstd);
     const int ngrid = (int)((S.Np + 3) / 4);
     if (a->norm && a->x_dtype == SCE_F32)
-      rmsnorm_quantize_kernel<float><<<ngrid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, a->norm_eps, xq, S.Np, S.dp, S.ldx, (float)(1.0 / a->x_s), rstd);
+      rmsnorm_quantize_kernel<float><<<ngrid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, a->norm_eps, xq, S.Np, S.dp, S.ldx, inv_xs, a->x_s_dev, rstd);
     else if (a->norm && a->x_dtype == SCE_BF16)
-      rmsnorm_quantize_kernel<bf16_t><<<ngrid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, a->norm_eps, xq, S.Np, S.dp, S.ldx, (float)(1.0 / a->x_s), rstd);
+      rmsnorm_quantize_kernel<bf16_t><<<ngrid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, a->norm_eps, xq, S.Np, S.dp, S.ldx, inv_xs, a->x_s_dev, rstd);
     else if (a->x_dtype == SCE_F32)
-      quantize_pad_kernel<float><<<grid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, S.ldx, (float)(1.0 / a->x_s));
+      quantize_pad_kernel<float><<<grid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, S.ldx, inv_xs, a->x_s_dev);
     else if (a->x_dtype == SCE_BF16)
-      quantize_pad_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, S.ldx, (float)(1.0 / a->x_s));
+      quantize_pad_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, S.ldx, inv_xs, a->x_s_dev);
     else return fail(SCE_EINVAL, "unsupported x dtype %d", a->x_dtype);
     dim3 gw((unsigned)(S.Vp / 64), (unsigned)(S.dq / 64));
     if (a->wcache && a->wcache_valid) {
       // the caller vouches that the cache holds e4m3(W / w_s) of this W (unchanged since an earlier call)
     } else if (a->w_dtype == SCE_F32)
-      quantize_w_kernel<float><<<gw, 256, 0, st>>>((const float*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.Vp / BK, (float)(1.0 / a->w_s));
+      quantize_w_kernel<float><<<gw, 256, 0, st>>>((const float*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.Vp / BK, inv_ws, a->w_s_dev);
     else if (a->w_dtype == SCE_BF16)
-      quantize_w_kernel<bf16_t><<<gw, 256, 0, st>>>((const bf16_t*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.Vp / BK, (float)(1.0 / a->w_s));
+      quantize_w_kernel<bf16_t><<<gw, 256, 0, st>>>((const bf16_t*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.Vp / BK, inv_ws, a->w_s_dev);
     else return fail(SCE_EINVAL, "unsupported w dtype %d", a->w_dtype);
   }
   const bool emit = a->dlogits_from_forward != 0;
@@ -1882,6 +1994,7 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
   p.ghat_t = emit ? gbase + S.rel_g : nullptr; p.gexp = emit ? (uint32_t*)(gbase + S.rel_gexp) : nullptr; p.kbw = S.Np / BK;
   p.dp = S.dp; p.ldx = S.ldx; p.N = (int)N; p.V = (int)Vl; p.Np = (int)S.Np; p.RT = RT; p.CT = CTw; p.S = nsplit;
   p.sc = (float)a->x_s * (float)a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.c2 = -2.0f * a->cap * LOG2E; p.ic2 = 1.0f / p.c2;
+  p.dc = dcp;
   const int grid = 8 * nsplit * ((RT + 7) / 8);
   {
     // the exponent boosts of the rows, from the tile in the middle of the vocabulary (kept for backward in either mode)
@@ -1999,6 +2112,7 @@ extern "C" int sce_backward(const sce_args* a) {
   const float* s_lse = (const float*)(sv + S.off_lse);
   const float* s_zy = (const float*)(sv + S.off_zy);
   const int32_t* hdr = (const int32_t*)(sv + S.off_hdr);
+  const DevConsts* dcp = (a->x_s_dev || a->w_s_dev) ? (const DevConsts*)(sv + S.off_hdr + 32) : nullptr;     // as forward left it
   uint8_t* gkept = sv + need_saved;
   uint32_t* gexp = kept ? (uint32_t*)(gkept + S.rel_gexp) : (uint32_t*)(ws + B.off_gexp);
   float* rho = (float*)(ws + B.off_rho);
@@ -2053,7 +2167,7 @@ extern "C" int sce_backward(const sce_args* a) {
     if (!kept) {
       RecomputeParams rp;
       rp.xq = xq + p0 * S.ldx; rp.wqt = wqt; rp.ghat_t = ghat_t; rp.gexp = gexp; rp.rowinfo = rowinfo + p0; rp.Np = S.Np; rp.n_predict = K;
-      rp.dp = S.dp; rp.ldx = S.ldx; rp.kbw = gkb; rp.kb0 = (p0 - gorg) / BK; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2;
+      rp.dp = S.dp; rp.ldx = S.ldx; rp.kbw = gkb; rp.kb0 = (p0 - gorg) / BK; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2; rp.dc = dcp;
       {
         KernelTimer tm(SCE_K_RECOMPUTE, st);
         bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_RECOMPUTE, st>>>(rp);
@@ -2064,7 +2178,7 @@ extern "C" int sce_backward(const sce_args* a) {
     dp_.wq = wq; dp_.ghat_t = ghat_t + ((p0 - gorg) / BK) * BLOCKED_KSTEP; dp_.gexp = gexp + (p0 - gorg) / BK; dp_.kbw = gkb; dp_.wqt = wqt; dp_.rho = rho + p0; dp_.hcoef = hcoef + p0; dp_.targets = a->targets + p0;
     dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.ldx = S.ldx; dp_.Np = S.Np; dp_.dq = S.dq; dp_.RT = RTp; dp_.CT = CTd;
     dp_.n_predict = K; dp_.rows_left = (int)(N - p0 > 0 ? N - p0 : 0);
-    dp_.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); dp_.d = (int)d; dp_.V = (int)Vl; dp_.w_s = (float)a->w_s;
+    dp_.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); dp_.d = (int)d; dp_.V = (int)Vl; dp_.w_s = (float)a->w_s; dp_.dc = dcp;
     dp_.part = (float*)(ws + B.off_dxpart);
     // a panel with fewer than half as many tiles as there are CUs shares each tile's K loop among several workgroups
     const int tiles = RTp * CTd, kpairs = (int)(S.Vp / BK / 2);
@@ -2122,10 +2236,10 @@ extern "C" int sce_backward(const sce_args* a) {
   {
     dim3 g((unsigned)((V + 63) / 64), (unsigned)((d + 63) / 64));
     if (a->dw_dtype == SCE_F32)
-      bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, longbase, S.dq, (float)a->x_s, (int)d, (int)V,
+      bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, longbase, S.dq, (float)a->x_s, dcp, (int)d, (int)V,
                                                    (float*)a->dw, a->dw_ld);
     else
-      bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, longbase, S.dq, (float)a->x_s, (int)d, (int)V,
+      bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, longbase, S.dq, (float)a->x_s, dcp, (int)d, (int)V,
                                                     (bf16_t*)a->dw, a->dw_ld);
   }
   HIP_TRY(hipGetLastError());

@@ -46,11 +46,34 @@ _DTYPES = {torch.float32: _lib.SCE_F32, torch.bfloat16: _lib.SCE_BF16}
 
 
 def _scale_value(s, like):
-    """Python float, or a 0-dim tensor.  torch casts a 0-dim tensor operand to the
-    dtype of the tensor it divides, so the same rounding is applied here."""
+    """A scale as the C ABI takes it: a Python float, or -- for a one-element tensor on ``like``'s device -- that tensor
+    as float32, which the kernels read when they run (no host read, so the value may come from earlier work on the
+    stream, e.g. ``amax_scale``, and may change between replays of a captured graph).  A tensor on the CPU is read here."""
     if isinstance(s, torch.Tensor):
-        return float(s.detach().to(like.dtype))
+        if s.numel() != 1:
+            raise ValueError("a scale must have one element")
+        if s.device.type != "cuda":
+            return float(s)
+        return s.detach().to(dtype=torch.float32).reshape(())
     return float(s)
+
+
+def _split_scale(s):
+    """(float, None) for a host scale, (1.0, tensor) for a device scale: the two slots of the custom ops' signatures."""
+    return (1.0, s) if isinstance(s, torch.Tensor) else (s, None)
+
+
+def _set_scales(a, x_s, w_s):
+    """Fills x_s / w_s or x_s_dev / w_s_dev of an SceArgs; returns the tensors that must stay alive over the call."""
+    keep = []
+    for name, s in (("x_s", x_s), ("w_s", w_s)):
+        if isinstance(s, torch.Tensor):
+            setattr(a, name, 1.0)
+            setattr(a, name + "_dev", s.data_ptr())
+            keep.append(s)
+        else:
+            setattr(a, name, s)
+    return keep
 
 
 def _dtype_code(t, what):
@@ -82,7 +105,8 @@ def _base_args(x_like, N, d, V, x_s, w_s, cap, grad_scale, reduction, targets, n
     a.shape = SceShape(N, d, V, n_predict, 0)
     a.targets = targets.data_ptr()
     a.mtp_weights = mtp_w.data_ptr() if mtp_w is not None else None
-    a.x_s, a.w_s, a.cap, a.grad_scale = x_s, w_s, cap, grad_scale
+    a._scale_refs = _set_scales(a, x_s, w_s)
+    a.cap, a.grad_scale = cap, grad_scale
     a.ignore_index = IGNORE_INDEX
     a.reduction = _lib.SCE_REDUCE_MEAN if reduction == "mean" else _lib.SCE_REDUCE_NONE
     return a
@@ -122,7 +146,8 @@ class WeightCache:
 
     def prepare(self, w, w_s, nbytes):
         """Returns (buffer, valid)."""
-        key = (w.data_ptr(), w._version, tuple(w.shape), w.dtype, float(w_s), w.device)
+        skey = (w_s.data_ptr(), w_s._version) if isinstance(w_s, torch.Tensor) else float(w_s)
+        key = (w.data_ptr(), w._version, tuple(w.shape), w.dtype, skey, w.device)
         if self.buf is None or self.buf.numel() < nbytes or self.buf.device != w.device:
             self.buf = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
             self.key = None
@@ -238,14 +263,15 @@ def ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale,
 # ---------------------------------------------------------------------------------------------
 @torch.library.custom_op("slowrun_amd::ce_forward", mutates_args=())
 def ce_forward_op(x: torch.Tensor, w: torch.Tensor, targets: torch.Tensor, mtp_weights: Optional[torch.Tensor],
-                  x_s: float, w_s: float, cap: float, mean: bool, keep: bool) -> Tuple[torch.Tensor, torch.Tensor]:
-    out, saved, _lse, _am, _nv = ce_forward(x, w, targets, x_s, w_s, cap, "mean" if mean else "none", mtp_weights=mtp_weights,
-                                            keep_dlogits=keep)
+                  x_s: float, w_s: float, cap: float, mean: bool, keep: bool,
+                  x_s_t: Optional[torch.Tensor] = None, w_s_t: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    out, saved, _lse, _am, _nv = ce_forward(x, w, targets, x_s if x_s_t is None else x_s_t, w_s if w_s_t is None else w_s_t, cap,
+                                            "mean" if mean else "none", mtp_weights=mtp_weights, keep_dlogits=keep)
     return out, saved
 
 
 @ce_forward_op.register_fake
-def _ce_forward_fake(x, w, targets, mtp_weights, x_s, w_s, cap, mean, keep):
+def _ce_forward_fake(x, w, targets, mtp_weights, x_s, w_s, cap, mean, keep, x_s_t=None, w_s_t=None):
     N, d = x.shape
     V = w.shape[1]
     n_predict = 1 if mtp_weights is None else mtp_weights.numel()
@@ -257,42 +283,49 @@ def _ce_forward_fake(x, w, targets, mtp_weights, x_s, w_s, cap, mean, keep):
 @torch.library.custom_op("slowrun_amd::ce_backward", mutates_args=())
 def ce_backward_op(saved: torch.Tensor, targets: torch.Tensor, grad_output: torch.Tensor, mtp_weights: Optional[torch.Tensor],
                    N: int, d: int, V: int, x_s: float, w_s: float, cap: float, grad_scale: float, mean: bool,
-                   x_bf16: bool, w_bf16: bool, keep: bool) -> Tuple[torch.Tensor, torch.Tensor]:
-    return ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale, "mean" if mean else "none",
+                   x_bf16: bool, w_bf16: bool, keep: bool,
+                   x_s_t: Optional[torch.Tensor] = None, w_s_t: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    return ce_backward(saved, targets, grad_output, N, d, V, x_s if x_s_t is None else x_s_t, w_s if w_s_t is None else w_s_t, cap,
+                       grad_scale, "mean" if mean else "none",
                        torch.bfloat16 if x_bf16 else torch.float32, torch.bfloat16 if w_bf16 else torch.float32,
                        mtp_weights=mtp_weights, keep_dlogits=keep)
 
 
 @ce_backward_op.register_fake
-def _ce_backward_fake(saved, targets, grad_output, mtp_weights, N, d, V, x_s, w_s, cap, grad_scale, mean, x_bf16, w_bf16, keep):
+def _ce_backward_fake(saved, targets, grad_output, mtp_weights, N, d, V, x_s, w_s, cap, grad_scale, mean, x_bf16, w_bf16, keep,
+                      x_s_t=None, w_s_t=None):
     return (saved.new_empty((N, d), dtype=torch.bfloat16 if x_bf16 else torch.float32),
             saved.new_empty((d, V), dtype=torch.bfloat16 if w_bf16 else torch.float32))
 
 
 @torch.library.custom_op("slowrun_amd::norm_ce_forward", mutates_args=())
 def norm_ce_forward_op(h: torch.Tensor, w: torch.Tensor, targets: torch.Tensor, mtp_weights: Optional[torch.Tensor],
-                       x_s: float, w_s: float, cap: float, mean: bool, eps: float, keep: bool) -> Tuple[torch.Tensor, torch.Tensor]:
-    out, saved, _lse, _am, _nv = ce_forward(h, w, targets, x_s, w_s, cap, "mean" if mean else "none", mtp_weights=mtp_weights,
-                                            norm_eps=eps, keep_dlogits=keep)
+                       x_s: float, w_s: float, cap: float, mean: bool, eps: float, keep: bool,
+                       x_s_t: Optional[torch.Tensor] = None, w_s_t: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    out, saved, _lse, _am, _nv = ce_forward(h, w, targets, x_s if x_s_t is None else x_s_t, w_s if w_s_t is None else w_s_t, cap,
+                                            "mean" if mean else "none", mtp_weights=mtp_weights, norm_eps=eps, keep_dlogits=keep)
     return out, saved
 
 
-norm_ce_forward_op.register_fake(lambda h, w, targets, mtp_weights, x_s, w_s, cap, mean, eps, keep:
+norm_ce_forward_op.register_fake(lambda h, w, targets, mtp_weights, x_s, w_s, cap, mean, eps, keep, x_s_t=None, w_s_t=None:
                                  _ce_forward_fake(h, w, targets, mtp_weights, x_s, w_s, cap, mean, keep))
 
 
 @torch.library.custom_op("slowrun_amd::norm_ce_backward", mutates_args=())
 def norm_ce_backward_op(saved: torch.Tensor, h: torch.Tensor, targets: torch.Tensor, grad_output: torch.Tensor,
                         mtp_weights: Optional[torch.Tensor], V: int, x_s: float, w_s: float, cap: float, grad_scale: float,
-                        mean: bool, w_bf16: bool, eps: float, keep: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+                        mean: bool, w_bf16: bool, eps: float, keep: bool,
+                        x_s_t: Optional[torch.Tensor] = None, w_s_t: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     N, d = h.shape
-    return ce_backward(saved, targets, grad_output, N, d, V, x_s, w_s, cap, grad_scale, "mean" if mean else "none",
+    return ce_backward(saved, targets, grad_output, N, d, V, x_s if x_s_t is None else x_s_t, w_s if w_s_t is None else w_s_t, cap,
+                       grad_scale, "mean" if mean else "none",
                        h.dtype, torch.bfloat16 if w_bf16 else torch.float32, mtp_weights=mtp_weights, hidden=h, norm_eps=eps,
                        keep_dlogits=keep)
 
 
 @norm_ce_backward_op.register_fake
-def _norm_ce_backward_fake(saved, h, targets, grad_output, mtp_weights, V, x_s, w_s, cap, grad_scale, mean, w_bf16, eps, keep):
+def _norm_ce_backward_fake(saved, h, targets, grad_output, mtp_weights, V, x_s, w_s, cap, grad_scale, mean, w_bf16, eps, keep,
+                           x_s_t=None, w_s_t=None):
     return torch.empty_like(h), h.new_empty((h.shape[1], V), dtype=torch.bfloat16 if w_bf16 else torch.float32)
 
 
@@ -307,9 +340,11 @@ class FusedSoftcappedCrossEntropy(torch.autograd.Function):
         _dtype_code(x, "x")
         _dtype_code(lm_head_weight, "lm_head_weight")
         xs, ws_ = _scale_value(x_s, x), _scale_value(w_s, lm_head_weight)
+        (xs, xst), (ws_, wst) = _split_scale(xs), _split_scale(ws_)
         keep = bool(KEEP_DLOGITS if keep_dlogits is None else keep_dlogits)
         out, saved = ce_forward_op(x.detach(), lm_head_weight.detach(), targets, mtp_weights, xs, ws_, float(cap),
-                                   reduction == "mean", keep)
+                                   reduction == "mean", keep, xst, wst)
+        ctx.scale_tensors = (xst, wst)
         ctx.save_for_backward(saved, targets, mtp_weights if mtp_weights is not None else torch.empty(0, device=x.device))
         ctx.params = (x.shape[0], x.shape[1], lm_head_weight.shape[1], xs, ws_, float(cap), float(grad_scale),
                       reduction == "mean", x.dtype == torch.bfloat16, lm_head_weight.dtype == torch.bfloat16,
@@ -321,7 +356,7 @@ class FusedSoftcappedCrossEntropy(torch.autograd.Function):
         saved, targets, mtp_w = ctx.saved_tensors
         N, d, V, xs, ws_, cap, gscale, mean, x_bf16, w_bf16, has_mtp, keep = ctx.params
         dx, dw = ce_backward_op(saved, targets, grad_output.contiguous(), mtp_w if has_mtp else None, N, d, V, xs, ws_, cap,
-                                gscale, mean, x_bf16, w_bf16, keep)
+                                gscale, mean, x_bf16, w_bf16, keep, *ctx.scale_tensors)
         return dx, None, None, dw, None, None, None, None, None, None, None
 
 
@@ -340,10 +375,12 @@ class FusedNormSoftcappedCrossEntropy(torch.autograd.Function):
         _dtype_code(lm_head_weight, "lm_head_weight")
         eps = float(torch.finfo(torch.float32).eps if eps is None else eps)
         xs, ws_ = _scale_value(x_s, h), _scale_value(w_s, lm_head_weight)
+        (xs, xst), (ws_, wst) = _split_scale(xs), _split_scale(ws_)
         hd = h.detach()
         keep = bool(KEEP_DLOGITS if keep_dlogits is None else keep_dlogits)
         out, saved = norm_ce_forward_op(hd, lm_head_weight.detach(), targets, mtp_weights, xs, ws_, float(cap),
-                                        reduction == "mean", eps, keep)
+                                        reduction == "mean", eps, keep, xst, wst)
+        ctx.scale_tensors = (xst, wst)
         ctx.save_for_backward(saved, hd, targets, mtp_weights if mtp_weights is not None else torch.empty(0, device=h.device))
         ctx.params = (lm_head_weight.shape[1], xs, ws_, float(cap), float(grad_scale), reduction == "mean",
                       lm_head_weight.dtype == torch.bfloat16, mtp_weights is not None, eps, keep)
@@ -354,7 +391,7 @@ class FusedNormSoftcappedCrossEntropy(torch.autograd.Function):
         saved, h, targets, mtp_w = ctx.saved_tensors
         V, xs, ws_, cap, gscale, mean, w_bf16, has_mtp, eps, keep = ctx.params
         dh, dw = norm_ce_backward_op(saved, h, targets, grad_output.contiguous(), mtp_w if has_mtp else None, V, xs, ws_, cap,
-                                     gscale, mean, w_bf16, eps, keep)
+                                     gscale, mean, w_bf16, eps, keep, *ctx.scale_tensors)
         return dh, None, None, dw, None, None, None, None, None, None, None, None
 
 
@@ -379,9 +416,26 @@ def quantize_e4m3(t, scale):
         raise RuntimeError("quantize_e4m3 needs a GPU tensor")
     t = t.contiguous()
     out = torch.empty(t.shape, dtype=torch.uint8, device=t.device)
-    _lib.check(_lib.lib().sce_quantize_e4m3(t.data_ptr(), _dtype_code(t, "t"), out.data_ptr(), _scale_value(scale, t),
-                                           t.numel(), t.device.index, _stream_ptr(t.device)), "sce_quantize_e4m3")
+    sv = _scale_value(scale, t)
+    if isinstance(sv, torch.Tensor):            # a device scalar: divided by, as torch divides by a tensor
+        _lib.check(_lib.lib().sce_quantize_e4m3_dev(t.data_ptr(), _dtype_code(t, "t"), out.data_ptr(), sv.data_ptr(), t.numel(),
+                                                   t.device.index, _stream_ptr(t.device)), "sce_quantize_e4m3_dev")
+    else:
+        _lib.check(_lib.lib().sce_quantize_e4m3(t.data_ptr(), _dtype_code(t, "t"), out.data_ptr(), sv, t.numel(), t.device.index,
+                                               _stream_ptr(t.device)), "sce_quantize_e4m3")
     return out.view(torch.float8_e4m3fn)
+
+
+def amax_scale(t):
+    """``t.abs().max() / 448`` as a 0-dim float32 tensor on ``t``'s device, without a host read: the per-tensor scale of
+    the e4m3 cast, to be passed as ``x_s`` / ``w_s``."""
+    if not t.is_cuda:
+        raise RuntimeError("amax_scale needs a GPU tensor")
+    t = t.contiguous()
+    out = torch.empty((), dtype=torch.float32, device=t.device)
+    _lib.check(_lib.lib().sce_amax_scale(t.data_ptr(), _dtype_code(t, "t"), t.numel(), out.data_ptr(), t.device.index,
+                                        _stream_ptr(t.device)), "sce_amax_scale")
+    return out
 
 
 def transpose_copy(src, dst):
