@@ -62,6 +62,7 @@ typedef struct sce_sizes {
   /* with sce_args.dlogits_from_forward: */
   size_t dlogits_bytes;             /* `saved` grows by this much (N x V bytes and a little)  */
   size_t bwd_workspace_kept_bytes;  /* and backward needs this workspace, no more             */
+  size_t saved_bf16_bytes;          /* `saved` of a forward with operand_dtype = SCE_BF16     */
 } sce_sizes;
 
 typedef struct sce_args {
@@ -126,6 +127,12 @@ typedef struct sce_args {
                                 The quantiser then divides (x / s) as torch does for a tensor divisor.  Same in forward
                                 and backward (backward reads the value forward used from `saved`)                       */
   const float* w_s_dev;      /* the same for W                                                                           */
+  int32_t operand_dtype;     /* 0: X and W go into the GEMM as e4m3 (the training path); SCE_BF16: as bf16, the logits
+                                rounded to bf16 before the softcap -- the arithmetic of the eager head under bf16
+                                autocast (tiny/train.py:741-743 with CastedLinearT :496-497), for validation losses that
+                                compare with the reference's.  Forward only (sce_backward refuses it); x_s, w_s are not
+                                used; `saved` is then plain scratch of saved_bf16_bytes                              */
+  int32_t pad6;
 } sce_args;
 
 /* Library / ABI version (SCE_VERSION of the build). */

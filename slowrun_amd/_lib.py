@@ -28,7 +28,7 @@ class SceSizes(C.Structure):
     _fields_ = [("saved_bytes", C.c_size_t), ("saved_x_bytes", C.c_size_t), ("wcache_bytes", C.c_size_t),
                 ("fwd_workspace_bytes", C.c_size_t),
                 ("bwd_workspace_min_bytes", C.c_size_t), ("bwd_workspace_bytes", C.c_size_t),
-                ("bwd_panel_rows", C.c_int64), ("dlogits_bytes", C.c_size_t), ("bwd_workspace_kept_bytes", C.c_size_t)]
+                ("bwd_panel_rows", C.c_int64), ("dlogits_bytes", C.c_size_t), ("bwd_workspace_kept_bytes", C.c_size_t), ("saved_bf16_bytes", C.c_size_t)]
 
 
 class SceArgs(C.Structure):
@@ -47,7 +47,7 @@ class SceArgs(C.Structure):
         ("panel_rows", C.c_int64),
         ("vocab_limit", C.c_int64), ("wcache", C.c_void_p), ("wcache_bytes", C.c_size_t),
         ("wcache_valid", C.c_int32), ("norm", C.c_int32), ("norm_eps", C.c_float), ("dlogits_from_forward", C.c_int32),
-        ("x_s_dev", C.c_void_p), ("w_s_dev", C.c_void_p),
+        ("x_s_dev", C.c_void_p), ("w_s_dev", C.c_void_p), ("operand_dtype", C.c_int32), ("pad6", C.c_int32),
     ]
 
 

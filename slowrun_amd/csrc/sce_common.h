@@ -47,7 +47,7 @@ static inline int64_t row_stride(int64_t k) { return k + 128; }
 // (same relative offsets) and `saved` ends at x_total.
 struct SavedLayout {
   int64_t ldx;                       // row stride in bytes of the [..][dp] e4m3 arrays
-  int64_t N, d, V, Np, dp, dq, Vp;   // all padded sizes are multiples of 256 (every K loop runs over an even number of 128-byte blocks); dp = dq
+  int64_t N, d, V, Np, dp, dq, Vp;   // all padded sizes are multiples of 256 (every K loop runs over an even number of 128-byte blocks); dp: row bytes of X_q / W_q^T (= dq for e4m3)
   size_t off_hdr, off_xq, off_lse, off_umax, off_zy, off_rstd, off_lam, x_total;
   size_t rel_wqt, rel_wq, w_total;   // relative to the start of the W region
   size_t total;                      // x_total + w_total
@@ -55,10 +55,11 @@ struct SavedLayout {
 };
 // hdr: int32 n_valid, int32 n_bad_targets, float mean loss, float pad
 
-static inline SavedLayout saved_layout(int64_t N, int64_t d, int64_t V, int n_predict) {
+// eb: bytes per operand element, 1 (e4m3) or 2 (bf16 operands: forward only, so no second copy of W)
+static inline SavedLayout saved_layout(int64_t N, int64_t d, int64_t V, int n_predict, int eb = 1) {
   SavedLayout L;
   L.N = N; L.d = d; L.V = V;
-  L.Np = round_up(N, 256); L.dp = round_up(d, 256); L.dq = round_up(d, 256); L.Vp = round_up(V, 256);
+  L.Np = round_up(N, 256); L.dp = round_up(d * eb, 256); L.dq = round_up(d, 256); L.Vp = round_up(V, 256);
   L.ldx = row_stride(L.dp);
   size_t o = 0;
   auto take = [&](size_t bytes) { size_t r = o; o += (bytes + 255) / 256 * 256; return r; };
@@ -72,7 +73,7 @@ static inline SavedLayout saved_layout(int64_t N, int64_t d, int64_t V, int n_pr
   L.x_total = o;
   o = 0;
   L.rel_wqt = take((size_t)L.Vp * L.ldx);      // W_q^T [Vp][dp], row stride ldx
-  L.rel_wq = take((size_t)L.dq * L.Vp);        // W_q: dq rows, K = Vp, tile by tile (256 rows x 128 B per K block)
+  L.rel_wq = take(eb == 1 ? (size_t)L.dq * L.Vp : 0);        // W_q: dq rows, K = Vp, tile by tile (256 rows x 128 B per K block)
   L.w_total = o;
   L.total = L.x_total + L.w_total;
   o = 0;

@@ -370,6 +370,45 @@ __global__ __launch_bounds__(256) void quantize_w_kernel(const T* __restrict__ w
   }
 }
 
+// bf16 operands (the eval head, tiny/train.py:741 under bf16 autocast): no quantisation, only the layout.
+// dst [rows_p][cols_p] bf16 = src [rows][cols] rounded to bf16 (RNE, as autocast's cast), zero outside; 8 outputs per thread.
+template <typename T>
+__global__ __launch_bounds__(256) void prep_x_bf16_kernel(const T* __restrict__ src, int64_t ld, int64_t rows, int64_t cols,
+                                                         uint16_t* __restrict__ dst, int64_t rows_p, int64_t cols_p, int64_t dst_ld) {
+  const int64_t chunks_per_row = cols_p / 8;
+  const int64_t total = rows_p * chunks_per_row;
+  for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < total; q += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = q / chunks_per_row, c0 = (q - r * chunks_per_row) * 8;
+    uint32_t out[4] = {0, 0, 0, 0};
+    if (r < rows) {
+#pragma unroll
+      for (int m = 0; m < 8; ++m) {
+        const uint32_t h = (c0 + m < cols) ? float_to_bf16_bits(Elem<T>::load(src + r * ld + c0 + m)) : 0u;
+        out[m >> 1] |= h << (16 * (m & 1));
+      }
+    }
+    *reinterpret_cast<v4i*>(dst + r * dst_ld + c0) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
+  }
+}
+
+// W (d, V) -> W^T [Vp][dp2 / 2] in bf16 (row stride ldw elements); 64 x 64 tiles through LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void prep_w_bf16_kernel(const T* __restrict__ w, int64_t ld, int64_t d, int64_t V,
+                                                         uint16_t* __restrict__ wt, int64_t ldw) {
+  __shared__ uint16_t tile[64][66];
+  const int t = threadIdx.x;
+  const int64_t j0 = (int64_t)blockIdx.y * 64, v0 = (int64_t)blockIdx.x * 64;
+  for (int e = t; e < 64 * 64; e += 256) {
+    const int r = e >> 6, c = e & 63;
+    tile[r][c] = (j0 + r < d && v0 + c < V) ? float_to_bf16_bits(Elem<T>::load(w + (j0 + r) * ld + v0 + c)) : (uint16_t)0;
+  }
+  __syncthreads();
+  for (int e = t; e < 64 * 64; e += 256) {
+    const int vr = e >> 6, jc = e & 63;
+    wt[(v0 + vr) * ldw + j0 + jc] = tile[jc][vr];
+  }
+}
+
 // flat cast, for the standalone sce_quantize_e4m3 entry point
 template <typename T>
 __global__ __launch_bounds__(256) void quantize_flat_kernel(const T* __restrict__ src, uint8_t* __restrict__ dst,
@@ -604,7 +643,8 @@ struct FwdParams {
 //   t = tanh(u/cap) = 1 - 2/(E + 1), E = e^{2u/cap};   e^{z - cap} = exp2(c2 / (E + 1)).
 // The column of the maximum is looked up only on the (rare, after the first tiles) occasion that
 // a tile raises a row's running maximum.
-template <bool EDGE>
+// ROUND: the logits are rounded to bf16 first (bf16 operands: the GEMM of the eager head returns bf16).
+template <bool EDGE, bool ROUND = false>
 __device__ __forceinline__ void fwd_epilogue(const v16f (&acc)[4][4], const FwdParams& p, int vbase,
                                              float (&sum)[4], float (&amax)[4], int (&uarg)[4]) {
 #pragma unroll
@@ -615,7 +655,7 @@ __device__ __forceinline__ void fwd_epilogue(const v16f (&acc)[4][4], const FwdP
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int vo = a * 32 + 8 * (r >> 2) + (r & 3);
-        float x = acc[a][b][r];
+        float x = ROUND ? round_to_bf16(acc[a][b][r]) : acc[a][b][r];
         // z - cap = c2 / (1 + e^{2u/cap}) in units of log2: the reciprocal of (1 + e) / c2 gives it in one step
         float pt = fast_exp2(fast_rcp(fmaf(fast_exp2(x * p.k1), p.ic2, p.ic2)));
         if (EDGE) {
@@ -634,7 +674,7 @@ __device__ __forceinline__ void fwd_epilogue(const v16f (&acc)[4][4], const FwdP
 #pragma unroll
           for (int r = 15; r >= 0; --r) {
             const int vo = a * 32 + 8 * (r >> 2) + (r & 3);
-            if (acc[a][b][r] == tmax && (!EDGE || vo < p.V - vbase)) targ = vo;   // descending scan: lowest column wins
+            if ((ROUND ? round_to_bf16(acc[a][b][r]) : acc[a][b][r]) == tmax && (!EDGE || vo < p.V - vbase)) targ = vo;   // descending scan: lowest column wins
           }
         }
         amax[b] = tmax;
@@ -663,7 +703,7 @@ __device__ __forceinline__ bool target_valid(const int64_t* __restrict__ targets
 //        neighbours', out of the 8 bits.
 // STATS: with KNOCK, the row statistics (stat, as in form_dlogits) take the target's share here: e^{z_y - cap} into the
 //        sum, and the running maximum / argmax.
-template <bool STORE, bool KNOCK, bool STATS, int TGT_STRIDE>
+template <bool STORE, bool KNOCK, bool STATS, int TGT_STRIDE, bool ROUND = false>
 __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int* tgt, int n_predict, int col0, int rowbase,
                                                    float sc, float* s_uy_tile, int Np, float* stat, float k1, float ic2) {
   const int lane = lane_id(), half = lane >> 5;
@@ -704,7 +744,7 @@ __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int*
           }
           xk[k] = x;
           // (the lane index is taken anew: an address kept from outside the branch stays live across the main loop and is spilled)
-          if (STORE) s_uy_tile[(int64_t)k * Np + rowbase + b * 32 + (lane_id() & 31)] = x * sc;
+          if (STORE) s_uy_tile[(int64_t)k * Np + rowbase + b * 32 + (lane_id() & 31)] = ROUND ? round_to_bf16(x) * sc : x * sc;
         }
       }
     }
@@ -771,7 +811,8 @@ static_assert(FWD_STAGE_OFF + STG_BYTES <= FWD_STAT_OFF, "staging tile and row s
 
 // EMIT: the epilogue also leaves the block-scaled dlogits of the tile in G^T (see form_dlogits), for a backward pass
 // that does not compute the logits again.
-template <bool EMIT>
+// BF16 (without EMIT): bf16 operands, logits rounded to bf16 as the eager head's GEMM returns them (forward only).
+template <bool EMIT, bool BF16 = false>
 __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   FwdParams p = p_in;
@@ -805,8 +846,8 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
   // with EMIT it uses the second one, so only the first block travels and the rest follows after the epilogue)
   if (ct0 < ct1) mfma_prefetch(p.wqt + (int64_t)ct0 * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
   for (int ct = ct0; ct < ct1; ++ct) {
-    mfma_mainloop<true>(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, Bg, p.ldx, KT, smem, acc, rot_a, rot_b, wave, NoHook(), 0, 0, nullptr,
-                        EMIT && ct > ct0);
+    mfma_mainloop<true, NoHook, BK, false, 0, BF16>(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, Bg, p.ldx, KT, smem, acc, rot_a, rot_b, wave,
+                                                    NoHook(), 0, 0, nullptr, EMIT && ct > ct0);
     const uint8_t* Anext = p.wqt + (int64_t)(ct + 1) * 256 * p.ldx;
     if (ct + 1 < ct1) mfma_prefetch<EMIT ? 1 : 3>(Anext, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
     float* stat = reinterpret_cast<float*>(smem + FWD_STAT_OFF) + wave * 64 + lane_id();
@@ -829,14 +870,14 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
       for (int b = 0; b < 4; ++b) {
         sum[b] = stat[(0 + b) * NTHREADS]; amax[b] = stat[(4 + b) * NTHREADS]; uarg[b] = __float_as_int(stat[(8 + b) * NTHREADS]);
       }
-      if (ct * 256 + 256 > p.V) fwd_epilogue<true>(acc, p, vbase, sum, amax, uarg);
-      else fwd_epilogue<false>(acc, p, vbase, sum, amax, uarg);
+      if (ct * 256 + 256 > p.V) fwd_epilogue<true, BF16>(acc, p, vbase, sum, amax, uarg);
+      else fwd_epilogue<false, BF16>(acc, p, vbase, sum, amax, uarg);
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         stat[(0 + b) * NTHREADS] = sum[b]; stat[(4 + b) * NTHREADS] = amax[b]; stat[(8 + b) * NTHREADS] = __int_as_float(uarg[b]);
       }
     }
-    if (!EMIT) take_target_logits<true, false, false, 256>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, nullptr, 0.f, 0.f);
+    if (!EMIT) take_target_logits<true, false, false, 256, BF16>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, nullptr, 0.f, 0.f);
     if (EMIT && ct + 1 < ct1) {
       // every wave has read its part of the staging tile (its stores have their data) before the second K slot fills again
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -1679,6 +1720,7 @@ static int check_device(int dev) {
       // the MFMA kernels hold two 64 KB K-slots in LDS, and more behind them
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
+      HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_sample_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_recompute_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_RECOMPUTE));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
@@ -1841,6 +1883,7 @@ extern "C" int sce_sizes_for(const sce_shape* shape, sce_sizes* out) {
     out->dlogits_bytes = S.g_total;
     out->bwd_workspace_kept_bytes = bwd_layout(S, out->bwd_panel_rows, Pw, dw_launches(S, Pw), shape->n_predict, true).total;
   }
+  out->saved_bf16_bytes = saved_layout(shape->N, shape->d, shape->V, shape->n_predict, 2).total;
   return SCE_OK;
 }
 
@@ -1917,7 +1960,8 @@ static int check_common(const sce_args* a) {
   if (int rc = check_shape(&a->shape)) return rc;
   if (!a->targets) return fail(SCE_EINVAL, "targets is NULL");
   if (!(a->cap > 0.f) || a->cap > 40.f) return fail(SCE_EINVAL, "cap = %g must be in (0, 40]", (double)a->cap);
-  if ((!a->x_s_dev && !(a->x_s > 0.0)) || (!a->w_s_dev && !(a->w_s > 0.0))) return fail(SCE_EINVAL, "x_s and w_s must be positive");
+  if (a->operand_dtype == 0 && ((!a->x_s_dev && !(a->x_s > 0.0)) || (!a->w_s_dev && !(a->w_s > 0.0))))
+    return fail(SCE_EINVAL, "x_s and w_s must be positive");
   if (a->reduction != SCE_REDUCE_NONE && a->reduction != SCE_REDUCE_MEAN) return fail(SCE_EINVAL, "bad reduction %d", a->reduction);
   if (!a->saved) return fail(SCE_EINVAL, "saved is NULL");
   if (((uintptr_t)a->saved & 255) || ((uintptr_t)a->workspace & 255) || ((uintptr_t)a->wcache & 255))
@@ -1935,7 +1979,11 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
   if (a->reduction == SCE_REDUCE_MEAN && !a->loss) return fail(SCE_EINVAL, "loss is NULL with reduction = mean");
   if (a->reduction == SCE_REDUCE_MEAN && a->shape.n_predict != 1)
     return fail(SCE_EINVAL, "reduction = mean is defined for a single offset only; use reduction = none with n_predict > 1");
-  const SavedLayout S = saved_layout(N, d, V, a->shape.n_predict);
+  const bool bf16ops = a->operand_dtype == SCE_BF16;
+  if (a->operand_dtype != 0 && !bf16ops) return fail(SCE_EINVAL, "operand_dtype %d: 0 (e4m3) or SCE_BF16", a->operand_dtype);
+  if (bf16ops && (a->dlogits_from_forward || a->norm || a->wcache))
+    return fail(SCE_EINVAL, "bf16 operands are for the forward-only eval head: no kept dlogits, fused norm or weight cache");
+  const SavedLayout S = saved_layout(N, d, V, a->shape.n_predict, bf16ops ? 2 : 1);
   const size_t need_saved = a->wcache ? S.x_total : S.total;
   if (a->saved_bytes < need_saved) return fail(SCE_EINVAL, "saved buffer too small: %zu < %zu", a->saved_bytes, need_saved);
   if (a->wcache && a->wcache_bytes < S.w_total) return fail(SCE_EINVAL, "weight cache too small: %zu < %zu", a->wcache_bytes, S.w_total);
@@ -1961,11 +2009,23 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
   const float inv_xs = a->x_s_dev ? 0.f : (float)(1.0 / a->x_s), inv_ws = a->w_s_dev ? 0.f : (float)(1.0 / a->w_s);
   {
     KernelTimer tm(SCE_K_QUANT, st);
-    if (devsc) dev_consts_kernel<<<1, 1, 0, st>>>(a->x_s_dev, a->w_s_dev, (float)a->x_s, (float)a->w_s, a->cap, dcp);
+    if (bf16ops) {
+      const int grid = grid_for((size_t)S.Np * (S.dp / 16), 256);
+      if (a->x_dtype == SCE_F32) prep_x_bf16_kernel<float><<<grid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, (uint16_t*)xq, S.Np, S.dp / 2, S.ldx / 2);
+      else if (a->x_dtype == SCE_BF16) prep_x_bf16_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, (uint16_t*)xq, S.Np, S.dp / 2, S.ldx / 2);
+      else return fail(SCE_EINVAL, "unsupported x dtype %d", a->x_dtype);
+      dim3 gw((unsigned)(S.Vp / 64), (unsigned)(S.dp / 2 / 64));
+      if (a->w_dtype == SCE_F32) prep_w_bf16_kernel<float><<<gw, 256, 0, st>>>((const float*)a->w, a->w_ld, d, V, (uint16_t*)wqt, S.ldx / 2);
+      else if (a->w_dtype == SCE_BF16) prep_w_bf16_kernel<bf16_t><<<gw, 256, 0, st>>>((const bf16_t*)a->w, a->w_ld, d, V, (uint16_t*)wqt, S.ldx / 2);
+      else return fail(SCE_EINVAL, "unsupported w dtype %d", a->w_dtype);
+    }
+    if (devsc && !bf16ops) dev_consts_kernel<<<1, 1, 0, st>>>(a->x_s_dev, a->w_s_dev, (float)a->x_s, (float)a->w_s, a->cap, dcp);
     const int grid = grid_for((size_t)S.Np * (S.dp / 16), 256);
     float* rstd = (float*)(sv + S.off_rstd);
     const int ngrid = (int)((S.Np + 3) / 4);
-    if (a->norm && a->x_dtype == SCE_F32)
+    if (bf16ops) {
+      // operands laid out above
+    } else if (a->norm && a->x_dtype == SCE_F32)
       rmsnorm_quantize_kernel<float><<<ngrid, 256, 0, st>>>((const float*)a->x, a->x_ld, N, d, a->norm_eps, xq, S.Np, S.dp, S.ldx, inv_xs, a->x_s_dev, rstd);
     else if (a->norm && a->x_dtype == SCE_BF16)
       rmsnorm_quantize_kernel<bf16_t><<<ngrid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, a->norm_eps, xq, S.Np, S.dp, S.ldx, inv_xs, a->x_s_dev, rstd);
@@ -1975,7 +2035,8 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
       quantize_pad_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, S.ldx, inv_xs, a->x_s_dev);
     else return fail(SCE_EINVAL, "unsupported x dtype %d", a->x_dtype);
     dim3 gw((unsigned)(S.Vp / 64), (unsigned)(S.dq / 64));
-    if (a->wcache && a->wcache_valid) {
+    if (bf16ops) {
+    } else if (a->wcache && a->wcache_valid) {
       // the caller vouches that the cache holds e4m3(W / w_s) of this W (unchanged since an earlier call)
     } else if (a->w_dtype == SCE_F32)
       quantize_w_kernel<float><<<gw, 256, 0, st>>>((const float*)a->w, a->w_ld, d, V, wq, wqt, S.dp, S.ldx, S.Vp / BK, inv_ws, a->w_s_dev);
@@ -1993,19 +2054,20 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
   p.targets = a->targets; p.ignore_index = a->ignore_index; p.n_predict = a->shape.n_predict; p.s_uy = (float*)(sv + S.off_zy);
   p.ghat_t = emit ? gbase + S.rel_g : nullptr; p.gexp = emit ? (uint32_t*)(gbase + S.rel_gexp) : nullptr; p.kbw = S.Np / BK;
   p.dp = S.dp; p.ldx = S.ldx; p.N = (int)N; p.V = (int)Vl; p.Np = (int)S.Np; p.RT = RT; p.CT = CTw; p.S = nsplit;
-  p.sc = (float)a->x_s * (float)a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.c2 = -2.0f * a->cap * LOG2E; p.ic2 = 1.0f / p.c2;
-  p.dc = dcp;
+  p.sc = bf16ops ? 1.0f : (float)a->x_s * (float)a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.c2 = -2.0f * a->cap * LOG2E; p.ic2 = 1.0f / p.c2;
+  p.dc = bf16ops ? nullptr : dcp;
   const int grid = 8 * nsplit * ((RT + 7) / 8);
   {
     // the exponent boosts of the rows, from the tile in the middle of the vocabulary (kept for backward in either mode)
     KernelTimer tm(SCE_K_QUANT, st);
     float* lam = (float*)(sv + S.off_lam);
     p.lam = lam;
-    fwd_sample_kernel<<<RT, NTHREADS, SMEM_BYTES, st>>>(p, CT / 2, lam);
+    if (!bf16ops) fwd_sample_kernel<<<RT, NTHREADS, SMEM_BYTES, st>>>(p, CT / 2, lam);
   }
   {
     KernelTimer tm(SCE_K_FWD, st);
     if (emit) fwd_kernel<true><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
+    else if (bf16ops) fwd_kernel<false, true><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
     else fwd_kernel<false><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
   }
   KernelTimer tm_red(SCE_K_FWD_REDUCE, st);
@@ -2042,6 +2104,7 @@ extern "C" int sce_forward_noalloc(const sce_args* a) {
 extern "C" int sce_backward(const sce_args* a) {
   if (int rc = check_common(a)) return rc;
   const int64_t N = a->shape.N, d = a->shape.d, V = a->shape.V;
+  if (a->operand_dtype != 0) return fail(SCE_EINVAL, "bf16 operands are forward only (the eval head)");
   if (!a->grad_output) return fail(SCE_EINVAL, "grad_output is NULL");
   if (!a->dx || !a->dw) return fail(SCE_EINVAL, "dx or dw is NULL");
   if (a->norm) {

@@ -127,7 +127,16 @@ __device__ __forceinline__ v16f mfma_fp8_scaled_sel(int opb, const v8i& a, const
 // stores_between (PREFETCHED only, uniform): the caller issued at least 16 vector memory stores between its prefetch of
 // K block 0 and its 8 loads of K block 1 (mfma_prefetch<1>, the stores, mfma_prefetch<2>); they are younger than
 // block 0, so the first wait may leave them in flight.
-template <bool PREFETCHED = false, class Hook = NoHook, int KSTEP = BK, bool TRB = false, int SCALE = 0>
+// BF16: the operands are bf16 (64 K values per 128-byte block) and each step is two v_mfma_f32_32x32x16_bf16, on the
+// first and the second 16 bytes of the lanes' fragments; everything else -- loads, LDS, the schedule in bytes -- is the same.
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ v16f mfma_bf16_pair(const v8i& a, const v8i& b, v16f c) {
+  const v4i a0 = {a[0], a[1], a[2], a[3]}, a1 = {a[4], a[5], a[6], a[7]}, b0 = {b[0], b[1], b[2], b[3]}, b1 = {b[4], b[5], b[6], b[7]};
+  c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a0), __builtin_bit_cast(v8bf, b0), c, 0, 0, 0);
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a1), __builtin_bit_cast(v8bf, b1), c, 0, 0, 0);
+}
+
+template <bool PREFETCHED = false, class Hook = NoHook, int KSTEP = BK, bool TRB = false, int SCALE = 0, bool BF16 = false>
 __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, int64_t lda,
                                               const uint8_t* __restrict__ Bg, int64_t ldb, int KD,
                                               uint8_t* smem, v16f (&acc)[4][4], int rot_a, int rot_b, int wave, Hook&& hook = NoHook(),
@@ -197,14 +206,16 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
   // blk: which K block of the pair; cur: fragment register set = which 64-byte half of the block
   auto mm = [&](int blk, int cur, int i) {
     const int a = i >> 2, b = i & 3;
-    if (SCALE) acc[a][b] = mfma_fp8_scaled_sel(SCALE == 1 ? b : 2 * cur, fa[cur][a], fb[cur][b], acc[a][b], 127, sc[blk]);
+    if (BF16) acc[a][b] = mfma_bf16_pair(fa[cur][a], fb[cur][b], acc[a][b]);
+    else if (SCALE) acc[a][b] = mfma_fp8_scaled_sel(SCALE == 1 ? b : 2 * cur, fa[cur][a], fb[cur][b], acc[a][b], 127, sc[blk]);
     else acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[cur][a], fb[cur][b], acc[a][b], 0, 0, 0, 0, 0, 0);
   };
   // the very first MFMA of each accumulator block takes a zero constant instead of the register: nothing clears them
   auto mm0 = [&](int i) {
     const int a = i >> 2, b = i & 3;
     const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (SCALE) acc[a][b] = mfma_fp8_scaled_sel(SCALE == 1 ? b : 0, fa[0][a], fb[0][b], zero, 127, sc[0]);
+    if (BF16) acc[a][b] = mfma_bf16_pair(fa[0][a], fb[0][b], zero);
+    else if (SCALE) acc[a][b] = mfma_fp8_scaled_sel(SCALE == 1 ? b : 0, fa[0][a], fb[0][b], zero, 127, sc[0]);
     else acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[0][a], fb[0][b], zero, 0, 0, 0, 0, 0, 0);
   };
   // One K block = two sub-steps of 16 MFMAs; register set 0 feeds the first, set 1 the second.  The

@@ -159,9 +159,11 @@ class WeightCache:
 
 
 def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_weights=None, vocab_size=None,
-               weight_cache=None, norm_eps=None, keep_dlogits=False, no_alloc=False):
+               weight_cache=None, norm_eps=None, keep_dlogits=False, no_alloc=False, operand_dtype=None):
     """One call of sce_forward.  Returns (out, saved, lse, argmax, n_valid).
 
+    operand_dtype: None / torch.float8_e4m3fn (the fused path's e4m3 operands) or torch.bfloat16 (the arithmetic of the
+    eager head under bf16 autocast: bf16 operands, logits rounded to bf16; forward only, the scales are not used).
     no_alloc: call sce_forward_noalloc instead, which keeps its scratch in a static device array of the library (this
     wrapper still allocates the outputs with torch; a caller that may not allocate passes buffers of its own to the C ABI).
 
@@ -180,7 +182,15 @@ def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_w
     V = w.shape[1]
     dev = x.device
     sz = _lib.sizes_for(N, d, V, n_predict)
-    saved = torch.empty((sz.saved_x_bytes if weight_cache is not None else sz.saved_bytes) + (sz.dlogits_bytes if keep_dlogits else 0),
+    bf16_ops = operand_dtype == torch.bfloat16
+    if operand_dtype not in (None, torch.float8_e4m3fn, torch.bfloat16):
+        raise TypeError(f"operand_dtype must be float8_e4m3fn or bfloat16, got {operand_dtype}")
+    if bf16_ops:
+        if keep_dlogits or weight_cache is not None or norm_eps is not None:
+            raise ValueError("bf16 operands are for the forward-only eval head: no kept dlogits, weight cache or fused norm")
+        x_s = w_s = 1.0
+    saved = torch.empty(sz.saved_bf16_bytes if bf16_ops else
+                        (sz.saved_x_bytes if weight_cache is not None else sz.saved_bytes) + (sz.dlogits_bytes if keep_dlogits else 0),
                         dtype=torch.uint8, device=dev)
     ws = None if no_alloc else torch.empty(sz.fwd_workspace_bytes, dtype=torch.uint8, device=dev)
     losses = torch.empty(N, dtype=torch.float32, device=dev)
@@ -198,6 +208,7 @@ def ce_forward(x, w, targets, x_s, w_s, cap, reduction, want_argmax=False, mtp_w
         a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
     a.vocab_limit = 0 if vocab_size is None else int(vocab_size)
     a.dlogits_from_forward = int(bool(keep_dlogits))
+    a.operand_dtype = _lib.SCE_BF16 if bf16_ops else 0
     if norm_eps is not None:
         a.norm, a.norm_eps = 1, float(norm_eps)
     if weight_cache is not None:
@@ -395,18 +406,24 @@ class FusedNormSoftcappedCrossEntropy(torch.autograd.Function):
         return dh, None, None, dw, None, None, None, None, None, None, None, None
 
 
-def softcapped_cross_entropy(x, lm_head_weight, targets, x_s, w_s, cap=15.0, vocab_size=None, reduction="mean",
-                             norm_eps=None):
+def softcapped_cross_entropy(x, lm_head_weight, targets, x_s=None, w_s=None, cap=15.0, vocab_size=None, reduction="mean",
+                             norm_eps=None, operand_dtype=None):
     """Forward-only loss of the eager head (tiny/train.py:741-743) on the fused kernel:
-    ``F.cross_entropy(cap * tanh((x @ W)[..., :vocab_size] / cap), targets, ignore_index=-1, reduction=...)`` with
-    fp8 operands; the N x V logits are never stored.  ``x`` may have leading batch dimensions.  With ``norm_eps``
+    ``F.cross_entropy(cap * tanh((x @ W)[..., :vocab_size] / cap), targets, ignore_index=-1, reduction=...)``; the
+    N x V logits are never stored.  ``operand_dtype=torch.bfloat16`` computes what the reference's eval computes -- a bf16
+    matmul (CastedLinearT under autocast, tiny/train.py:496-497) whose bf16 result goes through the softcap in fp32 -- so
+    that validation losses compare; the default keeps the training path's e4m3 operands with scales ``x_s``, ``w_s``.  ``x`` may have leading batch dimensions.  With ``norm_eps``
     given, ``x`` is the hidden state before the final ``F.rms_norm(x, (d,), eps=norm_eps)`` (tiny/train.py:734),
     which is then applied inside the quantiser."""
     lead = x.shape[:-1]
     x2 = x.reshape(-1, x.shape[-1])
+    if operand_dtype == torch.bfloat16:
+        x_s = w_s = 1.0
+    elif x_s is None or w_s is None:
+        raise ValueError("e4m3 operands need their scales x_s and w_s")
     out, _saved, _lse, _am, _nv = ce_forward(x2.detach(), lm_head_weight.detach(), targets.reshape(-1),
                                              _scale_value(x_s, x2), _scale_value(w_s, lm_head_weight), float(cap),
-                                             reduction, vocab_size=vocab_size, norm_eps=norm_eps)
+                                             reduction, vocab_size=vocab_size, norm_eps=norm_eps, operand_dtype=operand_dtype)
     return out if reduction == "mean" else out.reshape(lead)
 
 

@@ -445,3 +445,48 @@ def test_fused_norm_with_multi_token_prediction_and_eval_head():
                                         norm_eps=torch.finfo(torch.float32).eps)
     ev_plain = softcapped_cross_entropy(F.rms_norm(h0, (d,)), w0, y, x_s, inp.w_s, vocab_size=1250, reduction="none")
     assert torch.equal(ev_fused, ev_plain)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_eval_head_with_bf16_operands(dtype):
+    """The reference evaluates with a bf16 matmul (CastedLinearT under autocast, tiny/train.py:496-497) whose bf16 logits
+    are sliced to the vocabulary, softcapped and fed to F.cross_entropy in fp32 (tiny/train.py:741-743).  With
+    operand_dtype=torch.bfloat16 the fused head computes that arithmetic: same operands, fp32 accumulation, logits
+    rounded to bf16.  The two GEMMs add in different orders, so a logit may land on the neighbouring bf16 value (one
+    part in 256 of it) now and then; the losses are compared at the tolerance stated for the loss."""
+    import torch.nn.functional as F
+    from slowrun_amd.cuda_kernels import softcapped_cross_entropy
+    inp = _small("irregular", 1100, 256, 2300)
+    vocab = 2250
+    inp.targets[inp.targets >= vocab] = 3
+    x = inp.x.cuda().to(dtype).reshape(2, 550, 256)
+    w = inp.w.cuda().to(dtype)
+    y = inp.targets.cuda().reshape(2, 550)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        logits = (x @ w.type_as(x))                                   # CastedLinearT.forward
+    assert logits.dtype == torch.bfloat16
+    logits = logits[..., :vocab].float()
+    logits = inp.cap * torch.tanh(logits / inp.cap)
+    for red in ("mean", "none"):
+        ref = F.cross_entropy(logits.view(-1, vocab), y.reshape(-1), ignore_index=-1, reduction=red)
+        got = softcapped_cross_entropy(x, w, y, cap=inp.cap, vocab_size=vocab, reduction=red, operand_dtype=torch.bfloat16)
+        assert got.shape == (() if red == "mean" else (2, 550))
+        err = float((got.reshape(-1) - ref.reshape(-1)).abs().max() / ref.abs().max())
+        print(dtype, red, "rel err", err)
+        assert err < pu.LOSS_RTOL if red == "mean" else err < 1e-2
+    # the e4m3 path on the same data differs from the bf16 one by more than that: the two are not the same arithmetic
+    fp8 = softcapped_cross_entropy(x, w, y, inp.x_s, inp.w_s, cap=inp.cap, vocab_size=vocab, reduction="none")
+    bf = softcapped_cross_entropy(x, w, y, cap=inp.cap, vocab_size=vocab, reduction="none", operand_dtype=torch.bfloat16)
+    assert float((fp8 - bf).abs().max()) > 1e-3
+
+
+def test_bf16_operands_are_forward_only():
+    from slowrun_amd import cuda_kernels as ck
+    inp = _small("tiny_track", 300, 128, 600)
+    x = inp.x.cuda().bfloat16()
+    w = inp.w.cuda().bfloat16()
+    y = inp.targets.cuda()
+    loss, saved, *_ = ck.ce_forward(x, w, y, 1.0, 1.0, inp.cap, "mean", operand_dtype=torch.bfloat16)
+    assert torch.isfinite(loss)
+    with pytest.raises(ValueError, match="forward-only"):
+        ck.ce_forward(x, w, y, 1.0, 1.0, inp.cap, "mean", operand_dtype=torch.bfloat16, keep_dlogits=True)
