@@ -218,6 +218,20 @@ typedef struct sce_timing {
 int sce_timing_enable(int on);            /* also clears the accumulators */
 int sce_timing_read(sce_timing* out);
 
+/* ---- measurement aids (no counterpart in the reference) ---------------------------------
+ * What the matrix pipe and the MFMA main loop of this library reach on their own, for the ceiling figures that
+ * `python -m slowrun_amd.ceiling` reports.  Both synchronise with the host (they time `reps` launches with HIP events)
+ * and return the rate in TFLOP/s and the shader clock that the kernels themselves saw (their cycle counter against the
+ * 100 MHz reference counter; median over workgroups).  scratch: device memory, 1 KiB per 256 x 256 tile and 16 KiB more.
+ *  sce_bench_mfma: 16 independent v_mfma_f32_32x32x64_f8f6f4 per wave and round, operands in registers, no memory traffic;
+ *                  random_bytes: NULL (all operands 1.0) or 64 KiB x (4 x CUs) of device bytes that become the operands.
+ *  sce_bench_gemm: C = A B^T through the library's main loop (256 x 256 tiles, global -> LDS -> MFMA), the sums of the
+ *                  accumulators stored; A is (M, K) and B (N, K) e4m3 bytes with a row stride of K + 128 bytes. */
+int sce_bench_mfma(const void* random_bytes, int32_t iters, int32_t reps, void* scratch, size_t scratch_bytes, int32_t device,
+                   void* stream, double* tflops, double* shader_mhz);
+int sce_bench_gemm(const void* A, const void* B, int64_t M, int64_t N, int64_t K, int32_t reps, void* scratch, size_t scratch_bytes,
+                   int32_t device, void* stream, double* tflops, double* shader_mhz);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,166 @@
+"""What the MI355X in front of us sustains on fp8 matrix work, measured: ``python -m slowrun_amd.ceiling``.
+
+The loss head is bound by the matrix pipe, whose published peak (5.0 PFLOP/s dense fp8) assumes the full 2.4 GHz
+shader clock.  This report puts numbers beside that peak, each from a short run on the GPU at hand:
+
+  1. the matrix instruction alone (operands in registers), on constant and on random operands, with the shader clock
+     the kernel itself saw;
+  2. the library's main loop alone (global -> LDS -> MFMA, no epilogue) on the three GEMM shapes of the headline
+     workload, on random and on all-zero operands;
+  3. the vendor library's fp8 GEMM (torch._scaled_mm -> hipBLASLt) on the same shapes;
+  4. the shader clock and package power that rocm-smi reports while the main loop runs flat out.
+
+Prints a plain-text report (and one JSON line at the end).  Nothing here is on the product path.
+"""
+import argparse
+import ctypes as C
+import json
+import subprocess
+import threading
+import time
+
+import torch
+
+from . import _lib
+
+PEAK_FP8_TFLOPS = 5000.0
+
+
+def _mfma(random, scratch, iters=20000, reps=3):
+    dev = scratch.device
+    data = None
+    if random:
+        ncu = torch.cuda.get_device_properties(dev).multi_processor_count
+        data = torch.randint(0, 256, (4 * ncu * 65536,), dtype=torch.uint8, device=dev)
+        data[(data & 0x7f) == 0x7f] = 0x38                          # no NaN codes among the operands
+    tf, mhz = C.c_double(), C.c_double()
+    _lib.check(_lib.lib().sce_bench_mfma(data.data_ptr() if random else None, iters, reps, scratch.data_ptr(), scratch.numel(),
+                                         dev.index, None, C.byref(tf), C.byref(mhz)), "sce_bench_mfma")
+    return tf.value, mhz.value
+
+
+def _operand(rows, K, kind, dev):
+    t = torch.zeros(rows, K + 128, dtype=torch.uint8, device=dev)
+    if kind == "random":
+        v = torch.randint(0, 256, (rows, K), dtype=torch.uint8, device=dev)
+        v[(v & 0x7f) == 0x7f] = 0x38
+        t[:, :K] = v
+    return t
+
+
+def _gemm(M, N, K, kind, scratch, reps=5):
+    dev = scratch.device
+    a, b = _operand(M, K, kind, dev), _operand(N, K, kind, dev)
+    tf, mhz = C.c_double(), C.c_double()
+    _lib.check(_lib.lib().sce_bench_gemm(a.data_ptr(), b.data_ptr(), M, N, K, reps, scratch.data_ptr(), scratch.numel(), dev.index,
+                                         None, C.byref(tf), C.byref(mhz)), "sce_bench_gemm")
+    return tf.value, mhz.value
+
+
+def _hipblaslt(M, N, K, dev, reps=5):
+    a = torch.randn(M, K, device=dev).to(torch.float8_e4m3fn)
+    b = torch.randn(N, K, device=dev).to(torch.float8_e4m3fn)
+    one = torch.ones((), device=dev)
+    try:
+        f = lambda: torch._scaled_mm(a, b.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+        f()
+    except Exception as e:                      # noqa: BLE001 - reported, not fatal
+        return None, str(e).splitlines()[0]
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        f()
+    e1.record()
+    torch.cuda.synchronize()
+    return 2.0 * M * N * K * reps / (e0.elapsed_time(e1) * 1e-3) * 1e-12, None
+
+
+def _smi_sample():
+    try:
+        out = subprocess.run(["rocm-smi", "--showclocks", "--showpower", "--json"], capture_output=True, text=True, timeout=10).stdout
+        card = next(iter(json.loads(out).values()))
+    except Exception:                            # noqa: BLE001
+        return None
+    sclk = next((v for k, v in card.items() if "sclk" in k.lower()), None)
+    power = next((v for k, v in card.items() if "power" in k.lower() and "socket" in k.lower()), None) or \
+        next((v for k, v in card.items() if "power" in k.lower()), None)
+    return {"sclk": sclk, "power": power}
+
+
+def _under_load(scratch, seconds=4.0):
+    """rocm-smi readings while the main loop runs on random operands."""
+    dev = scratch.device
+    a, b = _operand(8192, 8192, "random", dev), _operand(8192, 8192, "random", dev)
+    samples, stop = [], threading.Event()
+
+    def poll():
+        while not stop.is_set():
+            smp = _smi_sample()
+            if smp:
+                samples.append(smp)
+            time.sleep(0.3)
+
+    idle = _smi_sample()
+    th = threading.Thread(target=poll)
+    th.start()
+    tf, mhz = C.c_double(), C.c_double()
+    t0 = time.time()
+    rates = []
+    while time.time() - t0 < seconds:
+        _lib.check(_lib.lib().sce_bench_gemm(a.data_ptr(), b.data_ptr(), 8192, 8192, 8192, 40, scratch.data_ptr(), scratch.numel(),
+                                             dev.index, None, C.byref(tf), C.byref(mhz)), "sce_bench_gemm")
+        rates.append((tf.value, mhz.value))
+    stop.set()
+    th.join()
+    return idle, samples, rates
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--no-smi", action="store_true")
+    args = ap.parse_args()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    scratch = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+    rep = {"peak_fp8_tflops": PEAK_FP8_TFLOPS}
+    print(f"device: {torch.cuda.get_device_name(dev)}; published dense fp8 peak {PEAK_FP8_TFLOPS:.0f} TFLOP/s at 2400 MHz")
+    print("\n1. v_mfma_f32_32x32x64_f8f6f4 alone (operands in registers, 16 independent accumulators per wave)")
+    rep["mfma_only"] = {}
+    for kind in ("constant", "random"):
+        tf, mhz = _mfma(kind == "random", scratch)
+        rep["mfma_only"][kind] = {"tflops": round(tf, 1), "shader_mhz": round(mhz)}
+        print(f"   {kind:9s} operands: {tf:7.1f} TFLOP/s = {tf / PEAK_FP8_TFLOPS * 100:5.1f} % of peak, shader clock seen by the kernel {mhz:5.0f} MHz")
+    print("\n2. the main loop alone (global -> LDS -> MFMA, sums of the accumulators stored)")
+    shapes = [("square", 8192, 8192, 8192), ("logits  (V x N, K = d)", 50432, 65536, 2560), ("dX      (d x N, K = V)", 2560, 65536, 50432),
+              ("dW      (d x V, K = N)", 2560, 50432, 65536)]
+    rep["main_loop"] = {}
+    for name, M, N, K in shapes:
+        row = {}
+        for kind in ("random", "zero"):
+            tf, mhz = _gemm(M, N, K, kind, scratch, reps=3 if M * N * K > 1e12 else 10)
+            row[kind] = {"tflops": round(tf, 1), "shader_mhz": round(mhz)}
+        rep["main_loop"][name.split()[0]] = row
+        print(f"   {name:24s} random operands {row['random']['tflops']:7.1f} TFLOP/s at {row['random']['shader_mhz']:4d} MHz | "
+              f"all-zero operands {row['zero']['tflops']:7.1f} TFLOP/s at {row['zero']['shader_mhz']:4d} MHz")
+    print("\n3. torch._scaled_mm (hipBLASLt) fp8 e4m3, bf16 out, random operands")
+    rep["hipblaslt"] = {}
+    for name, M, N, K in shapes:
+        tf, err = _hipblaslt(N, M, K, dev, reps=3 if M * N * K > 1e12 else 10)
+        rep["hipblaslt"][name.split()[0]] = None if tf is None else round(tf, 1)
+        print(f"   {name:24s} " + (f"{tf:7.1f} TFLOP/s" if tf is not None else f"not available: {err}"))
+    if not args.no_smi:
+        print("\n4. rocm-smi while the main loop runs (8192^3, random operands)")
+        idle, samples, rates = _under_load(scratch)
+        rep["smi"] = {"idle": idle, "under_load": samples[:: max(1, len(samples) // 6)]}
+        rep["under_load"] = {"tflops": [round(r[0], 1) for r in rates][:: max(1, len(rates) // 6)],
+                             "shader_mhz": [round(r[1]) for r in rates][:: max(1, len(rates) // 6)]}
+        print(f"   idle: {idle}")
+        for smp in rep["smi"]["under_load"]:
+            print(f"   load: {smp}")
+        print(f"   main loop meanwhile: {rep['under_load']['tflops']} TFLOP/s at {rep['under_load']['shader_mhz']} MHz (in-kernel)")
+    print("\n" + json.dumps(rep))
+
+
+if __name__ == "__main__":
+    main()

@@ -23,6 +23,7 @@
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
+#include <algorithm>
 #include <mutex>
 #include <type_traits>
 #include <vector>
@@ -1616,6 +1617,76 @@ __global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restri
     if (j0 + m < d) Elem<T>::store(dw + (int64_t)(j0 + m) * dw_ld + v, o[m]);
 }
 
+// ------------------------------------------------------------------------------------------
+// measurement aids (sce_bench_*): what the matrix pipe and the main loop reach on their own
+// ------------------------------------------------------------------------------------------
+// The matrix instruction alone: every wave issues `iters` rounds of 16 independent v_mfma_f32_32x32x64_f8f6f4 on
+// operands it keeps in registers (bytes from `data`, or a constant when data is NULL); no memory traffic in the loop.
+// clk[2 w], clk[2 w + 1]: shader clocks and 100 MHz ticks that workgroup w's first wave spent in the loop.
+__global__ __launch_bounds__(256) void bench_mfma_kernel(const uint8_t* __restrict__ data, int iters, float* __restrict__ out,
+                                                        long long* __restrict__ clk) {
+  v8i fa[4], fb[4];
+#pragma unroll
+  for (int n = 0; n < 4; ++n) {
+    if (data) {
+      fa[n] = *reinterpret_cast<const v8i*>(data + ((size_t)(blockIdx.x * 256 + threadIdx.x) * 8 + n) * 32);
+      fb[n] = *reinterpret_cast<const v8i*>(data + ((size_t)(blockIdx.x * 256 + threadIdx.x) * 8 + 4 + n) * 32);
+    } else {
+      fa[n] = (v8i){0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838};
+      fb[n] = fa[n];
+    }
+  }
+  v16f acc[4][4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+  const long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+        acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[a], fb[b], acc[a][b], 0, 0, 0, 0, 0, 0);
+  }
+  const long long c1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
+  float sum = 0.f;
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sum += acc[a][b][r];
+  out[blockIdx.x * 256 + threadIdx.x] = sum;
+  if (threadIdx.x == 0 && blockIdx.x < 1024) { clk[2 * blockIdx.x] = c1 - c0; clk[2 * blockIdx.x + 1] = r1 - r0; }
+}
+
+// The main loop alone: C = A B^T over 256 x 256 tiles, both operands e4m3 rows of ld bytes; every thread writes the
+// sum of its accumulators (so that the work cannot be dropped), nothing else.
+__global__ __launch_bounds__(256) void bench_gemm_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, float* __restrict__ C,
+                                                        int KD, int RT, int CT, int64_t ld, long long* __restrict__ clk) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  int rt, ct;
+  if (!map_tile(blockIdx.x, RT, CT, rt, ct)) return;
+  const long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+  v16f acc[4][4];
+  mfma_mainloop(A + (int64_t)rt * 256 * ld, ld, B + (int64_t)ct * 256 * ld, ld, KD, smem, acc, ct & 7, 2 * (rt & 3),
+                __builtin_amdgcn_readfirstlane(threadIdx.x >> 6));
+  float sum = 0.f;
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sum += acc[a][b][r];
+  C[(int64_t)blockIdx.x * 256 + threadIdx.x] = sum;
+  if (threadIdx.x == 0 && blockIdx.x < 1024) {
+    clk[2 * blockIdx.x] = __builtin_readcyclecounter() - c0; clk[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - r0;
+  }
+}
+
 }  // namespace sce
 
 // ==========================================================================================
@@ -2306,5 +2377,80 @@ extern "C" int sce_backward(const sce_args* a) {
                                                     (bf16_t*)a->dw, a->dw_ld);
   }
   HIP_TRY(hipGetLastError());
+  return SCE_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// measurement aids
+// ------------------------------------------------------------------------------------------
+static double median_mhz(const long long* clk, int n) {
+  std::vector<double> v;
+  for (int i = 0; i < n; ++i)
+    if (clk[2 * i + 1] > 0) v.push_back((double)clk[2 * i] / (double)clk[2 * i + 1] * 100.0);
+  if (v.empty()) return 0.0;
+  std::sort(v.begin(), v.end());
+  return v[v.size() / 2];
+}
+
+extern "C" int sce_bench_mfma(const void* random_bytes, int32_t iters, int32_t reps, void* scratch, size_t scratch_bytes, int32_t device,
+                              void* stream, double* tflops, double* shader_mhz) {
+  if (!scratch || !tflops || !shader_mhz || iters <= 0 || reps <= 0) return fail(SCE_EINVAL, "bad argument");
+  if (int rc = check_device(device)) return rc;
+  DeviceGuard guard(device);
+  if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", device);
+  const int ncu = device_cus_or_default(device), grid = 4 * ncu;           // one wave per SIMD would be grid = ncu; four keep every SIMD fed
+  const size_t need = (size_t)grid * 256 * 4 + 2 * 1024 * sizeof(long long);
+  if (scratch_bytes < need) return fail(SCE_EINVAL, "scratch too small: %zu < %zu", scratch_bytes, need);
+  hipStream_t st = (hipStream_t)stream;
+  float* out = (float*)scratch;
+  long long* clk = (long long*)((uint8_t*)scratch + (size_t)grid * 256 * 4);
+  hipEvent_t e0, e1;
+  HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
+  bench_mfma_kernel<<<grid, 256, 0, st>>>((const uint8_t*)random_bytes, iters, out, clk);      // warm-up
+  HIP_TRY(hipEventRecord(e0, st));
+  for (int r = 0; r < reps; ++r) bench_mfma_kernel<<<grid, 256, 0, st>>>((const uint8_t*)random_bytes, iters, out, clk);
+  HIP_TRY(hipEventRecord(e1, st));
+  HIP_TRY(hipEventSynchronize(e1));
+  float ms = 0.f;
+  HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
+  std::vector<long long> h(2 * 1024);
+  HIP_TRY(hipMemcpy(h.data(), clk, h.size() * sizeof(long long), hipMemcpyDeviceToHost));
+  (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+  const double flops = (double)reps * grid * 4.0 * iters * 16.0 * (2.0 * 32 * 32 * 64);
+  *tflops = flops / (ms * 1e-3) * 1e-12;
+  *shader_mhz = median_mhz(h.data(), grid < 1024 ? grid : 1024);
+  return SCE_OK;
+}
+
+extern "C" int sce_bench_gemm(const void* A, const void* B, int64_t M, int64_t N, int64_t K, int32_t reps, void* scratch, size_t scratch_bytes,
+                              int32_t device, void* stream, double* tflops, double* shader_mhz) {
+  if (!A || !B || !scratch || !tflops || !shader_mhz || reps <= 0) return fail(SCE_EINVAL, "bad argument");
+  if (M <= 0 || N <= 0 || K <= 0 || M % 256 || N % 256 || K % 256) return fail(SCE_EINVAL, "M, N, K must be positive multiples of 256");
+  if (int rc = check_device(device)) return rc;
+  DeviceGuard guard(device);
+  if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", device);
+  const int RT = (int)(M / 256), CT = (int)(N / 256), grid = map_tile_grid(RT, CT);
+  const size_t need = (size_t)grid * 256 * 4 + 2 * 1024 * sizeof(long long);
+  if (scratch_bytes < need) return fail(SCE_EINVAL, "scratch too small: %zu < %zu", scratch_bytes, need);
+  HIP_TRY(hipFuncSetAttribute((const void*)bench_gemm_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+  hipStream_t st = (hipStream_t)stream;
+  float* out = (float*)scratch;
+  long long* clk = (long long*)((uint8_t*)scratch + (size_t)grid * 256 * 4);
+  const int64_t ld = row_stride(K);
+  hipEvent_t e0, e1;
+  HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
+  bench_gemm_kernel<<<grid, NTHREADS, SMEM_BYTES, st>>>((const uint8_t*)A, (const uint8_t*)B, out, (int)(K / BK), RT, CT, ld, clk);
+  HIP_TRY(hipEventRecord(e0, st));
+  for (int r = 0; r < reps; ++r)
+    bench_gemm_kernel<<<grid, NTHREADS, SMEM_BYTES, st>>>((const uint8_t*)A, (const uint8_t*)B, out, (int)(K / BK), RT, CT, ld, clk);
+  HIP_TRY(hipEventRecord(e1, st));
+  HIP_TRY(hipEventSynchronize(e1));
+  float ms = 0.f;
+  HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
+  std::vector<long long> h(2 * 1024);
+  HIP_TRY(hipMemcpy(h.data(), clk, h.size() * sizeof(long long), hipMemcpyDeviceToHost));
+  (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+  *tflops = 2.0 * M * N * K * reps / (ms * 1e-3) * 1e-12;
+  *shader_mhz = median_mhz(h.data(), grid < 1024 ? grid : 1024);
   return SCE_OK;
 }
