@@ -46,7 +46,7 @@ enum {
 typedef struct sce_shape {
   int64_t N;           /* rows (tokens)                         */
   int64_t d;           /* hidden size, multiple of 16, < 2^22   */
-  int64_t V;           /* vocabulary (columns of W); N, d, V < 2^24 */
+  int64_t V;           /* vocabulary (columns of W), at most 524288; N < 2^24 */
   int32_t n_predict;   /* number of MTP offsets, 1..4           */
   int32_t reserved;
 } sce_shape;
@@ -187,12 +187,12 @@ int sce_forward(const sce_args* args);
  * share the one array: calls that overlap in time on the same device (two streams, two threads) race. */
 int sce_forward_noalloc(const sce_args* args);
 
-/* Backward: recompute logit tiles from the saved fp8 operands, form dlogits on chip,
- * dX = dlogits * W_q^T, dW = X_q^T * dlogits.  Replaces
+/* Backward: dX = dlogits * W_q^T, dW = X_q^T * dlogits on the MFMA, the dlogits either as the forward pass left them
+ * (dlogits_from_forward) or formed again from recomputed logit tiles, row panel by row panel.  Replaces
  * FusedSoftcappedCrossEntropy.backward (tiny/cuda_kernels.py:375-414) and the dlogits half
  * of the reference kernel (tiny/cuda_kernels.py:242-301).  Needs the `saved` buffer of the
- * matching sce_forward call, the same shape/scales/cap/targets, and a workspace of at
- * least bwd_workspace_min_bytes. */
+ * matching sce_forward call, the same shape/scales/cap/targets, and a workspace of
+ * bwd_workspace_kept_bytes (dlogits_from_forward) or at least bwd_workspace_min_bytes. */
 int sce_backward(const sce_args* args);
 
 /* ---- optional per-kernel timing (off by default) --------------------------------------
