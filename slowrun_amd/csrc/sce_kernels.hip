@@ -524,9 +524,10 @@ __device__ __forceinline__ float wave_max_dpp(float v) {
 
 // lam (LDS, wave-uniform base; per row block LAM_STRIDE floats apart, one float for each of LAM_LANES lanes): the row's
 // exponent boost (see fwd_sample_kernel).
+// want_argmax (uniform, STATS only): see the lookup of the maximum's column below.
 template <bool EDGE, bool STATS, int LAM_STRIDE = NTHREADS, int LAM_LANES = 64>
 __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float k1, float c2, int vlim, int vabs0,
-                                                 uint8_t* TT, int wa, int wb, float* stat, const float* lam) {
+                                                 uint8_t* TT, int wa, int wb, float* stat, const float* lam, bool want_argmax = true) {
   const int lane = lane_id();
   const int vloc0 = wa * 128 + 4 * (lane >> 5);       // column (within the tile) of accumulator register 0 of block a = 0
   const int k = lane & 3;
@@ -547,7 +548,7 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
         tmax = fmaxf(tmax, x);
       }
     const float lamb = lam[b * LAM_STRIDE + (lane_id() & (LAM_LANES - 1))];      // (index taken anew: see lane_id)
-    const float lg = wave_max(fmaf(c2, fast_rcp(1.0f + fast_exp2(tmax * k1)), lamb));      // over the block: log2 of the largest boosted e^{z - cap}
+    const float lg = wave_max_dpp(fmaf(c2, fast_rcp(1.0f + fast_exp2(tmax * k1)), lamb));      // over the block: log2 of the largest boosted e^{z - cap}
     const float sb = floorf(8.8f - lg);                       // between -120 and 8 + 2 cap log2(e) <= 124 (cap <= 40, boost <= 120)
     const float cs = sb + 2.0f + lamb;                        // the 4 of 4 r (1 - r) and the row's boost ride along
     expword |= (uint32_t)(127 - (int)sb) << (8 * b);
@@ -597,9 +598,12 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
     if (STATS) {
       stat[(0 + b) * NTHREADS] += ssum * fast_exp2(-cs);
       const float amax = stat[(4 + b) * NTHREADS];
-      // the column of the maximum is looked up only when a tile reaches a lane's running maximum (on a tie the lower
-      // column wins: the running one may be a target of this very tile, which take_target_logits has put there)
-      if (__builtin_amdgcn_ballot_w64(tmax >= amax) != 0) {
+      // The column of the maximum is looked up only when a tile reaches a lane's running maximum (on a tie the lower
+      // column wins: the running one may be a target of this very tile, which take_target_logits has put there) -- which
+      // some lane of the 64 does in nearly every tile of a walk of a few dozen: a caller that does not ask for the argmax
+      // is spared it.  (A flag at run time, not a template parameter: without the lookup in the code the register
+      // allocation of the rest changes, and accumulators end up in scratch memory.)
+      if (want_argmax && __builtin_amdgcn_ballot_w64(tmax >= amax) != 0) {
         if (tmax >= amax) {
           int targ = 0x7fffffff;
 #pragma unroll
@@ -654,6 +658,7 @@ struct FwdParams {
   float ic2;               // 1 / c2, c2 = -2 cap log2(e): e^{z - cap} = exp2(c2 / (1 + e^{2u/cap}))
   float c2;
   const DevConsts* dc;     // non-NULL: sc and k1 come from here (a scale lives on the device)
+  int want_argmax;         // the caller asks for the rows' argmax: the column of the running maximum is tracked
 };
 
 // Per 256 x 256 tile and per row a lane owns: add up e^{z - cap} over its 64 columns and keep the
@@ -684,7 +689,7 @@ __device__ __forceinline__ void fwd_epilogue(const v16f (&acc)[4][4], const FwdP
       }
     }
     sum[b] += s;
-    if (__builtin_amdgcn_ballot_w64(tmax > amax[b]) != 0) {
+    if (p.want_argmax && __builtin_amdgcn_ballot_w64(tmax > amax[b]) != 0) {
       if (tmax > amax[b]) {
         int targ = 0x7fffffff;
 #pragma unroll
@@ -877,8 +882,8 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
       uint8_t* TT = smem + FWD_STAGE_OFF;
       uint32_t ew;
       const float* lam = reinterpret_cast<const float*>(smem + FWD_STAT_OFF) + 12 * NTHREADS + wave * 64;
-      if (vlim < 256) ew = form_dlogits<true, true>(acc, p.k1, p.c2, vlim, vbase, TT, wa, wb, stat, lam);
-      else ew = form_dlogits<false, true>(acc, p.k1, p.c2, vlim, vbase, TT, wa, wb, stat, lam);
+      if (vlim < 256) ew = form_dlogits<true, true>(acc, p.k1, p.c2, vlim, vbase, TT, wa, wb, stat, lam, p.want_argmax != 0);
+      else ew = form_dlogits<false, true>(acc, p.k1, p.c2, vlim, vbase, TT, wa, wb, stat, lam, p.want_argmax != 0);
       store_dlogits_quadrant(TT, p.ghat_t + ((int64_t)ct * p.kbw + 2 * rt + wb) * BLOCKED_KSTEP + wa * 128 * BK, wa, wb);
       if (lane_id() == 0) p.gexp[(int64_t)(2 * ct + wa) * p.kbw + 2 * rt + wb] = ew;
     } else {
@@ -2480,6 +2485,7 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
   p.dp = S.dp; p.ldx = S.ldx; p.N = (int)N; p.V = (int)Vl; p.Np = (int)S.Np; p.RT = RT; p.CT = CTw; p.S = nsplit;
   p.sc = bf16ops ? 1.0f : (float)a->x_s * (float)a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.c2 = -2.0f * a->cap * LOG2E; p.ic2 = 1.0f / p.c2;
   p.dc = bf16ops ? nullptr : dcp;
+  p.want_argmax = a->argmax != nullptr;
   const int grid = 8 * nsplit * ((RT + 7) / 8);
   {
     // the exponent boosts of the rows, from the tile in the middle of the vocabulary (kept for backward in either mode)
