@@ -88,6 +88,7 @@ struct BwdLayout {
   size_t off_gexp, off_rho, off_rowinfo, off_hcoef, off_blockmax, off_xi, off_xt, off_dwacc, off_perm, off_keys,
       off_segoff, off_longlist, off_longbase, off_longsum, off_sorttmp, off_dxpart, off_ghat_t, fixed, total;
   size_t sorttmp_bytes, part_stride;   // part_stride: bytes between consecutive fp32 dW partials
+  size_t off_dwtail, tail_bytes;       // partial tiles of the K-split last round of dW: behind `total`, used when the workspace reaches that far
   int nparts;
 };
 

@@ -1814,6 +1814,58 @@ __global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
 // sort keys: one entry per (offset k, row i): key = target y_{i+k} (V if the pair takes no part; targets at or
 // beyond the vocabulary limit Vl take no part),
 // value = entry id k * Np + i
+// The tiles of the last, partly filled round of dW (tile0 .. tile0 + ntail - 1 of the round-robin order), shared out
+// along K: a tile's K loop is kp pairs of K blocks long, all of them together W = ntail * kp pairs, and workgroup g takes
+// pairs [g share, (g + 1) share) of that line -- the end of one tile and the beginning of the next, when its range
+// straddles them.  Piece (g, t) of tile t goes to buf[g + t] as plain stores (g + t grows by one from each piece to the
+// next along the line, so no two pieces meet); bwd_dw_final_kernel adds up a tile's pieces in the order of g.
+// a pointer that is the same in every lane, moved to scalar registers
+__device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* q) {
+  const uint64_t u = (uint64_t)(uintptr_t)q;
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)u), hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(u >> 32));
+  return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+struct DwTail {
+  float* buf;
+  int tile0, ntail, kp, share;      // tile0 < 0: no tail (every tile is in the fp32 partial)
+};
+__global__ __launch_bounds__(256) void bwd_dw_tail_kernel(DwParams p, DwTail tl) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int g = blockIdx.x;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
+  int pos = g * tl.share;
+  const int end = min(tl.ntail * tl.kp, pos + tl.share);
+  uint32_t* lsc = reinterpret_cast<uint32_t*>(smem + SMEM_BYTES);
+  while (pos < end) {
+    // (everything here is uniform, but the divisions leave their results in vector registers: the main loop wants
+    // its addresses in scalar ones)
+    const int tt = __builtin_amdgcn_readfirstlane(pos / tl.kp);
+    const int k0 = pos - tt * tl.kp, k1 = min(tl.kp, k0 + (end - pos)), KD = 2 * (k1 - k0);
+    int rt, ct;
+    tile_from_index(tl.tile0 + tt, p.RT, p.CT, rt, ct);
+    rt = __builtin_amdgcn_readfirstlane(rt); ct = __builtin_amdgcn_readfirstlane(ct);
+    for (int e = t; e < 2 * KD; e += NTHREADS) {
+      const int w = e >= KD, kb = e - w * KD;
+      lsc[e] = p.gexp[(int64_t)(2 * ct + w) * p.kbw + 2 * k0 + kb];
+    }
+    __syncthreads();
+    v16f acc[4][4];
+    mfma_mainloop<false, NoHook, BLOCKED_KSTEP, false, 2>(uniform_ptr(p.xt + ((int64_t)rt * p.kbn + p.kb0 + 2 * k0) * BLOCKED_KSTEP), BK,
+                                                          uniform_ptr(p.ghat_t + ((int64_t)ct * p.kbw + 2 * k0) * BLOCKED_KSTEP), BK,
+                                                          __builtin_amdgcn_readfirstlane(KD), smem, acc, ct & 7, 2 * (rt & 3),
+                                                          __builtin_amdgcn_readfirstlane(wave), NoHook(), 0, 0,
+                                                          lsc + __builtin_amdgcn_readfirstlane(wb) * KD);
+    float* dst0 = tl.buf + (size_t)(g + tt) * 65536 + (wa * 128 + 4 * (lane >> 5)) * 256 + wb * 128 + (lane & 31);
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dst0[(a * 32 + 8 * (r >> 2) + (r & 3)) * 256 + b * 32] = acc[a][b][r];
+    pos += k1 - k0;
+  }
+}
+
 __global__ __launch_bounds__(256) void bwd_keys_kernel(const int64_t* __restrict__ targets, int64_t ignore_index, int N, int Np, int Vl,
                                                       int V, int n_predict, int32_t* __restrict__ keys, int32_t* __restrict__ vals,
                                                       int32_t* __restrict__ longlist) {
@@ -1922,7 +1974,8 @@ __global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restri
                                                           const int32_t* __restrict__ perm, const float* __restrict__ hcoef,
                                                           const uint8_t* __restrict__ xq, int64_t ldx, int Np, const float* __restrict__ xi,
                                                           const float* __restrict__ longsum, const int32_t* __restrict__ longbase, int64_t dq,
-                                                          float x_s_host, const DevConsts* __restrict__ dc, int d, int V, T* __restrict__ dw, int64_t dw_ld) {
+                                                          float x_s_host, const DevConsts* __restrict__ dc, int d, int V, T* __restrict__ dw, int64_t dw_ld,
+                                                          DwTail tl, int RT, int CT) {
   const float x_s = dc ? dc->x_s : x_s_host;
   const int t = threadIdx.x;
   const int v = blockIdx.x * 64 + (t & 63);
@@ -1930,11 +1983,30 @@ __global__ __launch_bounds__(256) void bwd_dw_final_kernel(const float* __restri
   if (v >= V || j0 >= d) return;
   const float scale = x_s * xi[0];
   float o[16];
+  // the block's 64 x 64 elements lie in one 256 x 256 tile: one of the K-split last round (see bwd_dw_tail_kernel)?
+  int tt = -1;
+  if (tl.tile0 >= 0) {
+    const int rt = blockIdx.y >> 2, ct = blockIdx.x >> 2, g8 = ct >> 3, gw = (CT - 8 * g8) < 8 ? (CT - 8 * g8) : 8;
+    tt = g8 * 8 * RT + rt * gw + (ct - 8 * g8) - tl.tile0;       // (tile_from_index the other way round)
+  }
+  if (tt >= 0) {
+    const int g0 = (tt * tl.kp) / tl.share, g1 = ((tt + 1) * tl.kp - 1) / tl.share;
+    const float* src = tl.buf + (size_t)tt * 65536 + (j0 & 255) * 256 + (v & 255);
 #pragma unroll
-  for (int m = 0; m < 16; ++m) {
-    float sum = dwacc[(int64_t)(j0 + m) * Vp + v];
-    for (int q = 1; q < nparts; ++q) sum += dwacc[q * part_stride + (int64_t)(j0 + m) * Vp + v];   // fixed order
-    o[m] = sum * scale;
+    for (int m = 0; m < 16; ++m) o[m] = 0.f;
+    for (int g = g0; g <= g1; ++g) {                      // fixed order; the 16 loads of a piece are in flight together
+#pragma unroll
+      for (int m = 0; m < 16; ++m) o[m] += src[(size_t)g * 65536 + m * 256];
+    }
+#pragma unroll
+    for (int m = 0; m < 16; ++m) o[m] *= scale;
+  } else {
+#pragma unroll
+    for (int m = 0; m < 16; ++m) {
+      float sum = dwacc[(int64_t)(j0 + m) * Vp + v];
+      for (int q = 1; q < nparts; ++q) sum += dwacc[q * part_stride + (int64_t)(j0 + m) * Vp + v];   // fixed order
+      o[m] = sum * scale;
+    }
   }
   const int s0 = segoff[v], L = segoff[v + 1] - s0;
   if (L >= LONG_SEG) {
@@ -2149,6 +2221,7 @@ static int check_device(int dev) {
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
+      HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_tail_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dw_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
       void* sp = nullptr;
       HIP_TRY(hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)));       // this device's copy of the array
@@ -2186,6 +2259,27 @@ static size_t sort_tmp_bytes(int64_t N, int64_t V) {
 // fp32 partial sums of a K-split dX panel: at most 256 tiles of 256 x 256
 constexpr size_t DX_PART_BYTES = (size_t)256 * 256 * 256 * 4;
 
+// The last round of dW tiles, when it is far from full, is shared out along K among DW_TAIL_WGS workgroups
+// (bwd_dw_tail_kernel); each leaves its piece of a tile as a 256 x 256 fp32 partial.  A workgroup's range can end inside
+// one tile and go on in the next, so there are fewer pieces than workgroups plus tiles.
+constexpr int DW_TAIL_WGS = 256;
+struct DwTailPlan {
+  int full, ntail, kp, share;      // tiles in full rounds, tiles of the last round, pairs of K blocks per tile and per workgroup
+  bool use;                        // measured: worth it when the shared-out round is at most half a tile long per workgroup
+  size_t bytes;                    // partial tiles: one per (workgroup, tile it touches)
+};
+static DwTailPlan dw_tail_plan(int64_t dq, int64_t Vp, int64_t krows) {
+  DwTailPlan t;
+  const int tiles = (int)((dq / 256) * (Vp / 256));
+  t.kp = (int)(krows / BK / 2);
+  t.full = tiles / DW_TAIL_WGS * DW_TAIL_WGS;
+  t.ntail = tiles - t.full;
+  t.share = t.ntail > 0 ? (int)(((int64_t)t.ntail * t.kp + DW_TAIL_WGS - 1) / DW_TAIL_WGS) : 0;
+  t.use = t.ntail > 0 && t.share >= 1 && t.share * 2 <= t.kp;
+  t.bytes = t.use ? (size_t)(DW_TAIL_WGS + t.ntail) * 256 * 256 * 4 : 0;
+  return t;
+}
+
 // kept: the dlogits come with `saved` (the forward pass emitted them): no panel scratch here
 static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int nparts, int K, bool kept = false) {
   BwdLayout B;
@@ -2213,6 +2307,8 @@ static BwdLayout bwd_layout(const SavedLayout& S, int64_t P, int64_t Pw, int npa
   B.part_stride = ((size_t)S.dq * S.Vp * 4 + 255) / 256 * 256;
   B.off_dwacc = take(B.part_stride * (size_t)nparts);     // fp32 dW partials, one per dW launch
   B.total = o;
+  B.off_dwtail = o;
+  B.tail_bytes = S.Np <= Pw ? dw_tail_plan(S.dq, S.Vp, S.Np).bytes : 0;       // (one dW launch over all rows, or no K-split)
   return B;
 }
 
@@ -2308,9 +2404,12 @@ extern "C" int sce_sizes_for(const sce_shape* shape, sce_sizes* out) {
   out->bwd_panel_rows = default_panel(S);
   {
     const int64_t Pw = default_dw_panel(S, out->bwd_panel_rows);
-    out->bwd_workspace_bytes = bwd_layout(S, out->bwd_panel_rows, Pw, dw_launches(S, Pw), shape->n_predict).total;
+    // (both with room for the partial tiles of a K-split last round of dW, where there is to be one)
+    const BwdLayout Bd = bwd_layout(S, out->bwd_panel_rows, Pw, dw_launches(S, Pw), shape->n_predict);
+    out->bwd_workspace_bytes = Bd.total + Bd.tail_bytes;
     out->dlogits_bytes = S.g_total;
-    out->bwd_workspace_kept_bytes = bwd_layout(S, out->bwd_panel_rows, Pw, dw_launches(S, Pw), shape->n_predict, true).total;
+    const BwdLayout Bk = bwd_layout(S, out->bwd_panel_rows, Pw, dw_launches(S, Pw), shape->n_predict, true);
+    out->bwd_workspace_kept_bytes = Bk.total + Bk.tail_bytes;
   }
   out->saved_bf16_bytes = saved_layout(shape->N, shape->d, shape->V, shape->n_predict, 2).total;
   return SCE_OK;
@@ -2657,6 +2756,8 @@ extern "C" int sce_backward(const sce_args* a) {
   const float k1 = (float)a->x_s * (float)a->w_s * 2.0f * LOG2E / a->cap, c2 = -2.0f * a->cap * LOG2E;
   const int CTv = (int)(S.Vp / 256), CTd = (int)(S.dq / 256);
   int launch = 0;
+  DwTail tail;
+  tail.buf = nullptr; tail.tile0 = -1; tail.ntail = 0; tail.kp = 1; tail.share = 1;
   int64_t w0 = 0;                      // first row of the rows gathered for the next dW launch
   for (int64_t p0 = 0; p0 < S.Np; p0 += P) {
     const int64_t prow = (S.Np - p0 < P) ? (S.Np - p0) : P;     // multiple of 256
@@ -2713,7 +2814,16 @@ extern "C" int sce_backward(const sce_args* a) {
       wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(gathered / BK);
       {
         KernelTimer tm(SCE_K_DW, st);
-        if (launch >= nparts) bwd_dw_kernel<true><<<map_tile_rr_grid(CTd, CTv), NTHREADS, smem_scaled(wp.KT, 0), st>>>(wp);
+        // When this launch is the only one and its last round of tiles would leave many CUs idle, that round is
+        // shared out along K instead (bwd_dw_tail_kernel): the full rounds run as they are.
+        const DwTailPlan tp = dw_tail_plan(S.dq, S.Vp, gathered);
+        const bool only = w0 == 0 && p0 + prow >= S.Np && launch == 0;
+        if (only && tp.use && B.tail_bytes >= tp.bytes && a->workspace_bytes >= B.off_dwtail + tp.bytes) {
+          const int full = tp.full;
+          tail.buf = (float*)(ws + B.off_dwtail); tail.tile0 = tp.full; tail.ntail = tp.ntail; tail.kp = tp.kp; tail.share = tp.share;
+          if (full > 0) bwd_dw_kernel<false><<<full, NTHREADS, smem_scaled(wp.KT, 0), st>>>(wp);
+          bwd_dw_tail_kernel<<<DW_TAIL_WGS, NTHREADS, smem_scaled(2 * tp.share, 0), st>>>(wp, tail);
+        } else if (launch >= nparts) bwd_dw_kernel<true><<<map_tile_rr_grid(CTd, CTv), NTHREADS, smem_scaled(wp.KT, 0), st>>>(wp);
         else bwd_dw_kernel<false><<<map_tile_rr_grid(CTd, CTv), NTHREADS, smem_scaled(wp.KT, 0), st>>>(wp);
       }
       ++launch;
@@ -2735,10 +2845,10 @@ extern "C" int sce_backward(const sce_args* a) {
     dim3 g((unsigned)((V + 63) / 64), (unsigned)((d + 63) / 64));
     if (a->dw_dtype == SCE_F32)
       bwd_dw_final_kernel<float><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, longbase, S.dq, (float)a->x_s, dcp, (int)d, (int)V,
-                                                   (float*)a->dw, a->dw_ld);
+                                                   (float*)a->dw, a->dw_ld, tail, CTd, CTv);
     else
       bwd_dw_final_kernel<bf16_t><<<g, 256, 0, st>>>(dwacc, launch < nparts ? launch : nparts, (int64_t)(B.part_stride / 4), S.Vp, segoff, perm, hcoef, xq, S.ldx, (int)S.Np, xi, longsum, longbase, S.dq, (float)a->x_s, dcp, (int)d, (int)V,
-                                                    (bf16_t*)a->dw, a->dw_ld);
+                                                    (bf16_t*)a->dw, a->dw_ld, tail, CTd, CTv);
   }
   HIP_TRY(hipGetLastError());
   return SCE_OK;

@@ -490,3 +490,25 @@ def test_bf16_operands_are_forward_only():
     assert torch.isfinite(loss)
     with pytest.raises(ValueError, match="forward-only"):
         ck.ce_forward(x, w, y, 1.0, 1.0, inp.cap, "mean", operand_dtype=torch.bfloat16, keep_dlogits=True)
+
+
+@pytest.mark.parametrize("N,d,V", [(2048, 512, 6000), (1024, 1024, 50304), (700, 272, 2049)])
+def test_dw_with_and_without_the_k_split_last_round(N, d, V):
+    """With room in the workspace a last round of dW tiles that is far from full is shared out along K (here: all of
+    the tiles, there being fewer than CUs); without it every tile has one workgroup.  Same sums, in a different order."""
+    from slowrun_amd import _lib, cuda_kernels as ck
+    inp = _small("tiny_track", N, d, V)
+    x, w, y = inp.x.cuda(), inp.w.cuda(), inp.targets.cuda()
+    sz = _lib.sizes_for(N, d, V)
+    out, saved, lse, _, _ = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, "mean", keep_dlogits=True)
+    go = torch.ones((), device="cuda")
+    args = (saved, y, go, N, d, V, inp.x_s, inp.w_s, inp.cap, 1.0, "mean", torch.float32, torch.float32)
+    dx1, dw1 = ck.ce_backward(*args, keep_dlogits=True)
+    # the same workspace without the room for the partial tiles: they lie at its end, one 256 x 256 fp32 tile for
+    # each of the 256 workgroups and one more for each tile of the shared-out round
+    tiles = -(-d // 256) * -(-V // 256)
+    small = sz.bwd_workspace_kept_bytes - (256 + tiles % 256) * 256 * 256 * 4
+    dx2, dw2 = ck.ce_backward(*args, keep_dlogits=True, workspace_bytes=small)
+    torch.cuda.synchronize()
+    assert torch.equal(dx1, dx2)
+    assert pu.maxrel(dw1, dw2) < 2e-6
