@@ -57,7 +57,8 @@ typedef struct sce_sizes {
   size_t wcache_bytes;       /* size of that weight cache                                    */
   size_t fwd_workspace_bytes;
   size_t bwd_workspace_min_bytes;   /* backward with the smallest row panel (256 rows)       */
-  size_t bwd_workspace_bytes;       /* backward with the default row panel                   */
+  size_t bwd_workspace_bytes;       /* backward with the default row panel (with room for the partial tiles of a
+                                       K-split last round of dW where there is to be one; less is accepted)   */
   int64_t bwd_panel_rows;           /* the default row panel                                 */
   /* with sce_args.dlogits_from_forward: */
   size_t dlogits_bytes;             /* `saved` grows by this much (N x V bytes and a little)  */

@@ -6,14 +6,16 @@
 //
 // Data flow
 //   forward : X, W --quantise--> X_q [Np][dp], W_q^T [Vp][dp], W_q [dq][Vp]   (OCP e4m3, zero padded)
-//             fwd_kernel: 256x256 logit tiles on v_mfma_f32_32x32x64_f8f6f4, epilogue keeps
-//             per-row sum exp(z - cap), max/argmax of u and the target logit in registers;
-//             the logits never leave the chip.  Partials per (row, V-split) -> combine.
-//   backward: per panel of P rows: recompute the logit tiles, turn them in registers into
-//             G = 256 * (1 - t^2) * exp(z - zmax_row) (e4m3), written once row-major and once
-//             transposed into a panel-sized scratch; dX = rho_row * G W_q^T and
-//             dW += (rho X_q)^T G run on the same MFMA main loop.  The one-hot part of
-//             dlogits never goes through fp8: it is applied in fp32 in the dX epilogue
+//             fwd_kernel: 256x256 logit tiles on v_mfma_f32_32x32x64_f8f6f4; the epilogue keeps per-row
+//             sum exp(z - cap), the target logits and (on request) max/argmax of u; the logits never leave
+//             the chip.  With dlogits_from_forward it also leaves D = (1 - t^2) exp(z - cap) as e4m3 bytes
+//             with one power-of-two exponent per 32 rows x 128 columns (G^T, tile by tile), the targets'
+//             entries zero.  Partials per (row, V-split) -> combine.  (fwd_pp_kernel: the same from 256x128
+//             tiles with two waves per SIMD; opt-in.)
+//   backward: the dlogits as forward left them, or formed again panel by panel from recomputed logit tiles
+//             (bwd_recompute_kernel, same format); dX = rho_row * D W_q^T and dW = (rho X_q)^T D run on the
+//             same MFMA main loop with the exponents applied inside v_mfma_scale_f32_32x32x64_f8f6f4.  The
+//             one-hot part of dlogits never goes through fp8: it is applied in fp32 in the dX epilogue
 //             (gather of W_q^T rows) and in the dW finalisation (rows grouped by target).
 #include "sce_common.h"
 #include "sce_mainloop.h"
