@@ -232,6 +232,12 @@ int sce_bench_mfma(const void* random_bytes, int32_t iters, int32_t reps, void* 
                    void* stream, double* tflops, double* shader_mhz);
 int sce_bench_gemm(const void* A, const void* B, int64_t M, int64_t N, int64_t K, int32_t reps, void* scratch, size_t scratch_bytes,
                    int32_t device, void* stream, double* tflops, double* shader_mhz);
+/*  sce_bench_pingpong: the same product through the ping-pong walk of the opt-in forward kernel (256 x 128 tiles, two waves
+ *                  per SIMD that take turns accumulating), with a synthetic epilogue: valu_copies (0..3) times the
+ *                  transcendental and conversion work of the dlogits epilogue per value, 0 = only a sum.  Returns the
+ *                  time of one launch in ms.  scratch: 2 KiB per 256 rows of B times 8, rounded up to 8 workgroups. */
+int sce_bench_pingpong(const void* A, const void* B, int64_t M, int64_t N, int64_t K, int32_t valu_copies, int32_t reps, void* scratch,
+                       size_t scratch_bytes, int32_t device, void* stream, double* ms_per_launch);
 
 #ifdef __cplusplus
 }
