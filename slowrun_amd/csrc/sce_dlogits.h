@@ -1,0 +1,177 @@
+// The block-scaled e4m3 format of the stored dlogits and the epilogue that forms it from a finished logit tile
+// (shared by the forward kernel and the recompute kernel; internal header).
+// Part of the one translation unit sce_kernels.hip, which includes it after the headers it builds on.
+#pragma once
+
+namespace sce {
+
+// ------------------------------------------------------------------------------------------
+// dlogits on chip
+// ------------------------------------------------------------------------------------------
+// The softmax part of dlogits, without the factors that belong to a whole row, is
+//   D_iv = (1 - t^2) e^{z - cap} = 4 r (1 - r) e^{z - cap},  r = 1 / (1 + e^{2u/cap}),   0 <= D <= 1,
+// and  du_iv = rho_i D_iv - (one-hot terms),  rho_i = g_i S_i e^{cap - lse_i}.  D is kept in e4m3 with one power-of-two
+// exponent per block of 32 rows i x 128 columns v (MX style: byte * 2^(E - 127), E in an E8M0 byte), taken from the
+// block's own largest logit, so that neither the row's final lse nor its maximum has to be known when the block is
+// formed -- the forward pass can emit it -- and a peak in one place of a row costs the rest of the row nothing.  The
+// dX and dW GEMMs apply the exponents inside the matrix instruction (mfma_mainloop, SCALE).
+// Rows of very different temperature may share a block (a row whose logits saturate the cap next to ordinary ones:
+// D near 0.05 next to D near e^{-cap}), and 8 bits cannot hold both at one exponent.  So each row also has a boost of
+// its own, D_iv 2^{lam_i} is what is stored, with lam_i an integer estimated before the forward pass from a sample of
+// the row's logits (fwd_sample_kernel) and undone exactly in rho_i.  The block exponent is taken after the boost, so
+// a poor estimate costs precision, never range.
+//
+// Layout: G^T, tile by tile ([v tile][K block of 128 rows i][256 v][128 i] bytes): the B operand of dW as it lies,
+// and of dX through the transposing LDS read.  Exponents: one dword per (128 v, 128 i), byte c for rows [32 c, 32 c + 32),
+// as gexp[v / 128][i / 128].
+//
+// One wave turns its 128 (v) x 128 (i) quadrant of a finished logit tile into its quadrant of the staging tile TT
+// ([256 v][STG_PITCH], rows i contiguous) in LDS and returns the dword of exponents of its four 32-row blocks.  The
+// transposition happens in registers: the four lanes of a quad hold four consecutive rows of the same four
+// columns, and two quad-permute + byte-permute steps turn that 4 x 4 byte block around.
+// STATS: the forward pass's row statistics as well (sum of e^{z - cap}, largest raw logit and its column), kept in
+// `stat` (LDS, 12 floats per lane: [sum, max, argmax][4 row blocks], NTHREADS apart).
+constexpr int STG_PITCH = 272;                               // 256 + 16: 16-byte aligned, rows shifted by 4 banks
+constexpr int STG_BYTES = 256 * STG_PITCH;                   // 69632
+
+// Maximum over the 64 lanes, in every lane.  The lane exchanges are LDS-crossbar swizzles with the pattern in the
+// instruction (xor 1 .. 16 within a half-wave), and one ds_bpermute across the halves whose address comes from
+// lane_id(): __shfl_xor would keep its own copy of the lane index alive across the main loop, where it is spilled.
+__device__ __forceinline__ float wave_max(float v) {
+#define SCE_SWZ_MAX(X) v = fmaxf(v, __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), ((X) << 10) | 0x1f)))
+  SCE_SWZ_MAX(1); SCE_SWZ_MAX(2); SCE_SWZ_MAX(4); SCE_SWZ_MAX(8); SCE_SWZ_MAX(16);
+#undef SCE_SWZ_MAX
+  return fmaxf(v, __int_as_float(__builtin_amdgcn_ds_bpermute((lane_id() ^ 32) << 2, __float_as_int(v))));
+}
+
+// The same without the LDS crossbar (whose operations queue behind the fragment reads of the other wave of the SIMD in
+// the ping-pong kernel): four DPP steps leave the maximum of each row of 16 lanes in all of its lanes, the four rows
+// meet through scalar registers.
+__device__ __forceinline__ float wave_max_dpp(float v) {
+#define SCE_DPP_MAX(CTRL) v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xF, 0xF, false)))
+  SCE_DPP_MAX(0xB1);      // quad_perm [1, 0, 3, 2]
+  SCE_DPP_MAX(0x4E);      // quad_perm [2, 3, 0, 1]
+  SCE_DPP_MAX(0x141);     // row_half_mirror
+  SCE_DPP_MAX(0x140);     // row_mirror
+#undef SCE_DPP_MAX
+  const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0)), r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32)), r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
+// lam (LDS, wave-uniform base; per row block LAM_STRIDE floats apart, one float for each of LAM_LANES lanes): the row's
+// exponent boost (see fwd_sample_kernel).
+// want_argmax (uniform, STATS only): see the lookup of the maximum's column below.
+template <bool EDGE, bool STATS, int LAM_STRIDE = NTHREADS, int LAM_LANES = 64>
+__device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float k1, float c2, int vlim, int vabs0,
+                                                 uint8_t* TT, int wa, int wb, float* stat, const float* lam, bool want_argmax = true) {
+  const int lane = lane_id();
+  const int vloc0 = wa * 128 + 4 * (lane >> 5);       // column (within the tile) of accumulator register 0 of block a = 0
+  const int k = lane & 3;
+  const uint32_t sel1 = (k & 1) ? 0x03070105u : 0x06020400u;
+  const uint32_t sel2 = (k & 2) ? 0x03020706u : 0x05040100u;
+  uint32_t expword = 0;
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int iloc = wb * 128 + b * 32 + (lane & 31);        // row within the tile
+    // the block's largest logit fixes its exponent: D * 2^s <= 2^(lg + s) <= 446 with lg = log2 e^{zmax - cap}
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float x = acc[a][b][r];
+        if (EDGE && vloc0 + a * 32 + 8 * (r >> 2) + (r & 3) >= vlim) x = -INFINITY;
+        tmax = fmaxf(tmax, x);
+      }
+    const float lamb = lam[b * LAM_STRIDE + (lane_id() & (LAM_LANES - 1))];      // (index taken anew: see lane_id)
+    const float lg = wave_max_dpp(fmaf(c2, fast_rcp(1.0f + fast_exp2(tmax * k1)), lamb));      // over the block: log2 of the largest boosted e^{z - cap}
+    const float sb = floorf(8.8f - lg);                       // between -120 and 8 + 2 cap log2(e) <= 124 (cap <= 40, boost <= 120)
+    const float cs = sb + 2.0f + lamb;                        // the 4 of 4 r (1 - r) and the row's boost ride along
+    expword |= (uint32_t)(127 - (int)sb) << (8 * b);
+    float ssum = 0.f;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      // stage by stage over the 16 values of the block: the transcendental unit is pipelined, a chain
+      // of dependent exp2 / rcp / exp2 on one value at a time is not (the scheduler would rebuild the
+      // chains to save registers, hence the barriers)
+      constexpr int NB = 8;        // values per batch: 4, 8 and 16 measure alike
+      float rr[16], gg[16];
+#pragma unroll
+      for (int g0 = 0; g0 < 16; g0 += NB) {
+#pragma unroll
+        for (int m = g0; m < g0 + NB; ++m) rr[m] = fast_exp2(acc[a][b][m] * k1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = g0; m < g0 + NB; ++m) rr[m] = fast_rcp(rr[m] + 1.0f);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = g0; m < g0 + NB; ++m) gg[m] = fast_exp2(fmaf(c2, rr[m], cs));
+        __builtin_amdgcn_sched_barrier(0);
+        if (EDGE) {
+#pragma unroll
+          for (int m = g0; m < g0 + NB; ++m) gg[m] = (vloc0 + a * 32 + 8 * (m >> 2) + (m & 3) >= vlim) ? 0.f : gg[m];
+        }
+        if (STATS) {
+#pragma unroll
+          for (int m = g0; m < g0 + NB; ++m) ssum += gg[m];
+        }
+#pragma unroll
+        for (int m = g0; m < g0 + NB; ++m) gg[m] *= rr[m] - rr[m] * rr[m];
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int vloc = vloc0 + a * 32 + 8 * q;
+        const uint32_t w = cvt4_e4m3(gg[4 * q], gg[4 * q + 1], gg[4 * q + 2], gg[4 * q + 3]);
+        // 4 x 4 byte transpose inside the quad: lane k ends up with column vloc + k, rows (iloc & ~3) .. +3
+        const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xB1, 0xF, 0xF, true);     // lane ^ 1
+        const uint32_t x = __builtin_amdgcn_perm(p1, w, sel1);
+        const uint32_t p2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, true);     // lane ^ 2
+        const uint32_t yv = __builtin_amdgcn_perm(p2, x, sel2);
+        *reinterpret_cast<uint32_t*>(TT + (vloc + k) * STG_PITCH + (iloc & ~3)) = yv;
+      }
+    }
+    if (STATS) {
+      stat[(0 + b) * NTHREADS] += ssum * fast_exp2(-cs);
+      const float amax = stat[(4 + b) * NTHREADS];
+      // The column of the maximum is looked up only when a tile reaches a lane's running maximum (on a tie the lower
+      // column wins: the running one may be a target of this very tile, which take_target_logits has put there) -- which
+      // some lane of the 64 does in nearly every tile of a walk of a few dozen: a caller that does not ask for the argmax
+      // is spared it.  (A flag at run time, not a template parameter: without the lookup in the code the register
+      // allocation of the rest changes, and accumulators end up in scratch memory.)
+      if (want_argmax && __builtin_amdgcn_ballot_w64(tmax >= amax) != 0) {
+        if (tmax >= amax) {
+          int targ = 0x7fffffff;
+#pragma unroll
+          for (int a = 3; a >= 0; --a) {
+#pragma unroll
+            for (int r = 15; r >= 0; --r) {
+              const int vo = a * 32 + 8 * (r >> 2) + (r & 3);
+              if (acc[a][b][r] == tmax && (!EDGE || vloc0 + vo < vlim)) targ = vo;   // descending scan: lowest column wins
+            }
+          }
+          if (tmax > amax || (targ != 0x7fffffff && vabs0 + targ < __float_as_int(stat[(8 + b) * NTHREADS]))) {
+            stat[(4 + b) * NTHREADS] = tmax;
+            stat[(8 + b) * NTHREADS] = __int_as_float(vabs0 + targ);
+          }
+        }
+      }
+    }
+  }
+  return expword;
+}
+
+// The wave's quadrant of the staging tile (128 columns v x 128 rows i) is one contiguous 16 KB run of G^T: out in
+// 16-byte stores.  A wave reads only what it wrote itself, so no barrier is needed between forming and storing.
+__device__ __forceinline__ void store_dlogits_quadrant(const uint8_t* TT, uint8_t* gcol, int wa, int wb) {
+  const int lane = lane_id();
+  const uint8_t* tq = TT + wa * 128 * STG_PITCH + wb * 128;
+#pragma unroll
+  for (int n = 0; n < 16; ++n) {
+    const int cidx = lane + 64 * n, row = cidx >> 3, col = (cidx & 7) * 16;
+    *reinterpret_cast<v4i*>(gcol + row * BK + col) = *reinterpret_cast<const v4i*>(tq + row * STG_PITCH + col);
+  }
+}
+
+}  // namespace sce

@@ -1,0 +1,315 @@
+// Forward kernels: row-boost sample, the logit-tile walk with its epilogues, combination of the vocabulary splits,
+// mean reduction (internal header).
+// Part of the one translation unit sce_kernels.hip, which includes it after the headers it builds on.
+#pragma once
+
+namespace sce {
+
+// ------------------------------------------------------------------------------------------
+// forward
+// ------------------------------------------------------------------------------------------
+struct FwdParams {
+  const uint8_t* xq;       // [Np][dp]
+  const uint8_t* wqt;      // [Vp][dp]
+  float4* partials;        // [S][Np]: sum exp(z - cap), max u, argmax u (bits), unused
+  const int64_t* targets;  // (N,)
+  float* s_uy;             // [n_predict][Np]: raw logit u at the target of (offset, row), written by the workgroup that meets it
+  uint8_t* ghat_t;         // EMIT: G^T, all Np rows (K blocks per v tile: kbw)
+  uint32_t* gexp;          // EMIT: its block exponents [Vp / 128][kbw]
+  const float* lam;        // EMIT: exponent boost of every row
+  int64_t ignore_index;
+  int64_t dp, ldx;         // K extent and row stride of xq / wqt
+  int64_t kbw;
+  int N, V, Np, RT, CT, S, n_predict;      // V: columns that take part; CT: column tiles walked (EMIT: all of Vp / 256)
+  float sc;                // x_s * w_s
+  float k1;                // x_s * w_s * 2 log2(e) / cap : exp2(acc * k1) = e^{2u/cap}
+  float ic2;               // 1 / c2, c2 = -2 cap log2(e): e^{z - cap} = exp2(c2 / (1 + e^{2u/cap}))
+  float c2;
+  const DevConsts* dc;     // non-NULL: sc and k1 come from here (a scale lives on the device)
+  int want_argmax;         // the caller asks for the rows' argmax: the column of the running maximum is tracked
+};
+
+// Per 256 x 256 tile and per row a lane owns: add up e^{z - cap} over its 64 columns and keep the
+// largest raw accumulator.  z is bounded by +-cap, so no running maximum is needed for the sum:
+//   t = tanh(u/cap) = 1 - 2/(E + 1), E = e^{2u/cap};   e^{z - cap} = exp2(c2 / (E + 1)).
+// The column of the maximum is looked up only on the (rare, after the first tiles) occasion that
+// a tile raises a row's running maximum.
+// ROUND: the logits are rounded to bf16 first (bf16 operands: the GEMM of the eager head returns bf16).
+template <bool EDGE, bool ROUND = false>
+__device__ __forceinline__ void fwd_epilogue(const v16f (&acc)[4][4], const FwdParams& p, int vbase,
+                                             float (&sum)[4], float (&amax)[4], int (&uarg)[4]) {
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    float tmax = -INFINITY, s = 0.f;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int vo = a * 32 + 8 * (r >> 2) + (r & 3);
+        float x = ROUND ? round_to_bf16(acc[a][b][r]) : acc[a][b][r];
+        // z - cap = c2 / (1 + e^{2u/cap}) in units of log2: the reciprocal of (1 + e) / c2 gives it in one step
+        float pt = fast_exp2(fast_rcp(fmaf(fast_exp2(x * p.k1), p.ic2, p.ic2)));
+        if (EDGE) {
+          if (vo >= p.V - vbase) { pt = 0.f; x = -INFINITY; }
+        }
+        s += pt;
+        tmax = fmaxf(tmax, x);
+      }
+    }
+    sum[b] += s;
+    if (p.want_argmax && __builtin_amdgcn_ballot_w64(tmax > amax[b]) != 0) {
+      if (tmax > amax[b]) {
+        int targ = 0x7fffffff;
+#pragma unroll
+        for (int a = 3; a >= 0; --a) {
+#pragma unroll
+          for (int r = 15; r >= 0; --r) {
+            const int vo = a * 32 + 8 * (r >> 2) + (r & 3);
+            if ((ROUND ? round_to_bf16(acc[a][b][r]) : acc[a][b][r]) == tmax && (!EDGE || vo < p.V - vbase)) targ = vo;   // descending scan: lowest column wins
+          }
+        }
+        amax[b] = tmax;
+        uarg[b] = vbase + targ;
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ bool target_valid(const int64_t* __restrict__ targets, int64_t ignore_index, int i, int N, int V) {
+  if (i >= N) return false;
+  const int64_t y = targets[i];
+  return (y != ignore_index) && y >= 0 && y < V;
+}
+
+// The raw logit at a row's targets, taken from the accumulators of the tile that holds the target column, so that z_y
+// and lse come from the same numbers: the fp8 matrix instruction sums with less than fp32 care (about 2e-5 low on a
+// sum of like-signed terms), and a z_y from a separate fp32 dot product would leave that bias in z_y - lse, i.e. in
+// 1 - p_y, where rows the model is sure of cannot afford it.  tgt (LDS): [4 offsets][TGT_STRIDE rows] target column or
+// -1, already at the wave's first row.  A lane looks at its four rows; the 64-way select runs only when some lane of
+// the wave has a hit (a few per cent of the tiles).
+// STORE: the logit goes to s_uy_tile[offset][row] (global).
+// KNOCK: the accumulator of the target is then set to -inf, for the dlogits epilogue that follows: the target takes
+//        no part in the stored dlogits (its column is handled in fp32, see bwd_prep_kernel) and must not set the
+//        exponent of its block either -- a row the model is sure of would push its own other columns, and its
+//        neighbours', out of the 8 bits.
+// STATS: with KNOCK, the row statistics (stat, as in form_dlogits) take the target's share here: e^{z_y - cap} into the
+//        sum, and the running maximum / argmax.
+template <bool STORE, bool KNOCK, bool STATS, int TGT_STRIDE, bool ROUND = false>
+__device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int* tgt, int n_predict, int col0, int rowbase,
+                                                   float sc, float* s_uy_tile, int Np, float* stat, float k1, float ic2) {
+  const int lane = lane_id(), half = lane >> 5;
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int row = b * 32 + (lane & 31);
+    float xk[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < n_predict; ++k) {
+      const int y = tgt[k * TGT_STRIDE + row];
+      const int rel = y - col0;                        // column within the wave's 128
+      const bool hit = (unsigned)rel < 128u && ((rel >> 2) & 1) == half;
+      if (__builtin_amdgcn_ballot_w64(hit) != 0) {
+        if (hit) {
+          const int idx = (rel >> 5) * 16 + ((rel >> 3) & 3) * 4 + (rel & 3);
+          float x = 0.f;
+          bool again = false;                          // an earlier offset of this row has the same target
+          if (KNOCK) {
+            for (int k2 = 0; k2 < k; ++k2)
+              if (tgt[k2 * TGT_STRIDE + row] == y) { again = true; x = xk[k2]; }
+          }
+          if (!again) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+              for (int r = 0; r < 16; ++r) {
+                x = (idx == a * 16 + r) ? acc[a][b][r] : x;
+                if (KNOCK) acc[a][b][r] = (idx == a * 16 + r) ? -INFINITY : acc[a][b][r];
+              }
+            if (KNOCK && STATS) {
+              // (the -inf left behind reads as z = -cap to the epilogue that follows, which will add e^{-2 cap} for it)
+              stat[(0 + b) * NTHREADS] += fast_exp2(fast_rcp(fmaf(fast_exp2(x * k1), ic2, ic2))) - fast_exp2(fast_rcp(ic2));
+              const float amax = stat[(4 + b) * NTHREADS];
+              if (x > amax || (x == amax && y < __float_as_int(stat[(8 + b) * NTHREADS]))) {
+                stat[(4 + b) * NTHREADS] = x;
+                stat[(8 + b) * NTHREADS] = __int_as_float(y);
+              }
+            }
+          }
+          xk[k] = x;
+          // (the lane index is taken anew: an address kept from outside the branch stays live across the main loop and is spilled)
+          if (STORE) s_uy_tile[(int64_t)k * Np + rowbase + b * 32 + (lane_id() & 31)] = ROUND ? round_to_bf16(x) * sc : x * sc;
+        }
+      }
+    }
+  }
+}
+
+// The exponent boost of every row, from one tile of its logits (256 columns from the middle of the vocabulary):
+// lam_i = floor(-log2 m_i), m_i the smallest of the means of e^{z - cap} over 16 groups of 16 columns -- the smallest,
+// so that a few peaks inside the sample (a target, say) do not pass for the level of the row.  One workgroup per row tile.
+__global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct, float* __restrict__ lam_out) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  FwdParams p = p_in;
+  if (p.dc) { p.sc = p.dc->sc; p.k1 = p.dc->k1; }
+  const int rt = blockIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wa = wave >> 1, wb = wave & 1;
+  v16f acc[4][4];
+  mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 0, 0, wave);
+  const int lane = lane_id();
+  const int vlim = p.V - ct * 256, vloc0 = wa * 128 + 4 * (lane >> 5);
+  float gmin[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    gmin[b] = INFINITY;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      float sum = 0.f, cnt = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float pt = fast_exp2(fast_rcp(fmaf(fast_exp2(acc[a][b][r] * p.k1), p.ic2, p.ic2)));
+        const bool live = vloc0 + a * 32 + 8 * (r >> 2) + (r & 3) < vlim;
+        sum += live ? pt : 0.f;
+        cnt += live ? 1.f : 0.f;
+      }
+      if (cnt > 0.f) gmin[b] = fminf(gmin[b], sum / cnt);
+    }
+    gmin[b] = fminf(gmin[b], __shfl_xor(gmin[b], 32));
+  }
+  float* red = reinterpret_cast<float*>(smem);          // free: the main loop has ended in every wave
+  if (wa == 1 && lane < 32) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) red[wb * 128 + b * 32 + lane] = gmin[b];
+  }
+  __syncthreads();
+  if (wa == 0 && lane < 32) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const float m = fminf(gmin[b], red[wb * 128 + b * 32 + lane]);
+      float l = floorf(-log2f(m));
+      l = l > 0.f ? (l < 120.f ? l : 120.f) : 0.f;           // also: NaN -> 0
+      lam_out[rt * 256 + wb * 128 + b * 32 + lane] = l;
+    }
+  }
+}
+
+// LDS of the forward kernel: the two K slots; with EMIT the staging tile of the dlogits in the second slot (reaching
+// 4 KB beyond it); the row statistics of the workgroup's walk (12 values per lane, and the boosts of its rows: kept in registers they are spilled
+// around the main loop, and the reload -- a vector memory load -- makes the epilogue wait for the tile loads that were
+// just put in flight for the next tile); the targets of the workgroup's 256 rows.
+constexpr int FWD_STAGE_OFF = SLOT_BYTES;
+constexpr int FWD_STAT_OFF = SMEM_MAX - 4096 - 16 * 4 * NTHREADS;      // 12 statistics and the boosts of the lane's 4 rows
+constexpr int FWD_TGT_OFF = SMEM_MAX - 4096;
+constexpr int SMEM_FWD = SMEM_MAX;
+static_assert(FWD_STAGE_OFF + STG_BYTES <= FWD_STAT_OFF, "staging tile and row statistics overlap");
+
+// EMIT: the epilogue also leaves the block-scaled dlogits of the tile in G^T (see form_dlogits), for a backward pass
+// that does not compute the logits again.
+// BF16 (without EMIT): bf16 operands, logits rounded to bf16 as the eager head's GEMM returns them (forward only).
+template <bool EMIT, bool BF16 = false>
+__global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  FwdParams p = p_in;
+  if (p.dc) { p.sc = p.dc->sc; p.k1 = p.dc->k1; }
+  int rt, s;
+  if (!map_tile(blockIdx.x, p.RT, p.S, rt, s)) return;
+  const int ct0 = (int)((int64_t)p.CT * s / p.S), ct1 = (int)((int64_t)p.CT * (s + 1) / p.S);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wa = wave >> 1, wb = wave & 1;
+  {
+    float* stat = reinterpret_cast<float*>(smem + FWD_STAT_OFF) + wave * 64 + lane_id();   // [12][256]: sum, amax, uarg of the 4 row blocks
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      stat[(0 + b) * NTHREADS] = 0.f;
+      stat[(4 + b) * NTHREADS] = -INFINITY;
+      stat[(8 + b) * NTHREADS] = __int_as_float(0x7fffffff);
+      if (EMIT) stat[(12 + b) * NTHREADS] = p.lam[rt * 256 + wb * 128 + b * 32 + (lane_id() & 31)];
+    }
+    int* tgt = reinterpret_cast<int*>(smem + FWD_TGT_OFF);
+    for (int e = threadIdx.x; e < p.n_predict * 256; e += NTHREADS) {
+      const int i = rt * 256 + (e & 255) + (e >> 8);
+      tgt[e] = ((e & 255) + rt * 256 < p.N && target_valid(p.targets, p.ignore_index, i, p.N, p.V)) ? (int)p.targets[i] : -1;
+    }
+  }
+  __syncthreads();
+  v16f acc[4][4];
+  const uint8_t* Bg = p.xq + (int64_t)rt * 256 * p.ldx;
+  const int KT = (int)(p.dp / BK);
+  // of the workgroups that start together on this XCD, those with the same split share the W tiles, those with the same rt the X rows
+  const int rot_a = 2 * (rt & 3), rot_b = s & 7;
+  // the first K blocks of the next tile travel while the epilogue of this one runs (it does not touch the K slots;
+  // with EMIT it uses the second one, so only the first block travels and the rest follows after the epilogue)
+  if (ct0 < ct1) mfma_prefetch(p.wqt + (int64_t)ct0 * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
+  for (int ct = ct0; ct < ct1; ++ct) {
+    mfma_mainloop<true, NoHook, BK, false, 0, BF16>(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, Bg, p.ldx, KT, smem, acc, rot_a, rot_b, wave,
+                                                    NoHook(), 0, 0, nullptr, EMIT && ct > ct0);
+    const uint8_t* Anext = p.wqt + (int64_t)(ct + 1) * 256 * p.ldx;
+    if (ct + 1 < ct1) mfma_prefetch<EMIT ? 1 : 3>(Anext, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
+    float* stat = reinterpret_cast<float*>(smem + FWD_STAT_OFF) + wave * 64 + lane_id();
+    const int vbase = ct * 256 + wa * 128 + 4 * (lane_id() >> 5);
+    const int* tgt = reinterpret_cast<const int*>(smem + FWD_TGT_OFF) + wb * 128;
+    if (EMIT) {
+      take_target_logits<true, true, true, 256>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2);
+      const int vlim = p.V - ct * 256;
+      uint8_t* TT = smem + FWD_STAGE_OFF;
+      uint32_t ew;
+      const float* lam = reinterpret_cast<const float*>(smem + FWD_STAT_OFF) + 12 * NTHREADS + wave * 64;
+      if (vlim < 256) ew = form_dlogits<true, true>(acc, p.k1, p.c2, vlim, vbase, TT, wa, wb, stat, lam, p.want_argmax != 0);
+      else ew = form_dlogits<false, true>(acc, p.k1, p.c2, vlim, vbase, TT, wa, wb, stat, lam, p.want_argmax != 0);
+      store_dlogits_quadrant(TT, p.ghat_t + ((int64_t)ct * p.kbw + 2 * rt + wb) * BLOCKED_KSTEP + wa * 128 * BK, wa, wb);
+      if (lane_id() == 0) p.gexp[(int64_t)(2 * ct + wa) * p.kbw + 2 * rt + wb] = ew;
+    } else {
+      float sum[4], amax[4];
+      int uarg[4];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        sum[b] = stat[(0 + b) * NTHREADS]; amax[b] = stat[(4 + b) * NTHREADS]; uarg[b] = __float_as_int(stat[(8 + b) * NTHREADS]);
+      }
+      if (ct * 256 + 256 > p.V) fwd_epilogue<true, BF16>(acc, p, vbase, sum, amax, uarg);
+      else fwd_epilogue<false, BF16>(acc, p, vbase, sum, amax, uarg);
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        stat[(0 + b) * NTHREADS] = sum[b]; stat[(4 + b) * NTHREADS] = amax[b]; stat[(8 + b) * NTHREADS] = __int_as_float(uarg[b]);
+      }
+    }
+    if (!EMIT) take_target_logits<true, false, false, 256, BF16>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, nullptr, 0.f, 0.f);
+    if (EMIT && ct + 1 < ct1) {
+      // every wave has read its part of the staging tile (its stores have their data) before the second K slot fills again
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      mfma_prefetch<2>(Anext, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
+    }
+  }
+  if (EMIT) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");     // the staging tile gives way to the reduction below
+  float sum[4], amax[4];
+  int uarg[4];
+  const int lane = lane_id();
+  float* stat = reinterpret_cast<float*>(smem + FWD_STAT_OFF) + wave * 64 + lane;
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    sum[b] = stat[(0 + b) * NTHREADS]; amax[b] = stat[(4 + b) * NTHREADS]; uarg[b] = __float_as_int(stat[(8 + b) * NTHREADS]);
+  }
+  // the two half-waves hold different columns of the same rows
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const float s2 = __shfl_xor(sum[b], 32), um2 = __shfl_xor(amax[b], 32);
+    const int ua2 = __shfl_xor(uarg[b], 32);
+    sum[b] += s2;
+    if (um2 > amax[b] || (um2 == amax[b] && ua2 < uarg[b])) { amax[b] = um2; uarg[b] = ua2; }
+  }
+  // waves wa = 0 and wa = 1 hold different columns of the same rows
+  float4* red = reinterpret_cast<float4*>(smem);
+  if (wa == 1 && lane < 32) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) red[wb * 128 + b * 32 + lane] = make_float4(sum[b], amax[b], __int_as_float(uarg[b]), 0.f);
+  }
+  __syncthreads();
+  if (wa == 0 && lane < 32) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const float4 o = red[wb * 128 + b * 32 + lane];
+      const int ua2 = __float_as_int(o.z);
+      sum[b] += o.x;
+      if (o.y > amax[b] || (o.y == amax[b] && ua2 < uarg[b])) { amax[b] = o.y; uarg[b] = ua2; }
+      p.partials[(int64_t)s * p.Np + rt * 256 + wb * 128 + b * 32 + lane] =
+          make_float4(sum[b], amax[b] * p.sc, __int_as_float(uarg[b]), 0.f);
+    }
+  }
+}
+
+}  // namespace sce
