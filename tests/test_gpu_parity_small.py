@@ -512,3 +512,16 @@ def test_dw_with_and_without_the_k_split_last_round(N, d, V):
     torch.cuda.synchronize()
     assert torch.equal(dx1, dx2)
     assert pu.maxrel(dw1, dw2) < 2e-6
+
+
+@pytest.mark.parametrize("keep", [False, True])
+def test_more_rows_than_one_dw_launch_takes(keep):
+    """A dW launch takes at most 131072 rows (its K loop): with more rows there are several launches, each with an fp32
+    partial of its own, summed in a fixed order at the end; dX goes panel by panel as always."""
+    N, d, V = 140000, 64, 600
+    inp = _small("irregular", N, d, V)
+    ours = pu.run_ours(inp, "mean", keep_dlogits=keep)
+    ref = pu.run_oracle(inp, ours, "mean", row_chunk=16384)
+    rep = pu.check_parity(ours, ref, "mean")
+    assert rep["n_ignored"] > 0
+    print(rep)
