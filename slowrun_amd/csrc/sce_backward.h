@@ -194,8 +194,6 @@ struct DxParams {
   const DevConsts* dc;     // non-NULL: w_s comes from here
 };
 
-// Row scale and one-hot term of four consecutive dX columns j..j+3 of panel row il:
-//   dX = rho_i w_s (G W_q^T) - sum_k h_ik w_s W_q^T[y_{i+k}, :]
 // LDS a wave uses to stage its quadrant of a dX tile on the way out: 128 rows of 64 fp32 (or bf16) plus 16 bytes
 constexpr int DX_STAGE_BYTES = 128 * (64 * 4 + 16);
 constexpr int SMEM_DX = 4 * DX_STAGE_BYTES > SMEM_BYTES ? 4 * DX_STAGE_BYTES : SMEM_BYTES;
@@ -203,6 +201,8 @@ constexpr int SMEM_DX = 4 * DX_STAGE_BYTES > SMEM_BYTES ? 4 * DX_STAGE_BYTES : S
 constexpr int MAX_SCALE_KBLOCKS = (SMEM_MAX - SMEM_BYTES) / 8;      // K blocks of one scaled main loop: 4096
 static inline int smem_scaled(int kblocks, int at_least) { const int n = SMEM_BYTES + 8 * kblocks; return n > at_least ? n : at_least; }
 
+// Row scale and one-hot term of four consecutive dX columns j..j+3 of panel row il:
+//   dX = rho_i w_s (G W_q^T) - sum_k h_ik w_s W_q^T[y_{i+k}, :]
 struct DxRowTerms {
   float rs;
   float hs[4];
@@ -450,20 +450,17 @@ __global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
   }
 }
 
-// sort keys: one entry per (offset k, row i): key = target y_{i+k} (V if the pair takes no part; targets at or
-// beyond the vocabulary limit Vl take no part),
-// value = entry id k * Np + i
-// The tiles of the last, partly filled round of dW (tile0 .. tile0 + ntail - 1 of the round-robin order), shared out
-// along K: a tile's K loop is kp pairs of K blocks long, all of them together W = ntail * kp pairs, and workgroup g takes
-// pairs [g share, (g + 1) share) of that line -- the end of one tile and the beginning of the next, when its range
-// straddles them.  Piece (g, t) of tile t goes to buf[g + t] as plain stores (g + t grows by one from each piece to the
-// next along the line, so no two pieces meet); bwd_dw_final_kernel adds up a tile's pieces in the order of g.
 // a pointer that is the same in every lane, moved to scalar registers
 __device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* q) {
   const uint64_t u = (uint64_t)(uintptr_t)q;
   const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)u), hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(u >> 32));
   return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
 }
+// The tiles of the last, partly filled round of dW (tile0 .. tile0 + ntail - 1 of the round-robin order), shared out
+// along K: a tile's K loop is kp pairs of K blocks long, all of them together W = ntail * kp pairs, and workgroup g takes
+// pairs [g share, (g + 1) share) of that line -- the end of one tile and the beginning of the next, when its range
+// straddles them.  Piece (g, t) of tile t goes to buf[g + t] as plain stores (g + t grows by one from each piece to the
+// next along the line, so no two pieces meet); bwd_dw_final_kernel adds up a tile's pieces in the order of g.
 struct DwTail {
   float* buf;
   int tile0, ntail, kp, share;      // tile0 < 0: no tail (every tile is in the fp32 partial)
@@ -505,6 +502,9 @@ __global__ __launch_bounds__(256) void bwd_dw_tail_kernel(DwParams p, DwTail tl)
   }
 }
 
+// sort keys: one entry per (offset k, row i): key = target y_{i+k} (V if the pair takes no part; targets at or
+// beyond the vocabulary limit Vl take no part),
+// value = entry id k * Np + i
 __global__ __launch_bounds__(256) void bwd_keys_kernel(const int64_t* __restrict__ targets, int64_t ignore_index, int N, int Np, int Vl,
                                                       int V, int n_predict, int32_t* __restrict__ keys, int32_t* __restrict__ vals,
                                                       int32_t* __restrict__ longlist) {
