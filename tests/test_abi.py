@@ -63,6 +63,14 @@ def test_sizes_for_and_shape_errors(lib):
     for bad in [(0, 128, 100), (10, 100, 100), (10, 128, 0), (1 << 25, 128, 100)]:
         with pytest.raises(RuntimeError):
             _lib.sizes_for(*bad)
+    # the largest vocabulary: the block exponents of one dX tile's K loop (V / 128 blocks) wait in LDS behind the K slots
+    assert _lib.sizes_for(256, 64, 524288).dlogits_bytes == 524288 * 256 + 4096 * 2 * 4
+    with pytest.raises(RuntimeError, match="at most 524288"):
+        _lib.sizes_for(256, 64, 524288 + 64)
+    with pytest.raises(RuntimeError, match="multiple of 16"):
+        _lib.sizes_for(256, 72, 1000)
+    with pytest.raises(RuntimeError, match="below 2\\^24"):
+        _lib.sizes_for((1 << 24) - 100, 64, 1000)
     shape = _lib.SceShape(10, 128, 100, 5, 0)          # at most 4 multi-token-prediction offsets
     out = _lib.SceSizes()
     assert lib.sce_sizes_for(C.byref(shape), C.byref(out)) == 1

@@ -525,3 +525,14 @@ def test_more_rows_than_one_dw_launch_takes(keep):
     rep = pu.check_parity(ours, ref, "mean")
     assert rep["n_ignored"] > 0
     print(rep)
+
+
+@pytest.mark.parametrize("keep", [False, True])
+def test_largest_vocabulary(keep):
+    """V = 524288 is the most the dX kernel takes (the block exponents of a tile's K loop, one per 128 columns, fill the
+    LDS left beside the two K slots); one column beyond it is refused (tests/test_abi.py)."""
+    N, d, V = 300, 64, 524288
+    inp = _small("large_vocab", N, d, V)
+    ours = pu.run_ours(inp, "mean", keep_dlogits=keep)
+    ref = pu.run_oracle(inp, ours, "mean", row_chunk=64)
+    print(pu.check_parity(ours, ref, "mean"))
