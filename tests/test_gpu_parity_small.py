@@ -536,3 +536,13 @@ def test_largest_vocabulary(keep):
     ours = pu.run_ours(inp, "mean", keep_dlogits=keep)
     ref = pu.run_oracle(inp, ours, "mean", row_chunk=64)
     print(pu.check_parity(ours, ref, "mean"))
+
+
+@pytest.mark.parametrize("keep", [False, True])
+def test_wide_hidden_size(keep):
+    """d = 8208: a forward K loop of 66 blocks, 33 column tiles of dX per row tile, and a last tile of 16 columns."""
+    N, d, V = 600, 8208, 1500
+    inp = _small("limited_2p7b", N, d, V)
+    ours = pu.run_ours(inp, "none", keep_dlogits=keep)
+    ref = pu.run_oracle(inp, ours, "none")
+    print(pu.check_parity(ours, ref, "none"))
