@@ -546,3 +546,17 @@ def test_wide_hidden_size(keep):
     ours = pu.run_ours(inp, "none", keep_dlogits=keep)
     ref = pu.run_oracle(inp, ours, "none")
     print(pu.check_parity(ours, ref, "none"))
+
+
+@pytest.mark.parametrize("cap", [1.0, 5.0, 40.0])
+@pytest.mark.parametrize("keep", [False, True])
+def test_softcap_range(cap, keep):
+    """The two ends of the allowed softcap and one between, on inputs with rows that saturate it: at cap = 40 the
+    dlogits span e^-80 .. 1 (block exponents down to 2^-115), at cap = 1 every logit is within one unit of every other."""
+    inp = _small("irregular", 700, 128, 2500)
+    inp.cap = cap
+    ours = pu.run_ours(inp, "mean", keep_dlogits=keep)
+    ref = pu.run_oracle(inp, ours, "mean")
+    rep = pu.check_parity(ours, ref, "mean")
+    assert rep["n_ignored"] > 0
+    print(rep)
