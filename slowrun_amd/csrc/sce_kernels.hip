@@ -493,7 +493,7 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
     else if (a->x_dtype == SCE_BF16)
       quantize_pad_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)a->x, a->x_ld, N, d, xq, S.Np, S.dp, S.ldx, inv_xs, a->x_s_dev);
     else return fail(SCE_EINVAL, "unsupported x dtype %d", a->x_dtype);
-    dim3 gw((unsigned)(S.Vp / 64), (unsigned)(S.dq / 64));
+    dim3 gw((unsigned)(S.Vp / QW_TILE), (unsigned)(S.dq / QW_TILE));
     if (bf16ops) {
     } else if (a->wcache && a->wcache_valid) {
       // the caller vouches that the cache holds e4m3(W / w_s) of this W (unchanged since an earlier call)
