@@ -84,36 +84,44 @@ __global__ __launch_bounds__(1024) void bwd_xi_kernel(const float* __restrict__ 
   if (threadIdx.x == 0) xi[0] = (smax[0] > 0.f && isfinite(smax[0])) ? smax[0] : 1.0f;
 }
 
-// Xt (blocked, dq rows, K = Np) = e4m3( X_q[i][j] * rho_i / xi ), transposed through LDS in 64 x 64 tiles.
+// Xt (blocked, dq rows, K = Np) = e4m3( X_q[i][j] * rho_i / xi ), transposed through LDS in 128 x 128 tiles: a row of
+// the tile is one whole 128-byte line of the blocked layout on the way out, and 128 bytes of an X_q row on the way in.
+constexpr int XT_TILE = 128;
 __global__ __launch_bounds__(256) void bwd_xt_kernel(const uint8_t* __restrict__ xq, int64_t dp, int64_t ldx, int64_t kbn,
                                                     const float* __restrict__ rho, const float* __restrict__ xi,
                                                     uint8_t* __restrict__ xt) {
-  __shared__ uint8_t tile[64][68];
+  __shared__ uint8_t tile[XT_TILE][XT_TILE + 4];
   const int t = threadIdx.x;
-  const int64_t i0 = (int64_t)blockIdx.x * 64, j0 = (int64_t)blockIdx.y * 64;
+  const int64_t i0 = (int64_t)blockIdx.x * XT_TILE, j0 = (int64_t)blockIdx.y * XT_TILE;
   if (j0 < dp) {
-    const int r = t >> 2, c = (t & 3) * 16;
-    const v4i raw = *reinterpret_cast<const v4i*>(xq + (i0 + r) * ldx + j0 + c);
-    const float f = rho[i0 + r] / xi[0];
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      const uint32_t w = (uint32_t)raw[m];
-      const uint32_t o = cvt4_e4m3(e4m3_to_float<0>(w) * f, e4m3_to_float<1>(w) * f, e4m3_to_float<2>(w) * f,
-                                   e4m3_to_float<3>(w) * f);
-      *reinterpret_cast<uint32_t*>(&tile[r][c + 4 * m]) = o;
+    for (int pass = 0; pass < 4; ++pass) {
+      const int r = (t >> 3) + 32 * pass, c = (t & 7) * 16;
+      const v4i raw = *reinterpret_cast<const v4i*>(xq + (i0 + r) * ldx + j0 + c);
+      const float f = rho[i0 + r] / xi[0];
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const uint32_t w = (uint32_t)raw[m];
+        const uint32_t o = cvt4_e4m3(e4m3_to_float<0>(w) * f, e4m3_to_float<1>(w) * f, e4m3_to_float<2>(w) * f,
+                                     e4m3_to_float<3>(w) * f);
+        *reinterpret_cast<uint32_t*>(&tile[r][c + 4 * m]) = o;
+      }
     }
   } else {
-    for (int e = t; e < 64 * 17; e += 256) reinterpret_cast<uint32_t*>(&tile[0][0])[e] = 0;
+    for (int e = t; e < XT_TILE * (XT_TILE + 4) / 4; e += 256) reinterpret_cast<uint32_t*>(&tile[0][0])[e] = 0;
   }
   __syncthreads();
-  const int jr = t >> 2, ic = (t & 3) * 16;
-  uint32_t out[4];
 #pragma unroll
-  for (int m = 0; m < 4; ++m) {
-    out[m] = (uint32_t)tile[ic + 4 * m][jr] | ((uint32_t)tile[ic + 4 * m + 1][jr] << 8) |
-             ((uint32_t)tile[ic + 4 * m + 2][jr] << 16) | ((uint32_t)tile[ic + 4 * m + 3][jr] << 24);
+  for (int pass = 0; pass < 4; ++pass) {
+    const int jr = (t >> 3) + 32 * pass, ic = (t & 7) * 16;
+    uint32_t out[4];
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      out[m] = (uint32_t)tile[ic + 4 * m][jr] | ((uint32_t)tile[ic + 4 * m + 1][jr] << 8) |
+               ((uint32_t)tile[ic + 4 * m + 2][jr] << 16) | ((uint32_t)tile[ic + 4 * m + 3][jr] << 24);
+    }
+    *reinterpret_cast<v4i*>(xt + blocked_offset(j0 + jr, i0 + ic, kbn)) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
   }
-  *reinterpret_cast<v4i*>(xt + blocked_offset(j0 + jr, i0 + ic, kbn)) = (v4i){(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
 }
 
 struct RecomputeParams {

@@ -669,7 +669,7 @@ extern "C" int sce_backward(const sce_args* a) {
                                         (int)S.Np, (int)Vl, (const float*)(sv + S.off_lam), rho, hcoef, blockmax, kept ? nullptr : rowinfo);
   bwd_xi_kernel<<<1, 1024, 0, st>>>(blockmax, nblk, xi);
   {
-    dim3 g((unsigned)(S.Np / 64), (unsigned)(S.dq / 64));
+    dim3 g((unsigned)(S.Np / XT_TILE), (unsigned)(S.dq / XT_TILE));
     bwd_xt_kernel<<<g, 256, 0, st>>>(xq, S.dp, S.ldx, S.Np / BK, rho, xi, xt);
   }
   // rows grouped by target, for the one-hot part of dW
