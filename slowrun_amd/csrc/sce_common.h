@@ -24,7 +24,7 @@ constexpr int NTHREADS = 256;
 constexpr int SMEM_MAX = 160 * 1024;              // LDS a workgroup may hold on gfx950
 
 constexpr float LOG2E = 1.4426950408889634f;
-constexpr int LONG_SEG = 64;     // target columns hit by at least this many rows get their own reduction kernel
+constexpr int LONG_SEG = 16;     // target columns hit by at least this many rows get their own reduction kernel
 constexpr int LONG_CHUNK = 1024; // ... which handles at most about this many rows per workgroup
 
 // Lane index within the wavefront, computed from the execution mask each time it is asked for.  Kernels

@@ -272,11 +272,17 @@ def test_fixed_scales_of_the_trainer_and_overflow_to_nan():
 
 
 def test_frequent_target_segments_are_chunked():
-    """One target shared by 3000 rows (its one-hot part of dW is summed in three chunks), one by 70 rows
-    (a single chunk) and the rest spread out (summed in the final kernel)."""
+    """One target shared by 3000 rows (its one-hot part of dW is summed in three chunks), one by 70 rows and one by
+    exactly 16 (a single chunk each), one by 15 (one short of a chunk of its own) and the rest spread out (summed in
+    the final kernel)."""
     inp = _small("tiny_track", 4096, 128, 512)
     inp.targets[:3000] = 7
     inp.targets[3000:3070] = 11
+    others = inp.targets[3070:].clone()
+    others[(others == 13) | (others == 17)] = 19
+    inp.targets[3070:] = others
+    inp.targets[3070:3086] = 13
+    inp.targets[3086:3101] = 17
     ours = pu.run_ours(inp, "mean")
     ref = pu.run_oracle(inp, ours, "mean")
     print(pu.check_parity(ours, ref, "mean"))
