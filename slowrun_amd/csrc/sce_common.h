@@ -25,7 +25,7 @@ constexpr int SMEM_MAX = 160 * 1024;              // LDS a workgroup may hold on
 
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr int LONG_SEG = 16;     // target columns hit by at least this many rows get their own reduction kernel
-constexpr int LONG_CHUNK = 1024; // ... which handles at most about this many rows per workgroup
+constexpr int LONG_CHUNK = 256;  // ... which handles at most about this many rows per workgroup
 
 // Lane index within the wavefront, computed from the execution mask each time it is asked for.  Kernels
 // that loop over tiles use this (and a wave index kept in a scalar register) instead of threadIdx.x:

@@ -272,7 +272,7 @@ def test_fixed_scales_of_the_trainer_and_overflow_to_nan():
 
 
 def test_frequent_target_segments_are_chunked():
-    """One target shared by 3000 rows (its one-hot part of dW is summed in three chunks), one by 70 rows and one by
+    """One target shared by 3000 rows (its one-hot part of dW is summed in twelve chunks), one by 70 rows and one by
     exactly 16 (a single chunk each), one by 15 (one short of a chunk of its own) and the rest spread out (summed in
     the final kernel)."""
     inp = _small("tiny_track", 4096, 128, 512)
