@@ -427,6 +427,17 @@ def softcapped_cross_entropy(x, lm_head_weight, targets, x_s=None, w_s=None, cap
     return out if reduction == "mean" else out.reshape(lead)
 
 
+def target_probability(x, lm_head_weight, targets, x_s=None, w_s=None, cap=15.0, vocab_size=None, norm_eps=None,
+                       operand_dtype=None):
+    """p(target) of every row under the softcapped head, ``exp(logit[target] - logsumexp(logits))``: what the
+    reference's ensemble evaluation extracts from the full N x V logits of each model before it averages the models
+    (``_forward_pgt``, unlimited/train.py:1063-1069).  Here it is ``exp(-loss)`` of the per-row losses of
+    ``softcapped_cross_entropy(..., reduction='none')``, same arguments; a row whose target is -1 has no target
+    probability and gets 0."""
+    losses = softcapped_cross_entropy(x, lm_head_weight, targets, x_s, w_s, cap, vocab_size, "none", norm_eps, operand_dtype)
+    return torch.where(targets.reshape(losses.shape) == -1, torch.zeros_like(losses), torch.exp(-losses))
+
+
 def quantize_e4m3(t, scale):
     """``t.div(scale).to(torch.float8_e4m3fn)`` (tiny/cuda_kernels.py:340-341) on the HIP quantiser."""
     if not t.is_cuda:

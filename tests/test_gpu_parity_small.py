@@ -171,6 +171,31 @@ def test_eval_head_with_vocabulary_slice():
         assert float((got.reshape(-1) - ref.reshape(-1)).abs().max() / ref.abs().max()) < pu.LOSS_RTOL
 
 
+def test_target_probability_of_the_ensemble_evaluation():
+    """unlimited/train.py:1063-1069: p(target) = exp(logit[target] - logsumexp(logits)) from the full logits; here from
+    the per-row losses, with bf16 operands as the reference's evaluation has them under autocast."""
+    from slowrun_amd.cuda_kernels import target_probability
+    inp = _small("irregular", 600, 128, 1024)
+    x = inp.x.cuda().bfloat16().reshape(3, 200, 128)
+    w = inp.w.cuda().bfloat16()
+    y = inp.targets.cuda().reshape(3, 200)
+    logits = (x.reshape(-1, 128) @ w).float()                      # bf16 result of the bf16 matmul, then fp32
+    logits = inp.cap * torch.tanh(logits / inp.cap)
+    valid = y.reshape(-1) != -1
+    logit_gt = logits.gather(1, y.reshape(-1).clamp(min=0).unsqueeze(1)).squeeze(1)
+    ref = torch.exp(logit_gt - torch.logsumexp(logits, dim=-1))
+    got = target_probability(x, w, y, cap=inp.cap, operand_dtype=torch.bfloat16)
+    assert got.shape == (3, 200)
+    assert float((got.reshape(-1)[valid] - ref[valid]).abs().max() / ref[valid].max()) < pu.LOSS_RTOL
+    assert int((~valid).sum()) > 0 and float(got.reshape(-1)[~valid].abs().max()) == 0.0
+    # e4m3 operands: against the oracle's per-row losses
+    from oracle import eager
+    got8 = target_probability(x, w, y, inp.x_s, inp.w_s, cap=inp.cap)
+    ref8 = eager.softcapped_ce(x.reshape(-1, 128), w, y.reshape(-1), inp.x_s, inp.w_s, cap=inp.cap, reduction="none", want_grads=False)
+    want = torch.exp(-ref8["loss"])
+    assert float((got8.reshape(-1)[valid] - want[valid]).abs().max() / want[valid].max()) < pu.LOSS_RTOL
+
+
 def test_vocabulary_slice_backward_and_weight_cache():
     from oracle import eager
     from slowrun_amd import cuda_kernels as ck
