@@ -280,6 +280,84 @@ __global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p_in) {
                                                        lsc + __builtin_amdgcn_readfirstlane(wb) * KD);
   const int jbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
   T* dx = reinterpret_cast<T*>(p.dx);
+  if (!SPLIT && p.n_predict > 1 && ((reinterpret_cast<uintptr_t>(p.dx) | (uintptr_t)(p.dx_ld * (int64_t)sizeof(T))) & 15) == 0) {
+    // Several prediction offsets: the same staged way out as below, with the W_q^T words of all offsets loaded for one
+    // block of 32 rows and 64 columns at a time (all at once they would not fit the registers; folded into the
+    // accumulators beforehand, offset by offset, the whole kernel, main loop included, takes to scratch memory).
+    // Values and their order are those of DxRowTerms::store4.
+    const int K = p.n_predict;
+    float rs[4], hs[4][4];
+    int yrow[4][4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int il = rt * 256 + wb * 128 + b * 32 + (lane & 31);
+      const bool live = il < p.rows;
+      rs[b] = p.rho[live ? il : 0] * p.w_s;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        hs[b][k] = 0.f; yrow[b][k] = 0;
+        if (k < K) {
+          const bool there = live && il + k < p.rows_left;
+          const float hk = there ? p.hcoef[(int64_t)k * p.Np + il] * p.w_s : 0.f;
+          const int64_t y = there ? p.targets[il + k] : -1;
+          if (hk != 0.f && y >= 0 && y < p.V) { hs[b][k] = hk; yrow[b][k] = (int)y; }
+        }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    constexpr int RB = 64 * (int)sizeof(T), PITCH = RB + 16, CH = RB / 16;     // row bytes, staging pitch, chunks per row
+    uint8_t* stg = smem + wave * DX_STAGE_BYTES;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        uint32_t wk[4][8];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          if (k < K) {
+            const uint8_t* wrow = p.wqt + (int64_t)yrow[b][k] * p.ldx + jbase + pass * 64;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) wk[k][e] = *reinterpret_cast<const uint32_t*>(wrow + (e >> 2) * 32 + 8 * (e & 3));
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        uint8_t* srow = stg + (b * 32 + (lane & 31)) * PITCH + 4 * (lane >> 5) * (int)sizeof(T);
+#pragma unroll
+        for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int a = 2 * pass + a2;
+            float o0 = __fmul_rn(acc[a][b][4 * q + 0], rs[b]), o1 = __fmul_rn(acc[a][b][4 * q + 1], rs[b]);
+            float o2 = __fmul_rn(acc[a][b][4 * q + 2], rs[b]), o3 = __fmul_rn(acc[a][b][4 * q + 3], rs[b]);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              if (k < K) {
+                const uint32_t w = wk[k][a2 * 4 + q];
+                o0 = __builtin_fmaf(-hs[b][k], e4m3_to_float<0>(w), o0); o1 = __builtin_fmaf(-hs[b][k], e4m3_to_float<1>(w), o1);
+                o2 = __builtin_fmaf(-hs[b][k], e4m3_to_float<2>(w), o2); o3 = __builtin_fmaf(-hs[b][k], e4m3_to_float<3>(w), o3);
+              }
+            }
+            uint8_t* dst = srow + (a2 * 32 + 8 * q) * (int)sizeof(T);
+            if constexpr (sizeof(T) == 2)
+              *reinterpret_cast<v2i*>(dst) = (v2i){(int)((uint32_t)float_to_bf16_bits(o0) | ((uint32_t)float_to_bf16_bits(o1) << 16)),
+                                                   (int)((uint32_t)float_to_bf16_bits(o2) | ((uint32_t)float_to_bf16_bits(o3) << 16))};
+            else
+              *reinterpret_cast<v4f*>(dst) = (v4f){o0, o1, o2, o3};
+          }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int n = 0; n < 128 * CH / 64; ++n) {
+        const int c = lane + 64 * n, row = c / CH, k16 = c % CH;
+        const int il = rt * 256 + wb * 128 + row;
+        const int col = ct * 256 + wa * 128 + pass * 64 + k16 * (16 / (int)sizeof(T));
+        if (il < p.rows && col < p.d)
+          *reinterpret_cast<v4i*>(reinterpret_cast<uint8_t*>(dx) + ((int64_t)il * p.dx_ld + col) * (int64_t)sizeof(T)) =
+              *reinterpret_cast<const v4i*>(stg + row * PITCH + k16 * 16);
+      }
+    }
+    return;
+  }
   if (!SPLIT && p.n_predict == 1) {
     // One wave per SIMD has nothing to hide a load behind, so the epilogue is written in three phases with all
     // loads of a phase in flight together: the row terms of the lane's four rows, then the 64 words of the four

@@ -125,6 +125,39 @@ def test_multi_token_prediction(weights):
         assert torch.allclose(plain, losses.detach(), rtol=2e-6, atol=2e-6)
 
 
+@pytest.mark.parametrize("keep", [False, True])
+@pytest.mark.parametrize("x_dtype", [torch.bfloat16, torch.float32])
+def test_multi_token_prediction_through_both_dx_epilogues(keep, x_dtype):
+    """Enough dX tiles in one panel (14 row tiles x 10 column tiles) for the staged epilogue that takes several
+    offsets; with 256-row panels each tile's K loop is shared out and the finishing kernel applies the offsets: the two
+    must give the same bf16 values, and both agree with the oracle."""
+    from oracle import eager
+    from slowrun_amd import cuda_kernels as ck
+    N, d, V = 3400, 2560, 600
+    weights = [1.0, 0.6, 0.3, 0.1]
+    inp = _small("irregular", N, d, V)
+    x = inp.x.cuda().to(x_dtype)
+    w = inp.w.cuda().bfloat16()
+    y = inp.targets.cuda()
+    mw = torch.tensor(weights, device="cuda")
+    go = torch.rand(N, generator=torch.Generator().manual_seed(5)).cuda() / N
+    out, saved, _lse, _am, _nv = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, "none", mtp_weights=mw, keep_dlogits=keep)
+    args = (saved, y, go, N, d, V, inp.x_s, inp.w_s, inp.cap, 1.0, "none", x_dtype, torch.bfloat16)
+    dx1, dw1 = ck.ce_backward(*args, mtp_weights=mw, keep_dlogits=keep)
+    dx2, dw2 = ck.ce_backward(*args, mtp_weights=mw, keep_dlogits=keep, panel_rows=256)
+    torch.cuda.synchronize()
+    if x_dtype == torch.bfloat16:
+        assert torch.equal(dx1, dx2)
+    else:       # the shared-out K loop sums its fp32 parts in another order: visible in fp32 output
+        assert pu.maxrel(dx1, dx2) < 1e-5
+    ref = eager.softcapped_ce_mtp(x, w, y, weights, inp.x_s, inp.w_s, cap=inp.cap, grad_output=go)
+    assert float((out - ref["loss"]).abs().max() / ref["loss"].abs().max()) < pu.LOSS_RTOL
+    for got, want in ((dx1, ref["dx"]), (dw1, ref["dw"])):
+        assert pu.maxrel(got.float(), want) <= pu.GRAD_MAXREL and pu.cosine(got.float(), want) > pu.GRAD_COS
+    ign = y == -1
+    assert int(ign.sum()) > 0
+
+
 def test_traced_by_torch_compile():
     """The trainer wraps its model in torch.compile (tiny/train.py:1254): the loss head must trace without
     a graph break and give the eager result."""
