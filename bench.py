@@ -66,6 +66,80 @@ def cpu_baseline(inp, rows, threads):
     return rows / dt, dt
 
 
+def timed(step, steps, warmup=2):
+    """ms per step over exactly `steps` steps, HIP events on torch's current stream (where the library launches)."""
+    import torch
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def extras(args, inp, x, w, y, go, dev):
+    """Further timings after the headline's timed region, each `extra_steps` steps of forward + backward: the other
+    backward mode and the step with a weight cache at the headline workload, and the reference trainer's own call
+    (tiny/train.py:682-696,1417-1419: N = 65536, d = 1024, three prediction offsets, fixed scales, per-row losses reduced
+    with .mean()) through the autograd Function.  [{name, ms_per_step, frac_fp8_mfma_peak, ...}]"""
+    import torch
+    from slowrun_amd import configs
+    from slowrun_amd import cuda_kernels as ck
+    N, d, V = inp.shape
+    out = []
+
+    def entry(name, ms, n, dd, vv, **more):
+        tf = 6.0 * n * dd * vv / (ms * 1e-3) * 1e-12
+        e = {"name": name, "ms_per_step": round(ms, 4), "tokens_per_s": round(n / (ms * 1e-3), 1), "algorithmic_tflops": round(tf, 1),
+             "frac_fp8_mfma_peak": round(tf / PEAK_FP8_TFLOPS, 4)}
+        e.update(more)
+        return e
+
+    if args.rows is None and args.panel_rows == 0:
+        other_keep = args.dlogits != "keep"
+
+        def step_other():
+            loss, saved, _l, _a, _n = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, "mean", keep_dlogits=other_keep)
+            ck.ce_backward(saved, y, go, N, d, V, inp.x_s, inp.w_s, inp.cap, 1.0, "mean", torch.bfloat16, torch.bfloat16, keep_dlogits=other_keep)
+
+        ms = timed(step_other, args.extra_steps)
+        out.append(entry(f"{inp.name}, dlogits {'kept' if other_keep else 'recomputed in backward (nothing N x V held)'}", ms, N, d, V,
+                         hardware_flops_per_step=(6.0 if other_keep else 8.0) * N * d * V))
+        keep = args.dlogits == "keep"
+        cache = ck.WeightCache()
+
+        def step_cached():
+            loss, saved, _l, _a, _n = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, "mean", keep_dlogits=keep, weight_cache=cache)
+            ck.ce_backward(saved, y, go, N, d, V, inp.x_s, inp.w_s, inp.cap, 1.0, "mean", torch.bfloat16, torch.bfloat16, keep_dlogits=keep,
+                           weight_cache=cache, cache_generation=cache.generation)
+
+        ms = timed(step_cached, args.extra_steps)
+        out.append(entry(f"{inp.name}, dlogits {args.dlogits}, W quantised once and cached across steps (a trainer's micro-steps "
+                         "between optimizer steps)", ms, N, d, V))
+        del cache
+    # the trainer's call
+    tin = configs.make_inputs("tiny_track", N=65536)
+    tn, td, tv = tin.shape
+    tx = tin.x.to(dev, torch.bfloat16).requires_grad_(True)
+    tw = tin.w.to(dev, torch.bfloat16).requires_grad_(True)
+    ty = tin.targets.to(dev)
+    mw = torch.tensor([1.0, 0.5, 0.25], device=dev)
+
+    def step_trainer():
+        tx.grad = None
+        tw.grad = None
+        ck.FusedSoftcappedCrossEntropy.apply(tx, ty, mw, tw, 100 / 448, 1.6 / 448, 0.75 / 448, 1.0).mean().backward()
+
+    ms = timed(step_trainer, args.extra_steps)
+    out.append(entry(f"trainer call (tiny/train.py:694): N={tn}, d={td}, V={tv}, mtp_weights [1, 0.5, 0.25], x_s=100/448, w_s=1.6/448, "
+                     "bf16 in, FusedSoftcappedCrossEntropy.apply(...).mean().backward()", ms, tn, td, tv))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -78,6 +152,9 @@ def main():
                     help="keep: the forward pass emits the dlogits (N x V bytes held until backward, backward is two GEMMs); "
                          "recompute: backward computes the logit tiles again (nothing N x V is held)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the further timings that follow the headline's timed region (the line's `other` list)")
+    ap.add_argument("--extra-steps", type=int, default=10)
     ap.add_argument("--cpu-rows", type=int, default=16384)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the timed region, copy 1 GiB device to device once (a kernel of known traffic, "
@@ -140,6 +217,10 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    other = []
+    if not args.no_extras:
+        other = extras(args, inp, x, w, y, go, dev)
+
     flops_step = 6.0 * N * d * V                      # algorithmic: logits + dX + dW, no recompute
     tokens_per_s = N / (ms_per_step * 1e-3)
     # per-kernel achieved rate: algorithmic flops of the launches of that kind / their time
@@ -167,7 +248,9 @@ def main():
         "dtype": "fp8_e4m3", "data": "synthetic",
         "config": {"workload": f"{inp.name}: N={N}, d={d}, V={V}, cap={inp.cap}, fp8 e4m3 amax scales, bf16 dX/dW, mean reduction",
                    "dlogits": ("kept from the forward pass (8 bits per logit held until backward)" if keep
-                               else "recomputed in backward (nothing N x V held)")},
+                               else "recomputed in backward (nothing N x V held)"),
+                   "argmax": "not asked for in the timed step (a debug output of the forward kernel, about 0.25 ms when asked for)",
+                   "w_quantised": "every step, as the reference does (tiny/cuda_kernels.py:341-343); see `other` for the step with a weight cache"},
         "algorithmic_tflops": round(flops_step / (ms_per_step * 1e-3) * 1e-12, 1),
         "frac_fp8_mfma_peak": round(flops_step / (ms_per_step * 1e-3) * 1e-12 / PEAK_FP8_TFLOPS, 4),
         "hardware_flops_per_step": (6.0 if keep else 8.0) * N * d * V,
@@ -175,6 +258,7 @@ def main():
         "wall_s_timed_region": round(wall, 3),
         "roofline": roofline,
         "kernels": kernels,
+        "other": other,
     }
     if not args.no_cpu_baseline:
         # every core this process has been given: torch's default thread count follows the OMP_NUM_THREADS the box sets

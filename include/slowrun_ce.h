@@ -206,7 +206,7 @@ enum {
   SCE_K_FWD = 1,         /* fused logits + softcap + online LSE (one launch per forward)     */
   SCE_K_FWD_REDUCE = 2,  /* combine of the V-splits and the mean                             */
   SCE_K_BWD_PREP = 3,    /* row scales, scaled X^T, rows grouped by target                   */
-  SCE_K_RECOMPUTE = 4,   /* logit recompute -> on-chip dlogits panel (one launch per panel)  */
+  SCE_K_RECOMPUTE = 4,   /* logit recompute -> dlogits panel in the workspace (one launch per panel) */
   SCE_K_DX = 5,          /* dX panel GEMM                                                    */
   SCE_K_DW = 6,          /* dW panel GEMM                                                    */
   SCE_K_DW_FINAL = 7,    /* one-hot part of dW, scaling, cast                                */
@@ -225,19 +225,14 @@ int sce_timing_read(sce_timing* out);
  * and return the rate in TFLOP/s and the shader clock that the kernels themselves saw (their cycle counter against the
  * 100 MHz reference counter; median over workgroups).  scratch: device memory, 1 KiB per 256 x 256 tile and 16 KiB more.
  *  sce_bench_mfma: 16 independent v_mfma_f32_32x32x64_f8f6f4 per wave and round, operands in registers, no memory traffic;
- *                  random_bytes: NULL (all operands 1.0) or 64 KiB x (4 x CUs) of device bytes that become the operands.
+ *                  random_bytes: NULL (all operands 1.0) or random_bytes_size >= 64 KiB x (4 x CUs) device bytes that become
+ *                  the operands (a smaller buffer is refused).
  *  sce_bench_gemm: C = A B^T through the library's main loop (256 x 256 tiles, global -> LDS -> MFMA), the sums of the
  *                  accumulators stored; A is (M, K) and B (N, K) e4m3 bytes with a row stride of K + 128 bytes. */
-int sce_bench_mfma(const void* random_bytes, int32_t iters, int32_t reps, void* scratch, size_t scratch_bytes, int32_t device,
-                   void* stream, double* tflops, double* shader_mhz);
+int sce_bench_mfma(const void* random_bytes, size_t random_bytes_size, int32_t iters, int32_t reps, void* scratch, size_t scratch_bytes,
+                   int32_t device, void* stream, double* tflops, double* shader_mhz);
 int sce_bench_gemm(const void* A, const void* B, int64_t M, int64_t N, int64_t K, int32_t reps, void* scratch, size_t scratch_bytes,
                    int32_t device, void* stream, double* tflops, double* shader_mhz);
-/*  sce_bench_pingpong: the same product through the ping-pong walk of the opt-in forward kernel (256 x 128 tiles, two waves
- *                  per SIMD that take turns accumulating), with a synthetic epilogue: valu_copies (0..3) times the
- *                  transcendental and conversion work of the dlogits epilogue per value, 0 = only a sum.  Returns the
- *                  time of one launch in ms.  scratch: 2 KiB per 256 rows of B times 8, rounded up to 8 workgroups. */
-int sce_bench_pingpong(const void* A, const void* B, int64_t M, int64_t N, int64_t K, int32_t valu_copies, int32_t reps, void* scratch,
-                       size_t scratch_bytes, int32_t device, void* stream, double* ms_per_launch);
 
 #ifdef __cplusplus
 }

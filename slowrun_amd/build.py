@@ -19,6 +19,7 @@ HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "
 
 def build_library(verbose=True, jobs=2):
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    warn_if_other_toolchain()
     objs, procs = [], []
     for src in SOURCES:
         obj = os.path.join(CSRC, src.replace(".hip", ".o"))
@@ -35,6 +36,83 @@ def build_library(verbose=True, jobs=2):
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
     return LIB_PATH
+
+
+# The toolchain the hand-scheduled parts of the kernels were written and measured against: the main loop's direct-to-LDS
+# loads write M0 inside inline asm (the compiler refuses the register as a clobber) and count their own s_waitcnt vmcnt,
+# and the register allocation of the 256-accumulator kernels decides whether anything is spilled around the main loop.
+# Another compiler may well be fine; kernel_resources() and the GPU tests are what tells.
+TESTED_HIPCC = "7.2.26015"
+
+
+def hipcc_version():
+    """The 'HIP version' line of `hipcc --version` ('' if it cannot be run)."""
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    try:
+        out = subprocess.run([hipcc, "--version"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True).stdout
+    except OSError:
+        return ""
+    for ln in out.splitlines():
+        if ln.startswith("HIP version:"):
+            return ln.split(":", 1)[1].strip()
+    return ""
+
+
+def warn_if_other_toolchain():
+    v = hipcc_version()
+    if v and not v.startswith(TESTED_HIPCC):
+        print(f"slowrun_amd.build: warning: hipcc reports HIP version {v}; the kernels' hand-placed waits and register budgets were "
+              f"checked with {TESTED_HIPCC}.  Run `python -m slowrun_amd.build --resources` and the GPU tests before trusting results.",
+              file=sys.stderr, flush=True)
+    return v
+
+
+_RES_KEYS = {"TotalSGPRs": "sgprs", "VGPRs": "vgprs", "AGPRs": "agprs", "ScratchSize [bytes/lane]": "scratch", "Occupancy [waves/SIMD]": "occupancy",
+             "SGPRs Spill": "sgpr_spill", "VGPRs Spill": "vgpr_spill", "LDS Size [bytes/block]": "lds"}
+
+
+def kernel_resources(verbose=False):
+    """{demangled kernel name: {sgprs, vgprs, agprs, scratch, occupancy, sgpr_spill, vgpr_spill, lds}} of every kernel in
+    sce_kernels.hip, from the compiler's own remarks (-Rpass-analysis=kernel-resource-usage; device code only, nothing is
+    linked or written)."""
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    cmd = [hipcc, *HIP_FLAGS, "--cuda-device-only", "-c", os.path.join(CSRC, "sce_kernels.hip"), "-o", os.devnull,
+           "-Rpass-analysis=kernel-resource-usage"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if out.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + out.stdout)
+    res, cur = {}, None
+    for ln in out.stdout.splitlines():
+        if "remark:" not in ln:
+            continue
+        body = ln.split("remark:", 1)[1].replace("[-Rpass-analysis=kernel-resource-usage]", "").strip()
+        key, _, val = body.partition(":")
+        key, val = key.strip(), val.strip()
+        if key == "Function Name":
+            cur = res.setdefault(val, {})
+        elif cur is not None and key in _RES_KEYS:
+            cur[_RES_KEYS[key]] = int(val)
+    names = list(res)
+    filt = shutil.which("c++filt") or shutil.which("llvm-cxxfilt") or "c++filt"
+    try:
+        dem = subprocess.run([filt], input="\n".join(names), stdout=subprocess.PIPE, text=True, check=True).stdout.splitlines()
+    except (OSError, subprocess.CalledProcessError):
+        dem = names
+    table = {}
+    for m, dname in zip(names, dem):
+        short = dname.split("(")[0].replace("sce::", "").replace("void ", "").strip()
+        table[short] = res[m]
+    return table
+
+
+def format_resources(table):
+    rows = [f"{'kernel':48s} {'VGPR':>5s} {'AGPR':>5s} {'SGPR':>5s} {'SGPR spill':>10s} {'VGPR spill':>10s} {'scratch B/lane':>14s} {'waves/SIMD':>10s} {'LDS B':>7s}"]
+    for k in sorted(table):
+        r = table[k]
+        rows.append(f"{k:48s} {r['vgprs']:5d} {r['agprs']:5d} {r['sgprs']:5d} {r['sgpr_spill']:10d} {r['vgpr_spill']:10d} {r['scratch']:14d} {r['occupancy']:10d} {r['lds']:7d}")
+    return "\n".join(rows)
 
 
 def build_abi_example(verbose=True):
@@ -66,6 +144,10 @@ def _wait(procs, verbose):
 
 
 if __name__ == "__main__":
+    if "--resources" in sys.argv[1:]:
+        print(f"hipcc HIP version {hipcc_version()}")
+        print(format_resources(kernel_resources(verbose=True)))
+        sys.exit(0)
     print(build_library())
     print(build_abi_example())
     sys.exit(0)

@@ -34,7 +34,7 @@ def _mfma(random, scratch, iters=20000, reps=3):
         data = torch.randint(0, 256, (4 * ncu * 65536,), dtype=torch.uint8, device=dev)
         data[(data & 0x7f) == 0x7f] = 0x38                          # no NaN codes among the operands
     tf, mhz = C.c_double(), C.c_double()
-    _lib.check(_lib.lib().sce_bench_mfma(data.data_ptr() if random else None, iters, reps, scratch.data_ptr(), scratch.numel(),
+    _lib.check(_lib.lib().sce_bench_mfma(data.data_ptr() if random else None, data.numel() if random else 0, iters, reps, scratch.data_ptr(), scratch.numel(),
                                          dev.index, None, C.byref(tf), C.byref(mhz)), "sce_bench_mfma")
     return tf.value, mhz.value
 
@@ -149,23 +149,8 @@ def main():
         tf, err = _hipblaslt(N, M, K, dev, reps=3 if M * N * K > 1e12 else 10)
         rep["hipblaslt"][name.split()[0]] = None if tf is None else round(tf, 1)
         print(f"   {name:24s} " + (f"{tf:7.1f} TFLOP/s" if tf is not None else f"not available: {err}"))
-    print("\n4. the ping-pong walk (256 x 128 tiles, two waves per SIMD taking turns) on the logits product, random operands:")
-    print("   time of one launch with 0 to 3 copies of the dlogits epilogue's arithmetic per value (0: a plain sum)")
-    rep["pingpong_ms"] = {}
-    for name, M, N, K in (("d = 2560", 50432, 65536, 2560), ("d = 1024", 50432, 65536, 1024)):
-        a, b = _operand(M, K, "random", dev), _operand(N, K, "random", dev)
-        row = []
-        for copies in range(4):
-            ms = C.c_double()
-            _lib.check(_lib.lib().sce_bench_pingpong(a.data_ptr(), b.data_ptr(), M, N, K, copies, 5, scratch.data_ptr(), scratch.numel(),
-                                                     dev.index, None, C.byref(ms)), "sce_bench_pingpong")
-            row.append(round(ms.value, 3))
-        tf, _ = _gemm(M, N, K, "random", scratch, reps=3)
-        rep["pingpong_ms"][name] = {"copies_0_to_3": row, "main_loop_256x256_ms": round(2.0 * M * N * K / tf * 1e-9, 3)}
-        print(f"   {name}: {row} ms; the 256 x 256 main loop alone on the same product: {rep['pingpong_ms'][name]['main_loop_256x256_ms']} ms")
-        del a, b
     if not args.no_smi:
-        print("\n5. rocm-smi while the main loop runs (8192^3, random operands)")
+        print("\n4. rocm-smi while the main loop runs (8192^3, random operands)")
         idle, samples, rates = _under_load(scratch)
         rep["smi"] = {"idle": idle, "under_load": samples[:: max(1, len(samples) // 6)]}
         rep["under_load"] = {"tflops": [round(r[0], 1) for r in rates][:: max(1, len(rates) // 6)],

@@ -23,11 +23,15 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__
                                                       const float* __restrict__ mtp_weights, int n_predict,
                                                       float cap, int N, int Np, int V, const float* __restrict__ lam,
                                                       float* __restrict__ rho, float* __restrict__ hcoef,
-                                                      float* __restrict__ blockmax, int32_t* __restrict__ rowinfo) {
+                                                      float* __restrict__ blockmax, int32_t* __restrict__ rowinfo, CallMode mode) {
   __shared__ float smax[256];
   const int i = blockIdx.x * 256 + threadIdx.x;
   float r = 0.f;
   float h[4] = {0.f, 0.f, 0.f, 0.f};
+  // the forward call that wrote `saved` was asked for something else (kept dlogits, vocabulary limit, offsets, cap):
+  // its state does not fit this call, and every gradient comes out NaN rather than silently wrong
+  const CallMode fm = *reinterpret_cast<const CallMode*>(reinterpret_cast<const uint8_t*>(hdr) + HDR_MODE_OFF);
+  const bool mismatch = fm.emit != mode.emit || fm.vocab_limit != mode.vocab_limit || fm.n_predict != mode.n_predict || fm.cap_bits != mode.cap_bits;
   if (rowinfo && i < Np) {          // what the recompute kernel wants to know of a row: its boost and its target columns
     rowinfo[i] = __float_as_int(i < N ? lam[i] : 0.f);
     for (int k = 0; k < 4; ++k)
@@ -57,6 +61,10 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__
       }
       r = ldexpf(g * sw * expf(cap - lse), -(int)lam[i]);      // the stored dlogits carry the row's boost 2^lam
     }
+  }
+  if (mismatch && i < N) {
+    r = NAN;
+    for (int k = 0; k < 4; ++k) h[k] = NAN;
   }
   if (i < Np) {
     rho[i] = r;
@@ -158,16 +166,21 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p_in
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wa = wave >> 1, wb = wave & 1;
   // The boosts and targets of the wave's 128 rows go straight to LDS, behind the two slots: requested before the K
   // loop (whose waits for its own, younger loads cover them), read after it, no register held in between.
+  // (Through the compiler's builtin, which knows that the instruction reads M0 and sets it itself; the price -- the
+  // compiler makes the first LDS read after it wait for every vector memory load in flight, the tile loads of the
+  // main loop's prologue included -- is paid once per tile here.)
   {
-    const uint32_t dst = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)(smem + SMEM_BYTES)) + wave * (ROWINFO_PLANES * 512);
-    const int voff = lane_id() * 4;
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    typedef const __attribute__((address_space(1))) int32_t global_i32;
+    lds_u8* dst = (lds_u8*)(smem + SMEM_BYTES) + wave * (ROWINFO_PLANES * 512);
+    const int lane = lane_id();
 #pragma unroll
     for (int q = 0; q < ROWINFO_PLANES; ++q) {
-      const int32_t* src = p.rowinfo + (int64_t)q * p.Np + rt * 256 + wb * 128;
-      // the instruction's offset moves the memory address and the LDS address alike: the second half of the rows
-      asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %2, %3\n\t"
-                   "global_load_lds_dword %2, %3 offset:256"
-                   ::"s"(dst), "n"(q * 512), "v"(voff), "s"(src) : "memory", "scc");
+      global_i32* src = (global_i32*)(uintptr_t)(p.rowinfo + (int64_t)q * p.Np + rt * 256 + wb * 128 + lane);
+      // lane l's dword lands at the LDS base + 4 l; the instruction's offset moves the memory address and the LDS
+      // address alike: the second half of the rows
+      __builtin_amdgcn_global_load_lds(src, dst + q * 512, 4, 0, 0);
+      __builtin_amdgcn_global_load_lds(src, dst + q * 512, 4, 256, 0);
     }
   }
   v16f acc[4][4];
@@ -175,7 +188,7 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p_in
   const int vlim = p.V - ct * 256;           // columns >= vlim of this tile do not exist
   const float* lam = reinterpret_cast<const float*>(smem + SMEM_BYTES) + wave * (ROWINFO_PLANES * 128);     // row block b: 32 floats on
   const int* tgt = reinterpret_cast<const int*>(smem + SMEM_BYTES) + wave * (ROWINFO_PLANES * 128) + 128;
-  take_target_logits<false, true, false, 128>(acc, tgt, p.n_predict, ct * 256 + wa * 128, 0, 0.f, nullptr, 0, nullptr, 0.f, 0.f);
+  take_target_logits<false, true, false, 128>(acc, tgt, p.n_predict, ct * 256 + wa * 128, 0, 0.f, nullptr, 0, nullptr, 0.f, 0.f, 0.f);
   uint32_t ew;
   if (vlim < 256) ew = form_dlogits<true, false, 32, 32>(acc, p.k1, p.c2, vlim, 0, smem, wa, wb, nullptr, lam);
   else ew = form_dlogits<false, false, 32, 32>(acc, p.k1, p.c2, vlim, 0, smem, wa, wb, nullptr, lam);

@@ -27,7 +27,9 @@ __device__ __forceinline__ uint32_t cvt2_e4m3(float a, float b) {
   return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xffffu;
 }
 __device__ __forceinline__ uint32_t cvt4_e4m3(float a, float b, float c, float d) {
-  int w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  // (the instruction keeps the other half of its destination: both halves are written here, so what the destination held
+  // does not matter, and `a` as that old value lets the compiler convert in place instead of clearing a register first)
+  int w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, __float_as_int(a), false);
   w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
   return (uint32_t)w;
 }

@@ -31,8 +31,11 @@ namespace sce {
 // columns, and two quad-permute + byte-permute steps turn that 4 x 4 byte block around.
 // STATS: the forward pass's row statistics as well (sum of e^{z - cap}, largest raw logit and its column), kept in
 // `stat` (LDS, 12 floats per lane: [sum, max, argmax][4 row blocks], NTHREADS apart).
-constexpr int STG_PITCH = 272;                               // 256 + 16: 16-byte aligned, rows shifted by 4 banks
-constexpr int STG_BYTES = 256 * STG_PITCH;                   // 69632
+// 256 + 32: 16-byte aligned, and a row is 72 dwords, 8 banks on from the row before: the dword writes of a wave (the 4 lanes
+// of a quad write 4 consecutive rows, its 8 quads consecutive dwords, the upper half-wave 4 rows on) then fall on
+// 32 h + 8 k + j, all 64 banks once.
+constexpr int STG_PITCH = 288;
+constexpr int STG_BYTES = 256 * STG_PITCH;                   // 73728
 
 // Maximum over the 64 lanes, in every lane.  The lane exchanges are LDS-crossbar swizzles with the pattern in the
 // instruction (xor 1 .. 16 within a half-wave), and one ds_bpermute across the halves whose address comes from

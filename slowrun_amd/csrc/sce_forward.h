@@ -25,6 +25,7 @@ struct FwdParams {
   float k1;                // x_s * w_s * 2 log2(e) / cap : exp2(acc * k1) = e^{2u/cap}
   float ic2;               // 1 / c2, c2 = -2 cap log2(e): e^{z - cap} = exp2(c2 / (1 + e^{2u/cap}))
   float c2;
+  float em2cap;            // e^{-2 cap}: what a logit of -inf adds to the sum of e^{z - cap}
   const DevConsts* dc;     // non-NULL: sc and k1 come from here (a scale lives on the device)
   int want_argmax;         // the caller asks for the rows' argmax: the column of the running maximum is tracked
 };
@@ -96,7 +97,7 @@ __device__ __forceinline__ bool target_valid(const int64_t* __restrict__ targets
 //        sum, and the running maximum / argmax.
 template <bool STORE, bool KNOCK, bool STATS, int TGT_STRIDE, bool ROUND = false>
 __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int* tgt, int n_predict, int col0, int rowbase,
-                                                   float sc, float* s_uy_tile, int Np, float* stat, float k1, float ic2) {
+                                                   float sc, float* s_uy_tile, int Np, float* stat, float k1, float ic2, float em2cap) {
   const int lane = lane_id(), half = lane >> 5;
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
@@ -125,7 +126,7 @@ __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int*
               }
             if (KNOCK && STATS) {
               // (the -inf left behind reads as z = -cap to the epilogue that follows, which will add e^{-2 cap} for it)
-              stat[(0 + b) * NTHREADS] += fast_exp2(fast_rcp(fmaf(fast_exp2(x * k1), ic2, ic2))) - fast_exp2(fast_rcp(ic2));
+              stat[(0 + b) * NTHREADS] += fast_exp2(fast_rcp(fmaf(fast_exp2(x * k1), ic2, ic2))) - em2cap;
               const float amax = stat[(4 + b) * NTHREADS];
               if (x > amax || (x == amax && y < __float_as_int(stat[(8 + b) * NTHREADS]))) {
                 stat[(4 + b) * NTHREADS] = x;
@@ -245,7 +246,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
     const int vbase = ct * 256 + wa * 128 + 4 * (lane_id() >> 5);
     const int* tgt = reinterpret_cast<const int*>(smem + FWD_TGT_OFF) + wb * 128;
     if (EMIT) {
-      take_target_logits<true, true, true, 256>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2);
+      take_target_logits<true, true, true, 256>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2, p.em2cap);
       const int vlim = p.V - ct * 256;
       uint8_t* TT = smem + FWD_STAGE_OFF;
       uint32_t ew;
@@ -268,7 +269,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
         stat[(0 + b) * NTHREADS] = sum[b]; stat[(4 + b) * NTHREADS] = amax[b]; stat[(8 + b) * NTHREADS] = __int_as_float(uarg[b]);
       }
     }
-    if (!EMIT) take_target_logits<true, false, false, 256, BF16>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, nullptr, 0.f, 0.f);
+    if (!EMIT) take_target_logits<true, false, false, 256, BF16>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, nullptr, 0.f, 0.f, 0.f);
     if (EMIT && ct + 1 < ct1) {
       // every wave has read its part of the staging tile (its stores have their data) before the second K slot fills again
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -309,6 +310,117 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
       p.partials[(int64_t)s * p.Np + rt * 256 + wb * 128 + b * 32 + lane] =
           make_float4(sum[b], amax[b] * p.sc, __int_as_float(uarg[b]), 0.f);
     }
+  }
+}
+
+// What a block of 256 rows contributes to the mean loss: left by fwd_combine_kernel in the first 16 bytes of the
+// block's own rows of the partial records (which it has consumed by then), summed by fwd_reduce_kernel.
+struct BlockLoss {
+  double sum;      // sum of lse_i - z[i, y_i] over the valid rows
+  int32_t cnt;     // valid rows
+  int32_t bad;     // targets outside [0, V) other than ignore_index
+};
+static_assert(sizeof(BlockLoss) == 16, "one float4 slot");
+
+// one thread per row: fold the V-splits, write lse / loss / argmax and the saved row statistics
+__global__ __launch_bounds__(256) void fwd_combine_kernel(float4* __restrict__ partials, int S, int N, int Np, int V,
+                                                         const int64_t* __restrict__ targets, int64_t ignore_index, float cap,
+                                                         const float* __restrict__ mtp_weights, int n_predict,
+                                                         float* __restrict__ s_lse, float* __restrict__ s_umax,
+                                                         float* __restrict__ s_zy, float* __restrict__ losses,
+                                                         float* __restrict__ lse_out, int32_t* __restrict__ argmax_out) {
+  __shared__ double ssum[256];
+  __shared__ int scnt[256], sbad[256];
+  const int t = threadIdx.x, i = blockIdx.x * 256 + t;      // the grid covers Np = 256 * gridDim.x rows exactly
+  double term = 0.0;
+  int cnt = 0, bad = 0;
+  if (i >= N) {
+    s_lse[i] = 0.f; s_umax[i] = 0.f;
+    for (int k = 0; k < n_predict; ++k) s_zy[(int64_t)k * Np + i] = 0.f;
+  } else {
+    float sum = 0.f, umax = -INFINITY;
+    int uarg = 0x7fffffff;
+    for (int s = 0; s < S; ++s) {
+      const float4 o = partials[(int64_t)s * Np + i];
+      const int ua = __float_as_int(o.z);
+      sum += o.x;
+      if (o.y > umax || (o.y == umax && ua < uarg)) { umax = o.y; uarg = ua; }
+    }
+    const float lse = cap + logf(sum);
+    s_lse[i] = lse; s_umax[i] = umax;
+    // the forward kernel left the raw logit at each target that takes part: z_y = cap tanh(u_y / cap) replaces it (0 for the others);
+    // loss_i = sum_k w_k (lse_i - z[i, y_{i+k}]) over the offsets that take part (tiny/cuda_kernels.py:226-240)
+    float l = 0.f;
+    for (int k = 0; k < n_predict; ++k) {
+      float zy = 0.f;
+      if (target_valid(targets, ignore_index, i + k, N, V)) {
+        zy = cap * tanhf(s_zy[(int64_t)k * Np + i] / cap);
+        l += (mtp_weights ? mtp_weights[k] : 1.0f) * (lse - zy);
+      }
+      s_zy[(int64_t)k * Np + i] = zy;
+    }
+    if (losses) losses[i] = l;
+    if (lse_out) lse_out[i] = lse;
+    if (argmax_out) argmax_out[i] = (uarg == 0x7fffffff) ? 0 : uarg;
+    const int64_t y = targets[i];
+    if (y != ignore_index) {
+      if (y < 0 || y >= V) bad = 1;
+      else { term = (double)(lse - s_zy[i]); cnt = 1; }
+    }
+  }
+  ssum[t] = term; scnt[t] = cnt; sbad[t] = bad;
+  __syncthreads();               // also: every row of this block has read its partial records
+  for (int w = 128; w > 0; w >>= 1) {
+    if (t < w) { ssum[t] += ssum[t + w]; scnt[t] += scnt[t + w]; sbad[t] += sbad[t + w]; }
+    __syncthreads();
+  }
+  if (t == 0) {
+    BlockLoss bl;
+    bl.sum = ssum[0]; bl.cnt = scnt[0]; bl.bad = sbad[0];
+    *reinterpret_cast<BlockLoss*>(partials + (int64_t)blockIdx.x * 256) = bl;
+  }
+}
+
+// What a forward call was asked for, as far as the matching backward call must have been asked the same: left in the header
+// of the saved state (HDR_MODE_OFF bytes in) by fwd_reduce_kernel and compared by bwd_prep_kernel.  A backward call whose
+// flags differ would read dlogits that were never written, or mask other columns: it gets NaN gradients instead.
+struct CallMode {
+  int32_t emit, vocab_limit, n_predict, cap_bits;
+};
+constexpr int HDR_MODE_OFF = 64;
+static inline CallMode call_mode(bool emit, int vocab_limit, int n_predict, float cap) {
+  CallMode m;
+  m.emit = emit ? 1 : 0; m.vocab_limit = vocab_limit; m.n_predict = n_predict;
+  memcpy(&m.cap_bits, &cap, 4);
+  return m;
+}
+
+// single workgroup: n_valid, number of out-of-range targets, mean loss from the per-block sums (fixed order)
+__global__ __launch_bounds__(1024) void fwd_reduce_kernel(const float4* __restrict__ partials, int nblk,
+                                                         int32_t* __restrict__ hdr, float* __restrict__ loss_out,
+                                                         int32_t* __restrict__ nvalid_out, CallMode mode) {
+  __shared__ double ssum[1024];
+  __shared__ int scnt[1024], sbad[1024];
+  const int t = threadIdx.x;
+  double acc = 0.0;
+  int cnt = 0, bad = 0;
+  for (int b = t; b < nblk; b += 1024) {
+    const BlockLoss bl = *reinterpret_cast<const BlockLoss*>(partials + (int64_t)b * 256);
+    acc += bl.sum; cnt += bl.cnt; bad += bl.bad;
+  }
+  ssum[t] = acc; scnt[t] = cnt; sbad[t] = bad;
+  __syncthreads();
+  for (int w = 512; w > 0; w >>= 1) {
+    if (t < w) { ssum[t] += ssum[t + w]; scnt[t] += scnt[t + w]; sbad[t] += sbad[t + w]; }
+    __syncthreads();
+  }
+  if (t == 0) {
+    hdr[0] = scnt[0]; hdr[1] = sbad[0];
+    const float mean = (float)(ssum[0] / (double)scnt[0]);   // 0/0 = NaN, as F.cross_entropy gives
+    reinterpret_cast<float*>(hdr)[2] = mean;
+    if (loss_out) *loss_out = mean;
+    if (nvalid_out) { nvalid_out[0] = scnt[0]; nvalid_out[1] = sbad[0]; }
+    *reinterpret_cast<CallMode*>(reinterpret_cast<uint8_t*>(hdr) + HDR_MODE_OFF) = mode;
   }
 }
 

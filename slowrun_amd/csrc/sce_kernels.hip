@@ -10,8 +10,7 @@
 //             sum exp(z - cap), the target logits and (on request) max/argmax of u; the logits never leave
 //             the chip.  With dlogits_from_forward it also leaves D = (1 - t^2) exp(z - cap) as e4m3 bytes
 //             with one power-of-two exponent per 32 rows x 128 columns (G^T, tile by tile), the targets'
-//             entries zero.  Partials per (row, V-split) -> combine.  (fwd_pp_kernel: the same from 256x128
-//             tiles with two waves per SIMD; opt-in.)
+//             entries zero.  Partials per (row, V-split) -> combine.
 //   backward: the dlogits as forward left them, or formed again panel by panel from recomputed logit tiles
 //             (bwd_recompute_kernel, same format); dX = rho_row * D W_q^T and dW = (rho X_q)^T D run on the
 //             same MFMA main loop with the exponents applied inside v_mfma_scale_f32_32x32x64_f8f6f4.  The
@@ -19,7 +18,6 @@
 //             (gather of W_q^T rows) and in the dW finalisation (rows grouped by target).
 #include "sce_common.h"
 #include "sce_mainloop.h"
-#include "sce_pingpong.h"
 #include "../../include/slowrun_ce.h"
 
 #include <math.h>
@@ -36,7 +34,6 @@
 #include "sce_quantize.h"
 #include "sce_dlogits.h"
 #include "sce_forward.h"
-#include "sce_forward_pp.h"
 #include "sce_backward.h"
 #include "sce_bench_kernels.h"
 
@@ -143,8 +140,6 @@ static int check_device(int dev) {
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
-      HIP_TRY(hipFuncSetAttribute((const void*)fwd_pp_kernel<12, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD_PP));
-      HIP_TRY(hipFuncSetAttribute((const void*)fwd_pp_kernel<12, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD_PP));
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_sample_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_recompute_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_RECOMPUTE));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
@@ -306,14 +301,6 @@ extern "C" const char* sce_last_error(void) { return g_err; }
 // small and gives every workgroup a long walk; more (up to 16) only where 8 would leave the last round of
 // workgroups, one per CU, mostly empty.
 constexpr int FWD_MAX_SPLITS = 16;
-// SCE_FWD_KERNEL=pingpong in the environment selects the ping-pong walk (fwd_pp_kernel) for the dlogits-emitting
-// forward pass.  It is complete and parity-tested, and on this part slower than fwd_kernel at every shape of the
-// workload table (its 256 x 128 tiles are bound by L2 -> LDS traffic where K is long, and the vector ALU work of one
-// wave delays the MFMAs of the other by about half its length where K is short), so it is not the default.
-static bool fwd_pingpong_wanted() {
-  const char* e = getenv("SCE_FWD_KERNEL");
-  return e && strcmp(e, "pingpong") == 0;
-}
 static int fwd_splits(int RT, int CT, int ncu) {
   if (CT <= 8) return CT;
   auto fill = [&](int S) { const int64_t wg = (int64_t)RT * S; return (double)wg / (double)((wg + ncu - 1) / ncu * ncu); };
@@ -413,7 +400,8 @@ extern "C" int sce_transpose_bytes(const void* src, void* dst, int64_t rows, int
   return SCE_OK;
 }
 
-static int check_common(const sce_args* a) {
+// own_scratch: the call brings its own scratch (sce_forward_noalloc): args->workspace is not looked at
+static int check_common(const sce_args* a, bool own_scratch = false) {
   if (!a) return fail(SCE_EINVAL, "args is NULL");
   if (a->struct_size != sizeof(sce_args)) return fail(SCE_EINVAL, "struct_size %u != %zu (ABI mismatch)", a->struct_size, sizeof(sce_args));
   if (int rc = check_shape(&a->shape)) return rc;
@@ -423,7 +411,7 @@ static int check_common(const sce_args* a) {
     return fail(SCE_EINVAL, "x_s and w_s must be positive");
   if (a->reduction != SCE_REDUCE_NONE && a->reduction != SCE_REDUCE_MEAN) return fail(SCE_EINVAL, "bad reduction %d", a->reduction);
   if (!a->saved) return fail(SCE_EINVAL, "saved is NULL");
-  if (((uintptr_t)a->saved & 255) || ((uintptr_t)a->workspace & 255) || ((uintptr_t)a->wcache & 255))
+  if (((uintptr_t)a->saved & 255) || (!own_scratch && ((uintptr_t)a->workspace & 255)) || ((uintptr_t)a->wcache & 255))
     return fail(SCE_EINVAL, "saved, workspace and wcache must be 256-byte aligned");
   if (a->vocab_limit < 0 || a->vocab_limit > a->shape.V) return fail(SCE_EINVAL, "vocab_limit must be in [0, V]");
   return check_device(a->device);
@@ -513,7 +501,7 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
   p.targets = a->targets; p.ignore_index = a->ignore_index; p.n_predict = a->shape.n_predict; p.s_uy = (float*)(sv + S.off_zy);
   p.ghat_t = emit ? gbase + S.rel_g : nullptr; p.gexp = emit ? (uint32_t*)(gbase + S.rel_gexp) : nullptr; p.kbw = S.Np / BK;
   p.dp = S.dp; p.ldx = S.ldx; p.N = (int)N; p.V = (int)Vl; p.Np = (int)S.Np; p.RT = RT; p.CT = CTw; p.S = nsplit;
-  p.sc = bf16ops ? 1.0f : (float)a->x_s * (float)a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.c2 = -2.0f * a->cap * LOG2E; p.ic2 = 1.0f / p.c2;
+  p.sc = bf16ops ? 1.0f : (float)a->x_s * (float)a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.c2 = -2.0f * a->cap * LOG2E; p.ic2 = 1.0f / p.c2; p.em2cap = expf(-2.0f * a->cap);
   p.dc = bf16ops ? nullptr : dcp;
   p.want_argmax = a->argmax != nullptr;
   const int grid = 8 * nsplit * ((RT + 7) / 8);
@@ -526,12 +514,7 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
   }
   {
     KernelTimer tm(SCE_K_FWD, st);
-    if (emit && fwd_pingpong_wanted()) {
-      // (all tile loads are issued by the accumulating waves: measured faster than sharing them out, and a wait that the
-      // compiler adds in an epilogue unit then has no tile load to wait for)
-      if (a->argmax) fwd_pp_kernel<12, true><<<grid, PP_THREADS, SMEM_FWD_PP, st>>>(p);
-      else fwd_pp_kernel<12, false><<<grid, PP_THREADS, SMEM_FWD_PP, st>>>(p);
-    } else if (emit) fwd_kernel<true><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
+    if (emit) fwd_kernel<true><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
     else if (bf16ops) fwd_kernel<false, true><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
     else fwd_kernel<false><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
   }
@@ -543,7 +526,8 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
                                                        a->cap, a->mtp_weights, a->shape.n_predict, s_lse, s_umax, s_zy, a->losses, a->lse,
                                                        a->argmax);
   fwd_reduce_kernel<<<1, 1024, 0, st>>>(p.partials, (int)(S.Np / 256), (int32_t*)(sv + S.off_hdr),
-                                        a->reduction == SCE_REDUCE_MEAN ? a->loss : nullptr, a->n_valid);
+                                        a->reduction == SCE_REDUCE_MEAN ? a->loss : nullptr, a->n_valid,
+                                        call_mode(emit, (int)Vl, a->shape.n_predict, a->cap));
   HIP_TRY(hipGetLastError());
   return SCE_OK;
 }
@@ -558,7 +542,7 @@ extern "C" int sce_forward(const sce_args* a) {
 // the array; nothing in it has to start at zero (the forward kernel writes every record that the combine kernel
 // reads), so nothing is cleared, but two calls in flight on one device at a time would overwrite each other's records.
 extern "C" int sce_forward_noalloc(const sce_args* a) {
-  if (int rc = check_common(a)) return rc;
+  if (int rc = check_common(a, true)) return rc;
   void* sp = g_scratch[a->device];              // set by check_device (inside check_common) for this very device
   if (!sp) return fail(SCE_EHIP, "no static scratch on device %d", a->device);
   return forward_impl(a, sp, NOALLOC_SCRATCH_BYTES,
@@ -666,7 +650,8 @@ extern "C" int sce_backward(const sce_args* a) {
   KernelTimer* tm_prep = new KernelTimer(SCE_K_BWD_PREP, st);
   bwd_prep_kernel<<<nblk, 256, 0, st>>>(s_lse, s_zy, a->targets, a->ignore_index, hdr, a->grad_output,
                                         a->reduction == SCE_REDUCE_NONE ? 1 : 0, a->grad_scale, a->mtp_weights, K, a->cap, (int)N,
-                                        (int)S.Np, (int)Vl, (const float*)(sv + S.off_lam), rho, hcoef, blockmax, kept ? nullptr : rowinfo);
+                                        (int)S.Np, (int)Vl, (const float*)(sv + S.off_lam), rho, hcoef, blockmax, kept ? nullptr : rowinfo,
+                                        call_mode(kept, (int)Vl, K, a->cap));
   bwd_xi_kernel<<<1, 1024, 0, st>>>(blockmax, nblk, xi);
   {
     dim3 g((unsigned)(S.Np / XT_TILE), (unsigned)(S.dq / XT_TILE));
@@ -788,6 +773,18 @@ extern "C" int sce_backward(const sce_args* a) {
 // ------------------------------------------------------------------------------------------
 // measurement aids
 // ------------------------------------------------------------------------------------------
+struct EventPair {   // two timing events that are destroyed on every way out
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  hipError_t create() {
+    hipError_t e = hipEventCreate(&e0);
+    return e != hipSuccess ? e : hipEventCreate(&e1);
+  }
+  ~EventPair() {
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+  }
+};
+
 static double median_mhz(const long long* clk, int n) {
   std::vector<double> v;
   for (int i = 0; i < n; ++i)
@@ -797,8 +794,8 @@ static double median_mhz(const long long* clk, int n) {
   return v[v.size() / 2];
 }
 
-extern "C" int sce_bench_mfma(const void* random_bytes, int32_t iters, int32_t reps, void* scratch, size_t scratch_bytes, int32_t device,
-                              void* stream, double* tflops, double* shader_mhz) {
+extern "C" int sce_bench_mfma(const void* random_bytes, size_t random_bytes_size, int32_t iters, int32_t reps, void* scratch, size_t scratch_bytes,
+                              int32_t device, void* stream, double* tflops, double* shader_mhz) {
   if (!scratch || !tflops || !shader_mhz || iters <= 0 || reps <= 0) return fail(SCE_EINVAL, "bad argument");
   if (int rc = check_device(device)) return rc;
   DeviceGuard guard(device);
@@ -806,11 +803,16 @@ extern "C" int sce_bench_mfma(const void* random_bytes, int32_t iters, int32_t r
   const int ncu = device_cus_or_default(device), grid = 4 * ncu;           // one wave per SIMD would be grid = ncu; four keep every SIMD fed
   const size_t need = (size_t)grid * 256 * 4 + 2 * 1024 * sizeof(long long);
   if (scratch_bytes < need) return fail(SCE_EINVAL, "scratch too small: %zu < %zu", scratch_bytes, need);
+  // every thread of the grid reads 8 fragments of 32 bytes
+  const size_t need_random = (size_t)grid * 256 * 8 * 32;
+  if (random_bytes && random_bytes_size < need_random)
+    return fail(SCE_EINVAL, "random_bytes too small: %zu < %zu (64 KiB for each of 4 workgroups per compute unit)", random_bytes_size, need_random);
   hipStream_t st = (hipStream_t)stream;
   float* out = (float*)scratch;
   long long* clk = (long long*)((uint8_t*)scratch + (size_t)grid * 256 * 4);
-  hipEvent_t e0, e1;
-  HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
+  EventPair ev;
+  HIP_TRY(ev.create());
+  const hipEvent_t e0 = ev.e0, e1 = ev.e1;
   bench_mfma_kernel<<<grid, 256, 0, st>>>((const uint8_t*)random_bytes, iters, out, clk);      // warm-up
   HIP_TRY(hipEventRecord(e0, st));
   for (int r = 0; r < reps; ++r) bench_mfma_kernel<<<grid, 256, 0, st>>>((const uint8_t*)random_bytes, iters, out, clk);
@@ -820,51 +822,9 @@ extern "C" int sce_bench_mfma(const void* random_bytes, int32_t iters, int32_t r
   HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
   std::vector<long long> h(2 * 1024);
   HIP_TRY(hipMemcpy(h.data(), clk, h.size() * sizeof(long long), hipMemcpyDeviceToHost));
-  (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
   const double flops = (double)reps * grid * 4.0 * iters * 16.0 * (2.0 * 32 * 32 * 64);
   *tflops = flops / (ms * 1e-3) * 1e-12;
   *shader_mhz = median_mhz(h.data(), grid < 1024 ? grid : 1024);
-  return SCE_OK;
-}
-
-extern "C" int sce_bench_pingpong(const void* A, const void* B, int64_t M, int64_t N, int64_t K, int32_t valu_copies, int32_t reps, void* scratch,
-                                  size_t scratch_bytes, int32_t device, void* stream, double* ms_per_launch) {
-  if (!A || !B || !scratch || !ms_per_launch || reps <= 0) return fail(SCE_EINVAL, "bad argument");
-  if (M <= 0 || N <= 0 || K <= 0 || M % 256 || N % 256 || K % 256 || M < 2048) return fail(SCE_EINVAL, "M, N, K must be positive multiples of 256, M at least 2048");
-  if (valu_copies < 0 || valu_copies > 3) return fail(SCE_EINVAL, "valu_copies must be 0..3");
-  if (int rc = check_device(device)) return rc;
-  DeviceGuard guard(device);
-  if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", device);
-  const int RT = (int)(N / 256), CT2 = (int)(M / 128), grid = map_tile_grid(RT, 8);
-  if (scratch_bytes < (size_t)grid * PP_THREADS * 4) return fail(SCE_EINVAL, "scratch too small: %zu < %zu", scratch_bytes, (size_t)grid * PP_THREADS * 4);
-  hipStream_t st = (hipStream_t)stream;
-  const int64_t ld = row_stride(K);
-  const int KD = (int)(K / BK);
-  auto launch = [&]() {
-    const uint8_t* a = (const uint8_t*)A; const uint8_t* b = (const uint8_t*)B; float* c = (float*)scratch;
-    switch (valu_copies) {
-      case 0: bench_pp_kernel<0><<<grid, PP_THREADS, PP_RING, st>>>(a, b, c, KD, RT, CT2, ld); break;
-      case 1: bench_pp_kernel<1><<<grid, PP_THREADS, PP_RING, st>>>(a, b, c, KD, RT, CT2, ld); break;
-      case 2: bench_pp_kernel<2><<<grid, PP_THREADS, PP_RING, st>>>(a, b, c, KD, RT, CT2, ld); break;
-      default: bench_pp_kernel<3><<<grid, PP_THREADS, PP_RING, st>>>(a, b, c, KD, RT, CT2, ld); break;
-    }
-  };
-  HIP_TRY(hipFuncSetAttribute((const void*)bench_pp_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, PP_RING));
-  HIP_TRY(hipFuncSetAttribute((const void*)bench_pp_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, PP_RING));
-  HIP_TRY(hipFuncSetAttribute((const void*)bench_pp_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, PP_RING));
-  HIP_TRY(hipFuncSetAttribute((const void*)bench_pp_kernel<3>, hipFuncAttributeMaxDynamicSharedMemorySize, PP_RING));
-  hipEvent_t e0, e1;
-  HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
-  launch();
-  HIP_TRY(hipEventRecord(e0, st));
-  for (int r = 0; r < reps; ++r) launch();
-  HIP_TRY(hipEventRecord(e1, st));
-  HIP_TRY(hipEventSynchronize(e1));
-  float ms = 0.f;
-  HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
-  (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
-  HIP_TRY(hipGetLastError());
-  *ms_per_launch = ms / reps;
   return SCE_OK;
 }
 
@@ -883,8 +843,9 @@ extern "C" int sce_bench_gemm(const void* A, const void* B, int64_t M, int64_t N
   float* out = (float*)scratch;
   long long* clk = (long long*)((uint8_t*)scratch + (size_t)grid * 256 * 4);
   const int64_t ld = row_stride(K);
-  hipEvent_t e0, e1;
-  HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
+  EventPair ev;
+  HIP_TRY(ev.create());
+  const hipEvent_t e0 = ev.e0, e1 = ev.e1;
   bench_gemm_kernel<<<grid, NTHREADS, SMEM_BYTES, st>>>((const uint8_t*)A, (const uint8_t*)B, out, (int)(K / BK), RT, CT, ld, clk);
   HIP_TRY(hipEventRecord(e0, st));
   for (int r = 0; r < reps; ++r)
@@ -895,7 +856,6 @@ extern "C" int sce_bench_gemm(const void* A, const void* B, int64_t M, int64_t N
   HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
   std::vector<long long> h(2 * 1024);
   HIP_TRY(hipMemcpy(h.data(), clk, h.size() * sizeof(long long), hipMemcpyDeviceToHost));
-  (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
   *tflops = 2.0 * M * N * K * reps / (ms * 1e-3) * 1e-12;
   *shader_mhz = median_mhz(h.data(), grid < 1024 ? grid : 1024);
   return SCE_OK;

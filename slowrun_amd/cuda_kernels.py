@@ -9,7 +9,11 @@ w_s, grad_s, grad_scale[, cap])`` keeps the positional signature of
 tiny/cuda_kernels.py:338 and returns the per-row losses (N,), which the caller
 reduces with ``.mean()`` (tiny/train.py:1417).  Underneath, the work is done by the
 HIP kernels of libslowrun_ce.so through its C ABI; the N x V logits are never
-stored, and nothing N x V sized is kept for backward.
+stored.  What is kept for backward depends on KEEP_DLOGITS (below): by default the
+forward pass leaves the dlogits in the saved state, 8 bits per logit (N x V bytes,
+3.3 GB at N = 65536, V = 50304; the reference keeps three times that,
+tiny/cuda_kernels.py:359-371), and backward is two GEMMs; with keep_dlogits=False
+nothing N x V sized is kept and backward computes the logit tiles again.
 
 Differences from the reference that a caller can see:
   * V is a runtime size (CE_KERNEL_VOCAB_SIZE is kept only for the trainer's asserts);

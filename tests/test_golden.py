@@ -38,8 +38,10 @@ def test_oracle_reproduces_golden(name):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("keep", [False, True])
 @pytest.mark.parametrize("name", CASES)
-def test_hip_path_reproduces_golden(name):
+def test_hip_path_reproduces_golden(name, keep):
+    """keep: the forward pass emits the dlogits (the default of the autograd Function) / backward computes them again."""
     from slowrun_amd import cuda_kernels as ck
     from tests import parity_util as pu
     c = _case(name)
@@ -51,9 +53,9 @@ def test_hip_path_reproduces_golden(name):
     x_s, w_s, cap = float(c["x_s"]), float(c["w_s"]), float(c["cap"])
     assert np.array_equal(ck.quantize_e4m3(x, x_s).view(torch.uint8).cpu().numpy(), c["xq_codes"])
     assert np.array_equal(ck.quantize_e4m3(w, w_s).view(torch.uint8).cpu().numpy(), c["wq_codes"])
-    loss, saved, lse, argmax, n_valid = ck.ce_forward(x, w, y, x_s, w_s, cap, "mean", want_argmax=True)
+    loss, saved, lse, argmax, n_valid = ck.ce_forward(x, w, y, x_s, w_s, cap, "mean", want_argmax=True, keep_dlogits=keep)
     dx, dw = ck.ce_backward(saved, y, torch.ones((), device="cuda"), N, d, V, x_s, w_s, cap, 1.0, "mean",
-                            torch.float32, torch.float32)
+                            torch.float32, torch.float32, keep_dlogits=keep)
     assert abs(float(loss) - float(c["loss"])) / abs(float(c["loss"])) < pu.LOSS_RTOL
     np.testing.assert_allclose(lse.cpu().numpy(), c["lse"], rtol=1e-5, atol=1e-5)
     assert np.array_equal(argmax.cpu().numpy().astype(np.int64), c["argmax"])

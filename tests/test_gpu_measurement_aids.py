@@ -1,4 +1,4 @@
-"""The measurement aids of the C ABI (sce_bench_mfma, sce_bench_gemm, sce_bench_pingpong; slowrun_amd.ceiling builds its
+"""The measurement aids of the C ABI (sce_bench_mfma, sce_bench_gemm; slowrun_amd.ceiling builds its
 report from them): they run at small sizes, return figures that make sense for this part, and refuse shapes their
 kernels do not take."""
 import ctypes as C
@@ -25,33 +25,23 @@ def test_matrix_instruction_alone():
     assert 0.3 * ceiling.PEAK_FP8_TFLOPS < tf_rand < tf_const * 1.02
 
 
-def test_main_loop_alone_and_the_ping_pong_walk():
+def test_main_loop_alone():
     scratch = _scratch()
     tf, mhz = ceiling._gemm(4096, 4096, 2048, "random", scratch, reps=3)
     assert 500 < tf < ceiling.PEAK_FP8_TFLOPS and 1000 < mhz < 2600
-    dev = scratch.device
-    a, b = ceiling._operand(4096, 1024, "random", dev), ceiling._operand(4096, 1024, "random", dev)
-    times = []
-    for copies in (0, 3):
-        ms = C.c_double()
-        _lib.check(_lib.lib().sce_bench_pingpong(a.data_ptr(), b.data_ptr(), 4096, 4096, 1024, copies, 3, scratch.data_ptr(),
-                                                 scratch.numel(), dev.index, None, C.byref(ms)), "sce_bench_pingpong")
-        times.append(ms.value)
-    flops = 2.0 * 4096 * 4096 * 1024
-    assert 0 < times[0] and flops / (times[0] * 1e-3) * 1e-12 < ceiling.PEAK_FP8_TFLOPS
-    assert times[1] > times[0]                      # three copies of the epilogue's arithmetic cost something
 
 
 def test_shapes_the_kernels_do_not_take_are_refused():
     scratch = _scratch()
     lib = _lib.lib()
     a = ceiling._operand(4096, 1024, "zero", scratch.device)
-    tf, mhz, ms = C.c_double(), C.c_double(), C.c_double()
+    tf, mhz = C.c_double(), C.c_double()
     args = (scratch.data_ptr(), scratch.numel(), scratch.device.index, None)
     assert lib.sce_bench_gemm(a.data_ptr(), a.data_ptr(), 4096, 4000, 1024, 1, *args, C.byref(tf), C.byref(mhz)) == 1
+    assert b"multiples of 256" in lib.sce_last_error()
     assert lib.sce_bench_gemm(None, a.data_ptr(), 4096, 4096, 1024, 1, *args, C.byref(tf), C.byref(mhz)) == 1
-    assert lib.sce_bench_pingpong(a.data_ptr(), a.data_ptr(), 1024, 4096, 1024, 0, 1, *args, C.byref(ms)) == 1     # M below 2048
-    assert b"M" in lib.sce_last_error()
-    assert lib.sce_bench_mfma(None, 0, 1, *args, C.byref(tf), C.byref(mhz)) == 1
+    assert lib.sce_bench_mfma(None, 0, 0, 1, *args, C.byref(tf), C.byref(mhz)) == 1
+    assert lib.sce_bench_mfma(a.data_ptr(), 4096, 10, 1, *args, C.byref(tf), C.byref(mhz)) == 1      # operand bytes too few
+    assert b"random_bytes" in lib.sce_last_error()
     assert lib.sce_bench_gemm(a.data_ptr(), a.data_ptr(), 4096, 4096, 1024, 1, scratch.data_ptr(), 16, scratch.device.index, None,
                               C.byref(tf), C.byref(mhz)) == 1                                                       # scratch too small
