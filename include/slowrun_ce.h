@@ -233,6 +233,15 @@ int sce_bench_mfma(const void* random_bytes, size_t random_bytes_size, int32_t i
                    int32_t device, void* stream, double* tflops, double* shader_mhz);
 int sce_bench_gemm(const void* A, const void* B, int64_t M, int64_t N, int64_t K, int32_t reps, void* scratch, size_t scratch_bytes,
                    int32_t device, void* stream, double* tflops, double* shader_mhz);
+/*  sce_bench_floor: the main loops of the three big kernels alone -- the tile walk of the forward kernel (which = SCE_K_FWD),
+ *                  all dX panels (SCE_K_DX), the dW launch (SCE_K_DW) -- in their own operand layouts, tile orders and MFMA
+ *                  variants, with nothing for an epilogue (a checksum per thread).  args: as passed to a forward call with
+ *                  dlogits_from_forward and to the matching backward call, after both have run (saved: X_q, W_q and the
+ *                  dlogits; workspace: the scaled transposed X); all-zero buffers of those sizes give the time of the same
+ *                  instruction stream on operands that draw little power.  N at most 131072.  Returns the time of one pass in
+ *                  ms and the shader clock the kernels saw.  scratch as for sce_bench_gemm, 1 KiB per workgroup of the largest grid. */
+int sce_bench_floor(const sce_args* args, int32_t which, int32_t reps, void* scratch, size_t scratch_bytes, double* ms_per_pass,
+                    double* shader_mhz);
 
 #ifdef __cplusplus
 }

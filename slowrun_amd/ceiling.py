@@ -116,6 +116,77 @@ def _under_load(scratch, seconds=4.0):
     return idle, samples, rates
 
 
+def _floor(workload, scratch, reps=5):
+    """One forward (dlogits kept) + backward of `workload`, timed per kernel kind by the library's events; then the main loops
+    of the three big kernels alone (sce_bench_floor) on the buffers those calls left, and on all-zero buffers of the same
+    sizes.  Returns {kind: {kernel_ms, floor_ms, floor_mhz, floor_zero_ms, floor_zero_mhz}}."""
+    from . import configs
+    from . import cuda_kernels as ck
+    inp = configs.make_inputs(workload)
+    N, d, V = inp.shape
+    dev = scratch.device
+    x, w, y = inp.x.to(dev, torch.bfloat16), inp.w.to(dev, torch.bfloat16), inp.targets.to(dev)
+    sz = _lib.sizes_for(N, d, V)
+    saved = torch.empty(sz.saved_bytes + sz.dlogits_bytes, dtype=torch.uint8, device=dev)
+    fws = torch.empty(sz.fwd_workspace_bytes, dtype=torch.uint8, device=dev)
+    bws = torch.empty(sz.bwd_workspace_kept_bytes, dtype=torch.uint8, device=dev)
+    loss = torch.empty(1, dtype=torch.float32, device=dev)
+    nv = torch.empty(2, dtype=torch.int32, device=dev)
+    go = torch.ones(1, dtype=torch.float32, device=dev)
+    dx = torch.empty(N, d, dtype=torch.bfloat16, device=dev)
+    dw = torch.empty(d, V, dtype=torch.bfloat16, device=dev)
+    a = ck._base_args(x, N, d, V, inp.x_s, inp.w_s, inp.cap, 1.0, "mean", y)
+    a.x, a.x_dtype, a.x_ld = x.data_ptr(), _lib.SCE_BF16, d
+    a.w, a.w_dtype, a.w_ld = w.data_ptr(), _lib.SCE_BF16, V
+    a.loss, a.n_valid = loss.data_ptr(), nv.data_ptr()
+    a.saved, a.saved_bytes = saved.data_ptr(), saved.numel()
+    a.dlogits_from_forward = 1
+    a.grad_output = go.data_ptr()
+    a.dx, a.dx_dtype, a.dx_ld = dx.data_ptr(), _lib.SCE_BF16, d
+    a.dw, a.dw_dtype, a.dw_ld = dw.data_ptr(), _lib.SCE_BF16, V
+
+    def step():
+        a.workspace, a.workspace_bytes = fws.data_ptr(), fws.numel()
+        _lib.check(_lib.lib().sce_forward(C.byref(a)), "sce_forward")
+        a.workspace, a.workspace_bytes = bws.data_ptr(), bws.numel()
+        _lib.check(_lib.lib().sce_backward(C.byref(a)), "sce_backward")
+
+    for _ in range(2):
+        step()
+    torch.cuda.synchronize()
+    _lib.timing_enable(True)
+    for _ in range(reps):
+        step()
+    torch.cuda.synchronize()
+    kt = _lib.timing_read()
+    _lib.timing_enable(False)
+    kinds = {"fwd": 1, "dx": 5, "dw": 6}          # SCE_K_FWD, SCE_K_DX, SCE_K_DW
+    out = {k: {"kernel_ms": round(kt[k][0] / reps, 3)} for k in kinds}
+    flops = 2.0 * N * d * V
+
+    def floors(tag):
+        for k, which in kinds.items():
+            ms, mhz = C.c_double(), C.c_double()
+            _lib.check(_lib.lib().sce_bench_floor(C.byref(a), which, reps, scratch.data_ptr(), scratch.numel(), C.byref(ms), C.byref(mhz)),
+                       "sce_bench_floor")
+            out[k][tag + "_ms"], out[k][tag + "_mhz"] = round(ms.value, 3), round(mhz.value)
+
+    floors("floor")
+    saved.zero_()
+    bws.zero_()
+    floors("floor_zero")
+    for k in kinds:
+        r = out[k]
+        print(f"   {k:3s}: kernel {r['kernel_ms']:6.3f} ms = {flops / r['kernel_ms'] * 1e-9:6.0f} TFLOP/s | main loop alone on the same operands "
+              f"{r['floor_ms']:6.3f} ms = {flops / r['floor_ms'] * 1e-9:6.0f} TFLOP/s at {r['floor_mhz']:4d} MHz | on all-zero operands "
+              f"{r['floor_zero_ms']:6.3f} ms = {flops / r['floor_zero_ms'] * 1e-9:6.0f} TFLOP/s at {r['floor_zero_mhz']:4d} MHz")
+    tot_k, tot_f = sum(out[k]["kernel_ms"] for k in kinds), sum(out[k]["floor_ms"] for k in kinds)
+    print(f"   sum: kernels {tot_k:.3f} ms, main loops alone {tot_f:.3f} ms = {3 * flops / tot_f * 1e-9 / PEAK_FP8_TFLOPS * 100:.1f} % of peak "
+          "for a step that did nothing else")
+    del saved, fws, bws
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--no-smi", action="store_true")
@@ -149,8 +220,10 @@ def main():
         tf, err = _hipblaslt(N, M, K, dev, reps=3 if M * N * K > 1e12 else 10)
         rep["hipblaslt"][name.split()[0]] = None if tf is None else round(tf, 1)
         print(f"   {name:24s} " + (f"{tf:7.1f} TFLOP/s" if tf is not None else f"not available: {err}"))
+    print("\n4. the three big kernels of a step and their main loops alone, on the step's own operand buffers (limited_2p7b: N = 65536, d = 2560, V = 50304)")
+    rep["floor"] = _floor("limited_2p7b", scratch)
     if not args.no_smi:
-        print("\n4. rocm-smi while the main loop runs (8192^3, random operands)")
+        print("\n5. rocm-smi while the main loop runs (8192^3, random operands)")
         idle, samples, rates = _under_load(scratch)
         rep["smi"] = {"idle": idle, "under_load": samples[:: max(1, len(samples) // 6)]}
         rep["under_load"] = {"tflops": [round(r[0], 1) for r in rates][:: max(1, len(rates) // 6)],

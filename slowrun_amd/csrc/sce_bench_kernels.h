@@ -75,4 +75,93 @@ __global__ __launch_bounds__(256) void bench_gemm_kernel(const uint8_t* __restri
   }
 }
 
+// The main loops of the three big kernels alone, on the very buffers a forward and backward call have filled, in their
+// own layouts and tile orders: what fwd_kernel, bwd_dx_kernel and bwd_dw_kernel would take with an epilogue of nothing
+// (each thread stores the sum of its accumulators at the end).  The difference to the real kernels is their epilogues,
+// the difference to the peak is the main loop's.
+__device__ __forceinline__ float acc_sum(const v16f (&acc)[4][4]) {
+  float sum = 0.f;
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sum += acc[a][b][r];
+  return sum;
+}
+__device__ __forceinline__ void floor_clock(long long* clk, long long c0, long long r0) {
+  if (threadIdx.x == 0 && blockIdx.x < 1024) {
+    clk[2 * blockIdx.x] = __builtin_readcyclecounter() - c0; clk[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - r0;
+  }
+}
+
+// the walk of fwd_kernel (one workgroup: a row tile and its share of the column tiles, next tile prefetched), no epilogue
+__global__ __launch_bounds__(256) void floor_fwd_kernel(FwdParams p, float* __restrict__ out, long long* __restrict__ clk) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  int rt, s;
+  if (!map_tile(blockIdx.x, p.RT, p.S, rt, s)) return;
+  const long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+  const int ct0 = (int)((int64_t)p.CT * s / p.S), ct1 = (int)((int64_t)p.CT * (s + 1) / p.S);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  v16f acc[4][4];
+  const uint8_t* Bg = p.xq + (int64_t)rt * 256 * p.ldx;
+  const int KT = (int)(p.dp / BK);
+  const int rot_a = 2 * (rt & 3), rot_b = s & 7;
+  float sum = 0.f;
+  if (ct0 < ct1) mfma_prefetch(p.wqt + (int64_t)ct0 * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
+  for (int ct = ct0; ct < ct1; ++ct) {
+    mfma_mainloop<true>(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, Bg, p.ldx, KT, smem, acc, rot_a, rot_b, wave);
+    if (ct + 1 < ct1) mfma_prefetch(p.wqt + (int64_t)(ct + 1) * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) sum += acc[a][b][0];      // (one value of each block keeps its MFMAs alive)
+  }
+  out[(int64_t)blockIdx.x * 256 + threadIdx.x] = sum;
+  floor_clock(clk, c0, r0);
+}
+
+__global__ __launch_bounds__(256) void floor_dx_kernel(DxParams p, float* __restrict__ out, long long* __restrict__ clk) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  int rt, ct;
+  if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
+  const long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+  const int KD = (int)(p.Vp / BK);
+  const int t = threadIdx.x, wave = t >> 6, wb = wave & 1;
+  uint32_t* lsc = reinterpret_cast<uint32_t*>(smem + SMEM_BYTES);
+  for (int e = t; e < 2 * KD; e += NTHREADS) {
+    const int w = e >= KD, kb = e - w * KD;
+    lsc[e] = p.gexp[(int64_t)kb * p.kbw + 2 * rt + w];
+  }
+  __syncthreads();
+  v16f acc[4][4];
+  const int64_t bpair = p.kbw * BLOCKED_KSTEP;
+  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, true, 1>(p.wq + (int64_t)ct * (p.Vp / BK) * BLOCKED_KSTEP, BK,
+                                                       p.ghat_t + 2 * (int64_t)rt * BLOCKED_KSTEP, BLOCKED_KSTEP, KD, smem, acc,
+                                                       2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave), NoHook(), 128 * BK, bpair,
+                                                       lsc + __builtin_amdgcn_readfirstlane(wb) * KD);
+  out[(int64_t)blockIdx.x * 256 + threadIdx.x] = acc_sum(acc);
+  floor_clock(clk, c0, r0);
+}
+
+__global__ __launch_bounds__(256) void floor_dw_kernel(DwParams p, float* __restrict__ out, long long* __restrict__ clk) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  int rt, ct;
+  if (!map_tile_rr(blockIdx.x, p.RT, p.CT, rt, ct)) return;
+  const long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+  const int t = threadIdx.x, wave = t >> 6, wb = wave & 1;
+  uint32_t* lsc = reinterpret_cast<uint32_t*>(smem + SMEM_BYTES);
+  for (int e = t; e < 2 * p.KT; e += NTHREADS) {
+    const int w = e >= p.KT, kb = e - w * p.KT;
+    lsc[e] = p.gexp[(int64_t)(2 * ct + w) * p.kbw + kb];
+  }
+  __syncthreads();
+  v16f acc[4][4];
+  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, false, 2>(p.xt + ((int64_t)rt * p.kbn + p.kb0) * BLOCKED_KSTEP, BK, p.ghat_t + (int64_t)ct * p.kbw * BLOCKED_KSTEP, BK, p.KT,
+                                                        smem, acc, ct & 7, 2 * (rt & 3), __builtin_amdgcn_readfirstlane(wave), NoHook(), 0, 0,
+                                                        lsc + __builtin_amdgcn_readfirstlane(wb) * p.KT);
+  out[(int64_t)blockIdx.x * 256 + threadIdx.x] = acc_sum(acc);
+  floor_clock(clk, c0, r0);
+}
+
 }  // namespace sce

@@ -860,3 +860,77 @@ extern "C" int sce_bench_gemm(const void* A, const void* B, int64_t M, int64_t N
   *shader_mhz = median_mhz(h.data(), grid < 1024 ? grid : 1024);
   return SCE_OK;
 }
+
+// The main loops of the forward, dX and dW kernels alone on the buffers that a forward call with dlogits_from_forward and
+// the matching backward call have filled (see include/slowrun_ce.h).
+extern "C" int sce_bench_floor(const sce_args* a, int32_t which, int32_t reps, void* scratch, size_t scratch_bytes, double* ms_per_pass,
+                               double* shader_mhz) {
+  if (int rc = check_common(a)) return rc;
+  if (!scratch || !ms_per_pass || !shader_mhz || reps <= 0) return fail(SCE_EINVAL, "bad argument");
+  if (which != SCE_K_FWD && which != SCE_K_DX && which != SCE_K_DW) return fail(SCE_EINVAL, "which must be SCE_K_FWD, SCE_K_DX or SCE_K_DW");
+  if (!a->dlogits_from_forward || a->operand_dtype != 0 || a->wcache) return fail(SCE_EINVAL, "needs the saved state of a forward call with dlogits_from_forward (e4m3 operands, no weight cache)");
+  const int64_t N = a->shape.N, d = a->shape.d, V = a->shape.V;
+  const int K = a->shape.n_predict;
+  const SavedLayout S = saved_layout(N, d, V, K);
+  if (a->saved_bytes < S.total + S.g_total) return fail(SCE_EINVAL, "saved buffer too small: %zu < %zu", a->saved_bytes, S.total + S.g_total);
+  if (S.Np > 131072) return fail(SCE_EINVAL, "at most 131072 rows (one dW launch)");
+  const int64_t P = default_panel(S);
+  const BwdLayout B = bwd_layout(S, P, default_dw_panel(S, P), 1, K, true);
+  if (which == SCE_K_DW && (!a->workspace || a->workspace_bytes < B.off_xt + (size_t)S.dq * S.Np)) return fail(SCE_EINVAL, "backward workspace too small");
+  HIP_TRY(hipFuncSetAttribute((const void*)floor_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+  HIP_TRY(hipFuncSetAttribute((const void*)floor_dx_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
+  HIP_TRY(hipFuncSetAttribute((const void*)floor_dw_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
+  DeviceGuard guard(a->device);
+  if (!guard.ok) return fail(SCE_EHIP, "cannot select device %d", a->device);
+  hipStream_t st = (hipStream_t)a->stream;
+  const uint8_t* sv = (const uint8_t*)a->saved;
+  const uint8_t* xq = sv + S.off_xq;
+  const uint8_t* wqt = sv + S.x_total + S.rel_wqt;
+  const uint8_t* wq = sv + S.x_total + S.rel_wq;
+  const uint8_t* ghat_t = sv + S.total + S.rel_g;
+  const uint32_t* gexp = (const uint32_t*)(sv + S.total + S.rel_gexp);
+  const int RT = (int)(S.Np / 256), CTv = (int)(S.Vp / 256), CTd = (int)(S.dq / 256);
+  const int nsplit = fwd_splits(RT, CTv, device_cus_or_default(a->device));
+  const int fgrid = 8 * nsplit * ((RT + 7) / 8);
+  int maxgrid = std::max(fgrid, std::max(map_tile_grid((int)(P / 256), CTd), map_tile_rr_grid(CTd, CTv)));
+  const size_t need = (size_t)maxgrid * 256 * 4 + 2 * 1024 * sizeof(long long);
+  if (scratch_bytes < need) return fail(SCE_EINVAL, "scratch too small: %zu < %zu", scratch_bytes, need);
+  float* out = (float*)scratch;
+  long long* clk = (long long*)((uint8_t*)scratch + (size_t)maxgrid * 256 * 4);
+  auto pass = [&]() {
+    if (which == SCE_K_FWD) {
+      FwdParams p = {};
+      p.xq = xq; p.wqt = wqt; p.dp = S.dp; p.ldx = S.ldx; p.Np = (int)S.Np; p.RT = RT; p.CT = CTv; p.S = nsplit;
+      floor_fwd_kernel<<<fgrid, NTHREADS, SMEM_BYTES, st>>>(p, out, clk);
+    } else if (which == SCE_K_DX) {
+      for (int64_t p0 = 0; p0 < S.Np; p0 += P) {
+        const int64_t prow = (S.Np - p0 < P) ? (S.Np - p0) : P;
+        DxParams p = {};
+        p.wq = wq; p.ghat_t = ghat_t + (p0 / BK) * BLOCKED_KSTEP; p.gexp = gexp + p0 / BK; p.kbw = S.Np / BK; p.Vp = S.Vp;
+        p.RT = (int)(prow / 256); p.CT = CTd;
+        floor_dx_kernel<<<map_tile_grid(p.RT, CTd), NTHREADS, smem_scaled((int)(S.Vp / BK), 0), st>>>(p, out, clk);
+      }
+    } else {
+      DwParams p = {};
+      p.xt = (const uint8_t*)a->workspace + B.off_xt; p.ghat_t = ghat_t; p.gexp = gexp; p.kbn = S.Np / BK; p.kbw = S.Np / BK; p.kb0 = 0; p.Vp = S.Vp;
+      p.RT = CTd; p.CT = CTv; p.KT = (int)(S.Np / BK);
+      floor_dw_kernel<<<map_tile_rr_grid(CTd, CTv), NTHREADS, smem_scaled(p.KT, 0), st>>>(p, out, clk);
+    }
+  };
+  EventPair ev;
+  HIP_TRY(ev.create());
+  pass();      // warm-up
+  HIP_TRY(hipEventRecord(ev.e0, st));
+  for (int r = 0; r < reps; ++r) pass();
+  HIP_TRY(hipEventRecord(ev.e1, st));
+  HIP_TRY(hipEventSynchronize(ev.e1));
+  HIP_TRY(hipGetLastError());
+  float ms = 0.f;
+  HIP_TRY(hipEventElapsedTime(&ms, ev.e0, ev.e1));
+  std::vector<long long> h(2 * 1024);
+  HIP_TRY(hipMemcpy(h.data(), clk, h.size() * sizeof(long long), hipMemcpyDeviceToHost));
+  *ms_per_pass = ms / reps;
+  *shader_mhz = median_mhz(h.data(), 250);
+  return SCE_OK;
+}
+

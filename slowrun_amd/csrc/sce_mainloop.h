@@ -20,8 +20,53 @@
 // and the others find it there (measured +7 to +13 % on operands that come from HBM).
 #pragma once
 #include "sce_common.h"
+#include <type_traits>
 
 namespace sce {
+
+// The schedule of one K block: what a wave issues in each of the block's 32 MFMA slots (64 clocks each) besides the
+// MFMA itself.  Two kinds of work are placed:
+//   * fragment reads, in units of half a fragment (one ds_read_b128, or two transposing 8-byte reads): r1 = the 16
+//     units of this block's second sub-step, n0 = units of the next block's first sub-step (readable from the barrier
+//     `b2` on, which publishes that block), c0 = what n0 left of this block's own first sub-step.  Units go in the order in
+//     which the MFMAs need their fragments: A0, B0..B3, A1, A2, A3.
+//   * the 16 direct-to-LDS loads of a block: ldEM = loads of the block after the next into this block's LDS slot -- from
+//     b2 on, or earlier behind an extra barrier `b1_after` that tells that every wave has its last fragments of this
+//     block; ldL = the rest of the next block's loads.  The wait that publishes a block comes at b2 of the block before.
+// The four waves of a workgroup run in step and share the compute unit's one path from L2 (64 bytes a clock: 16 clocks
+// for a wave's 1 KB load), so one load per wave and 64-clock MFMA slot already fills that path while it lasts.  Measured
+// at N = 65536, d = 2560, V = 50304, all three big kernels alike: two loads to a slot -- all 16 early, behind the publishing
+// barrier, or all late -- 5 to 10 % slower than schedule 0; reads spread one to a slot (1), loads spread over 22 slots behind
+// an extra barrier (2), and mixtures of the two: within 0.5 % of schedule 0.  At the clock this part grants under fp8 MFMA
+// load the loop is bound neither by where its LDS reads sit nor by the lead its loads have.
+#ifndef SCE_SCHED
+#define SCE_SCHED 0
+#endif
+struct KSched {
+  signed char ldL[32], ldEM[32], r1[32], c0[32], n0[32];
+  int b1_after, b2;
+};
+constexpr KSched KSCHEDS[] = {
+    // 0: fragment reads two to a slot in the second half of each sub-step, loads behind the barrier in the middle of the second
+    {{1, 1, 1, 1, 1, 1, 1, 1}, {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 1, 1, 1, 1, 1, 1, 1},
+     {0, 0, 0, 0, 0, 0, 0, 0, 2, 2, 2, 2, 2, 2, 2, 2}, {0}, {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 2, 2, 2, 2, 2, 2, 2, 2}, -1, 24},
+    // 1: one read unit to a slot almost everywhere, barrier at slot 22, loads 22..31 and 0..5
+    {{1, 1, 1, 1, 1, 1}, {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1},
+     {0, 0, 0, 0, 0, 0, 2, 2, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1}, {1, 1, 1, 1, 1, 1},
+     {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1}, -1, 22},
+    // 2: the reads of 0; an extra barrier after slot 17 lets six loads go out in slots 18..23, the slots with reads take a load every other time
+    {{1, 1, 0, 1, 1, 0, 1, 1}, {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 1, 1, 1, 1, 1, 1, 0, 1, 0, 1, 0, 1, 0},
+     {0, 0, 0, 0, 0, 0, 0, 0, 2, 2, 2, 2, 2, 2, 2, 2}, {0}, {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 2, 2, 2, 2, 2, 2, 2, 2}, 17, 24},
+};
+constexpr KSched KS = KSCHEDS[SCE_SCHED];
+constexpr int ksum(const signed char (&a)[32], int n) { int t = 0; for (int i = 0; i < n; ++i) t += a[i]; return t; }
+constexpr int LOADS_E = ksum(KS.ldEM, KS.b2), LOADS_EM = ksum(KS.ldEM, 32), UNITS_N0 = ksum(KS.n0, 32);
+static_assert(LOADS_EM + ksum(KS.ldL, 32) == 16, "a K block is 16 loads per wave");
+static_assert(ksum(KS.r1, 32) == 16 && UNITS_N0 + ksum(KS.c0, 32) == 16, "a sub-step is 16 read units");
+static_assert(ksum(KS.n0, KS.b2) == 0, "the next block cannot be read before the barrier that publishes it");
+static_assert(LOADS_E == 0 || (KS.b1_after >= 0 && ksum(KS.ldEM, KS.b1_after + 1) == 0), "loads before b2 need the extra barrier");
+constexpr int AHEAD_LOADS = LOADS_EM;      // loads of K block 1 that a prefetch (or the prologue) puts in flight
+constexpr int UNIT_FRAG[8] = {0, 4, 5, 6, 7, 1, 2, 3};      // fragment (0-3: A, 4-7: B) of the q-th pair of read units
 
 // The compiler must not see these loads: it would serialise every later LDS read behind
 // vmcnt(0).  Completion is tracked by hand with s_waitcnt vmcnt before the barrier that
@@ -73,12 +118,12 @@ struct TileLoads {
   }
 };
 
-// Puts K block 0 and the first half of the loads of K block 1 of a tile in flight (24 loads per wave).
+// Puts K block 0 and the first AHEAD_LOADS loads of K block 1 of a tile in flight (16 + AHEAD_LOADS loads per wave).
 // Both LDS slots must be free: every wave is past the closing barrier of the previous main loop.  A
-// main loop that follows with PREFETCHED = true expects these 24 loads to be the wave's newest
+// main loop that follows with PREFETCHED = true expects these loads to be the wave's newest
 // vector memory loads, in this order (stores issued in between do not disturb the count it waits for:
-// loads complete in order, so fewer than 9 operations outstanding means block 0 has landed).
-// PARTS: 1 = block 0 only (slot 0), 2 = the 8 loads of block 1 only (slot 1), 3 = both.
+// vector memory operations complete in order, so at most AHEAD_LOADS of them outstanding means block 0 has landed).
+// PARTS: 1 = block 0 only (slot 0), 2 = the loads of block 1 only (slot 1), 3 = both.
 template <int PARTS = 3>
 __device__ __forceinline__ void mfma_prefetch(const uint8_t* __restrict__ Ag, int64_t lda, const uint8_t* __restrict__ Bg,
                                               int64_t ldb, uint8_t* smem, int rot_a, int rot_b, int wave) {
@@ -89,7 +134,7 @@ __device__ __forceinline__ void mfma_prefetch(const uint8_t* __restrict__ Ag, in
   }
   if (PARTS & 2) {
 #pragma unroll
-    for (int n = 0; n < 8; ++n) ld.issue<1>(n, Ag + BK, Bg + BK);
+    for (int n = 0; n < AHEAD_LOADS; ++n) ld.issue<1>(n, Ag + BK, Bg + BK);
   }
 }
 
@@ -150,8 +195,9 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
   const int r = lane & 31, h = lane >> 5;
   const int sw = (r & 7) ^ ((r >> 3) & 1);
   const int abase = wa * 128 * BK + r * BK, bbase = TM * BK + wb * 128 * BK + r * BK;
-  // fragment n (0-3: A, 4-7: B) of the sub-step with K half `half` in LDS slot `slot`
-  auto rfrag1 = [&](int slot, int half, int n, v8i (&fa)[4], v8i (&fb)[4]) {
+  // half `u` (0, 1) of fragment n (0-3: A, 4-7: B) of the sub-step with K half `half` in LDS slot `slot`: registers 4 u .. 4 u + 3
+  auto runit = [&](int slot, int half, int n, int u, v8i (&fa)[4], v8i (&fb)[4]) {
+    v4i q;
     if (TRB && n >= 4) {
       // B block b = n - 4 from the [K row][N] layout.  ds_read_b64_tr_b8 works on groups of 16 lanes: lane j of a
       // group points at 8 bytes -- here the half (j & 1) of the 16-byte N chunk of K row (j >> 1) -- and gets byte j of
@@ -161,39 +207,38 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
       const int b = n - 4, g = lane >> 4, j = lane & 15;
       const uint8_t* s = smem + slot * SLOT_BYTES + TM * BK + wb * 128 * BK + (64 * half + 32 * (g >> 1) + (j >> 1)) * BK +
                          (((2 * b + (g & 1)) ^ (j >> 1)) << 4) + 8 * (j & 1);
-      v8i f;
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const v2i r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)(s + c * 8 * BK));
-        f[2 * c] = r2[0]; f[2 * c + 1] = r2[1];
-      }
-      fb[b] = f;
-      return;
+      const v2i r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)(s + (2 * u) * 8 * BK));
+      const v2i r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)(s + (2 * u + 1) * 8 * BK));
+      q = (v4i){r0[0], r0[1], r1[0], r1[1]};
+    } else {
+      // Which 32 of the sub-step's 64 K bytes a lane takes does not matter as long as both operands agree -- except
+      // to the block scales: the instruction counts registers 0..3 of lanes l and l + 32 as the first 32 K values (scale
+      // from lane l < 32) and registers 4..7 of both as the second 32 (scale from lane l + 32).  With per-K exponents
+      // (SCALE = 2) the lanes therefore take the 16-byte chunks h and 2 + h, otherwise 2 h and 2 h + 1.
+      const int c0 = ((SCALE == 2 ? 4 * half + h : 4 * half + 2 * h) ^ sw) * 16;
+      const uint8_t* s = smem + slot * SLOT_BYTES + ((n < 4) ? abase + n * 32 * BK : bbase + (n - 4) * 32 * BK);
+      q = *reinterpret_cast<const v4i*>(s + (u ? (c0 ^ (SCALE == 2 ? 32 : 16)) : c0));
     }
-    // Which 32 of the sub-step's 64 K bytes a lane takes does not matter as long as both operands agree -- except
-    // to the block scales: the instruction counts registers 0..3 of lanes l and l + 32 as the first 32 K values (scale
-    // from lane l < 32) and registers 4..7 of both as the second 32 (scale from lane l + 32).  With per-K exponents
-    // (SCALE = 2) the lanes therefore take the 16-byte chunks h and 2 + h, otherwise 2 h and 2 h + 1.
-    const int c0 = ((SCALE == 2 ? 4 * half + h : 4 * half + 2 * h) ^ sw) * 16;
-    const uint8_t* s = smem + slot * SLOT_BYTES + ((n < 4) ? abase + n * 32 * BK : bbase + (n - 4) * 32 * BK);
-    const v4i lo = *reinterpret_cast<const v4i*>(s + c0);
-    const v4i hi = *reinterpret_cast<const v4i*>(s + (c0 ^ (SCALE == 2 ? 32 : 16)));
-    const v8i f = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    if (n < 4) fa[n] = f; else fb[n - 4] = f;
+    v8i& f = n < 4 ? fa[n] : fb[n - 4];
+    f[4 * u] = q[0]; f[4 * u + 1] = q[1]; f[4 * u + 2] = q[2]; f[4 * u + 3] = q[3];
+  };
+  // read units [q0, q0 + cnt) of a sub-step, in the order in which its MFMAs need them
+  auto runits = [&](int slot, int half, int q0, int cnt, v8i (&fa)[4], v8i (&fb)[4]) {
+#pragma unroll
+    for (int q = q0; q < q0 + cnt; ++q) runit(slot, half, UNIT_FRAG[q >> 1], q & 1, fa, fb);
   };
   // prologue: K block 0 and half of block 1 in flight, block 0 visible, fragments of sub-step 0 in registers
   if (!PREFETCHED) {
 #pragma unroll
     for (int n = 0; n < 16; ++n) ld.template issue<0>(n, Ag, Bg);
 #pragma unroll
-    for (int n = 0; n < 8; ++n) ld.template issue<1>(n, Ag + KSTEP, Bg + bk1);
+    for (int n = 0; n < AHEAD_LOADS; ++n) ld.template issue<1>(n, Ag + KSTEP, Bg + bk1);
   }
-  // K block 0 has landed once at most the 8 loads of block 1 (and the stores a caller put between the two) are in flight
-  if (PREFETCHED && stores_between) asm volatile("s_waitcnt vmcnt(24)\n\ts_barrier" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+  // K block 0 has landed once at most the loads of block 1 (and the 16 stores a caller put between the two) are in flight
+  if (PREFETCHED && stores_between) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(AHEAD_LOADS + 16) : "memory");
+  else asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(AHEAD_LOADS) : "memory");
   v8i fa[2][4], fb[2][4];
-#pragma unroll
-  for (int n = 0; n < 8; ++n) rfrag1(0, 0, n, fa[0], fb[0]);
+  runits(0, 0, 0, 16, fa[0], fb[0]);
   // block scales of the current pair of K blocks and of the next one (read one pair ahead)
   const __attribute__((address_space(3))) v2i* scp = (const __attribute__((address_space(3))) v2i*)lds_scale;
   const int sc_shift = (SCALE == 2) ? 8 * (lane >> 5) : 0;      // SCALE = 2: the upper half-wave feeds the odd 32-blocks of K
@@ -218,84 +263,56 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
     else if (SCALE) acc[a][b] = mfma_fp8_scaled_sel(SCALE == 1 ? b : 0, fa[0][a], fb[0][b], zero, 127, sc[0]);
     else acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[0][a], fb[0][b], zero, 0, 0, 0, 0, 0, 0);
   };
-  // One K block = two sub-steps of 16 MFMAs; register set 0 feeds the first, set 1 the second.  The
-  // loop body handles the blocks in pairs (slot 0, then slot 1) so that every LDS address and every
-  // load offset is a constant.  While block k (slot s) is consumed:
-  //   first half of its first sub-step : loads 8..15 of block k+1 (other slot; its loads 0..7 went out before)
-  //   second half                      : fragments of the second sub-step from slot s
-  //   middle of the second sub-step    : every wave has the last fragments of block k in registers and waits
-  //                                      for its own loads of block k+1; the barrier then frees slot s
-  //                                      and publishes block k+1
-  //   second half                      : fragments of block k+1, loads 0..7 of block k+2 into slot s
-  // ga / gb point at the first block of the current pair; MORE tells whether a further pair follows.
+  // One K block = two sub-steps of 16 MFMAs; register set 0 feeds the first, set 1 the second.  The loop body handles
+  // the blocks in pairs (LDS slot 0, then slot 1) so that every LDS address and every load offset is a constant; what
+  // goes into which MFMA slot is the table KS (above).  ga / gb point at the first block of the current pair; `more` tells
+  // whether a further pair follows.
   const uint8_t* ga = Ag;
   const uint8_t* gb = Bg;
-  auto pair = [&](bool first, bool more) {
-    // ---- block 2p (slot 0)
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  // loads [n0, n0 + cnt) of the K block at pa / pb into LDS slot SLOT
+  auto loads = [&](auto slot_tag, int n0, int cnt, const uint8_t* pa, const uint8_t* pb) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      if (first) mm0(i); else mm(0, 0, i);
-      hook(0 + (i & 7));
-      ld.template issue<1>(8 + i, ga + KSTEP, gb + bk1);
-      __builtin_amdgcn_sched_barrier(0);
-    }
+    for (int n = n0; n < n0 + cnt; ++n) ld.template issue<decltype(slot_tag)::value>(n, pa, pb);
+  };
+  // block BLK (0, 1) of the pair, in LDS slot BLK.  p1a / p1b: the next block, p2a / p2b: the one after it; has1 / has2: they exist.
+  auto block = [&](auto blk_tag, bool first, bool has1, bool has2, const uint8_t* p1a, const uint8_t* p1b, const uint8_t* p2a, const uint8_t* p2b) {
+    constexpr int BLK = decltype(blk_tag)::value;
+    using Own = std::integral_constant<int, BLK>;
+    using Other = std::integral_constant<int, 1 - BLK>;
 #pragma unroll
-    for (int i = 8; i < 16; ++i) {
-      if (first) mm0(i); else mm(0, 0, i);
-      hook(8 + (i & 7));
-      rfrag1(0, 1, i - 8, fa[1], fb[1]);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      mm(0, 1, i);
-      hook(16 + (i & 7));
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 8; i < 16; ++i) {
-      mm(0, 1, i);
-      hook(24 + (i & 7));
-      rfrag1(1, 0, i - 8, fa[0], fb[0]);
-      if (more) ld.template issue<0>(i - 8, ga + 2 * KSTEP, gb + bk2);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    // ---- block 2p + 1 (slot 1)
-    if (SCALE && more) sc_load(scn);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      mm(1, 0, i);
-      hook(32 + (i & 7));
-      if (more) ld.template issue<0>(8 + i, ga + 2 * KSTEP, gb + bk2);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-#pragma unroll
-    for (int i = 8; i < 16; ++i) {
-      mm(1, 0, i);
-      hook(40 + (i & 7));
-      rfrag1(1, 1, i - 8, fa[1], fb[1]);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      mm(1, 1, i);
-      hook(48 + (i & 7));
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    if (more) asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 8; i < 16; ++i) {
-      mm(1, 1, i);
-      hook(56 + (i & 7));
-      if (more) {
-        rfrag1(0, 0, i - 8, fa[0], fb[0]);
-        ld.template issue<1>(i - 8, ga + 3 * KSTEP, gb + bk2 + bk1);
+    for (int s = 0; s < 32; ++s) {
+      if (s == KS.b2) {
+        // every wave has all fragments of this block in registers (its reads are complete, not only issued) and its own
+        // loads of the next block have landed: the barrier frees this block's LDS slot and publishes the next block
+        if (has1) {
+          if (has2) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(LOADS_E) : "memory");
+          else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
+      const int sub = s >> 4, i = s & 15;
+      if (first && BLK == 0 && sub == 0) mm0(i); else mm(BLK, sub, i);
+      hook(32 * BLK + s);
+      if (!(first && BLK == 0)) runits(BLK, 0, UNITS_N0 + ksum(KS.c0, s), KS.c0[s], fa[0], fb[0]);      // (the first block's came with the prologue)
+      runits(BLK, 1, ksum(KS.r1, s), KS.r1[s], fa[1], fb[1]);
+      if (has1) {
+        runits(1 - BLK, 0, ksum(KS.n0, s), KS.n0[s], fa[0], fb[0]);
+        loads(Other(), LOADS_EM + ksum(KS.ldL, s), KS.ldL[s], p1a, p1b);
+      }
+      if (has2) loads(Own(), ksum(KS.ldEM, s), KS.ldEM[s], p2a, p2b);
       __builtin_amdgcn_sched_barrier(0);
+      if (s == KS.b1_after && has2) {
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
+  };
+  auto pair = [&](bool first, bool more) {
+    block(I0(), first, true, more, ga + KSTEP, gb + bk1, ga + 2 * KSTEP, gb + bk2);
+    if (SCALE && more) sc_load(scn);
+    block(I1(), false, more, more, ga + 2 * KSTEP, gb + bk2, ga + 3 * KSTEP, gb + bk2 + bk1);
     if (SCALE && more) { sc[0] = scn[0]; sc[1] = scn[1]; }
   };
   const int P = KD >> 1;
