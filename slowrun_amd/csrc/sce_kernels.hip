@@ -674,12 +674,80 @@ extern "C" int sce_backward(const sce_args* a) {
   int launch = 0;
   DwTail tail;
   tail.buf = nullptr; tail.tile0 = -1; tail.ntail = 0; tail.kp = 1; tail.share = 1;
-  int64_t w0 = 0;                      // first row of the rows gathered for the next dW launch
-  for (int64_t p0 = 0; p0 < S.Np; p0 += P) {
-    const int64_t prow = (S.Np - p0 < P) ? (S.Np - p0) : P;     // multiple of 256
-    const int RTp = (int)(prow / 256);
-    const int64_t gorg = kept ? 0 : w0;                         // the row that K block 0 of the dlogits buffer stands for
-    if (!kept) {
+  const bool dx_f32 = a->dx_dtype == SCE_F32;
+  const int smem_dx = smem_scaled((int)(S.Vp / BK), SMEM_DX);
+  // dX of the rows [p0, p0 + prow) (a multiple of 256), the dlogits buffer standing for rows from gorg on
+  auto dx_params = [&](int64_t p0, int64_t prow, int64_t gorg) {
+    DxParams q;
+    q.wq = wq; q.ghat_t = ghat_t + ((p0 - gorg) / BK) * BLOCKED_KSTEP; q.gexp = gexp + (p0 - gorg) / BK; q.kbw = gkb; q.wqt = wqt; q.rho = rho + p0; q.hcoef = hcoef + p0; q.targets = a->targets + p0;
+    q.dx_ld = a->dx_ld; q.Vp = S.Vp; q.ldx = S.ldx; q.Np = S.Np; q.dq = S.dq; q.RT = (int)(prow / 256); q.CT = CTd;
+    q.n_predict = K; q.rows_left = (int)(N - p0 > 0 ? N - p0 : 0);
+    q.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); q.d = (int)d; q.V = (int)Vl; q.w_s = (float)a->w_s; q.dc = dcp;
+    q.part = (float*)(ws + B.off_dxpart);
+    q.ksplit = 1;
+    q.dx = dx_f32 ? (void*)((float*)a->dx + p0 * a->dx_ld) : (void*)((bf16_t*)a->dx + p0 * a->dx_ld);
+    return q;
+  };
+  auto dx_panel = [&](int64_t p0, int64_t prow, int64_t gorg) {
+    DxParams dp_ = dx_params(p0, prow, gorg);
+    // a panel with fewer than half as many tiles as there are CUs shares each tile's K loop among several workgroups
+    const int tiles = dp_.RT * CTd, kpairs = (int)(S.Vp / BK / 2);
+    int ksplit = tiles * 2 <= 256 ? 256 / tiles : 1;
+    if (ksplit > 8) ksplit = 8;
+    if (ksplit > kpairs) ksplit = kpairs;
+    dp_.ksplit = ksplit;
+    KernelTimer tm(SCE_K_DX, st);
+    if (ksplit == 1) {
+      if (dx_f32) bwd_dx_kernel<float, false><<<map_tile_grid(dp_.RT, CTd), NTHREADS, smem_dx, st>>>(dp_);
+      else bwd_dx_kernel<bf16_t, false><<<map_tile_grid(dp_.RT, CTd), NTHREADS, smem_dx, st>>>(dp_);
+    } else if (dp_.rows > 0) {
+      const int fgrid = (int)(((int64_t)dp_.rows * (d / 4) + 255) / 256);
+      if (dx_f32) {
+        bwd_dx_kernel<float, true><<<map_tile_grid(dp_.RT, CTd * ksplit), NTHREADS, smem_dx, st>>>(dp_);
+        bwd_dx_finish_kernel<float><<<fgrid, 256, 0, st>>>(dp_);
+      } else {
+        bwd_dx_kernel<bf16_t, true><<<map_tile_grid(dp_.RT, CTd * ksplit), NTHREADS, smem_dx, st>>>(dp_);
+        bwd_dx_finish_kernel<bf16_t><<<fgrid, 256, 0, st>>>(dp_);
+      }
+    }
+  };
+  // dW over the rows [w0, w0 + gathered)
+  auto dw_launch = [&](int64_t w0, int64_t gathered, int64_t gorg, bool last) {
+    DwParams wp;
+    const int part = launch < nparts ? launch : nparts - 1;
+    wp.xt = xt; wp.ghat_t = ghat_t + ((w0 - gorg) / BK) * BLOCKED_KSTEP; wp.gexp = gexp + (w0 - gorg) / BK; wp.dwacc = (float*)((uint8_t*)dwacc + (size_t)part * B.part_stride);
+    wp.kbn = S.Np / BK; wp.kbw = gkb; wp.kb0 = w0 / BK; wp.Vp = S.Vp;
+    wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(gathered / BK);
+    {
+      KernelTimer tm(SCE_K_DW, st);
+      // When this launch is the only one and its last round of tiles would leave many CUs idle, that round is
+      // shared out along K instead (bwd_dw_tail_kernel): the full rounds run as they are.
+      const DwTailPlan tp = dw_tail_plan(S.dq, S.Vp, gathered);
+      const bool only = w0 == 0 && last && launch == 0;
+      if (only && tp.use && B.tail_bytes >= tp.bytes && a->workspace_bytes >= B.off_dwtail + tp.bytes) {
+        const int full = tp.full;
+        tail.buf = (float*)(ws + B.off_dwtail); tail.tile0 = tp.full; tail.ntail = tp.ntail; tail.kp = tp.kp; tail.share = tp.share;
+        if (full > 0) bwd_dw_kernel<false><<<full, NTHREADS, smem_scaled(wp.KT, 0), st>>>(wp);
+        bwd_dw_tail_kernel<<<DW_TAIL_WGS, NTHREADS, smem_scaled(2 * tp.share, 0), st>>>(wp, tail);
+      } else if (launch >= nparts) bwd_dw_kernel<true><<<map_tile_rr_grid(CTd, CTv), NTHREADS, smem_scaled(wp.KT, 0), st>>>(wp);
+      else bwd_dw_kernel<false><<<map_tile_rr_grid(CTd, CTv), NTHREADS, smem_scaled(wp.KT, 0), st>>>(wp);
+    }
+    ++launch;
+  };
+  if (kept) {
+    // The dlogits of all rows are there: dX and dW are independent of each other.  dX still goes panel by panel, one
+    // round of tiles each.  (One grid of tiles over all rows, launched 256 tiles at a time -- ten full rounds at N = 65536,
+    // d = 2560 instead of ten panels of 250 tiles and a ragged eleventh -- was measured no faster: a launch of 256 tiles takes
+    // 0.58 ms where one of 250 takes 0.56.  Under fp8 MFMA load the part runs at the clock its power limit allows, and
+    // compute units left idle leave the others a higher one.)
+    for (int64_t p0 = 0; p0 < S.Np; p0 += P) dx_panel(p0, (S.Np - p0 < P) ? (S.Np - p0) : P, 0);
+    for (int64_t w0 = 0; w0 < S.Np; w0 += Pw) dw_launch(w0, (S.Np - w0 < Pw) ? (S.Np - w0) : Pw, 0, w0 + Pw >= S.Np);
+  } else {
+    int64_t w0 = 0;                      // first row of the rows gathered for the next dW launch
+    for (int64_t p0 = 0; p0 < S.Np; p0 += P) {
+      const int64_t prow = (S.Np - p0 < P) ? (S.Np - p0) : P;     // multiple of 256
+      const int RTp = (int)(prow / 256);
+      const int64_t gorg = w0;                                    // the row that K block 0 of the dlogits buffer stands for
       RecomputeParams rp;
       rp.xq = xq + p0 * S.ldx; rp.wqt = wqt; rp.ghat_t = ghat_t; rp.gexp = gexp; rp.rowinfo = rowinfo + p0; rp.Np = S.Np; rp.n_predict = K;
       rp.dp = S.dp; rp.ldx = S.ldx; rp.kbw = gkb; rp.kb0 = (p0 - gorg) / BK; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2; rp.dc = dcp;
@@ -687,63 +755,12 @@ extern "C" int sce_backward(const sce_args* a) {
         KernelTimer tm(SCE_K_RECOMPUTE, st);
         bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_RECOMPUTE, st>>>(rp);
       }
-    }
-
-    DxParams dp_;
-    dp_.wq = wq; dp_.ghat_t = ghat_t + ((p0 - gorg) / BK) * BLOCKED_KSTEP; dp_.gexp = gexp + (p0 - gorg) / BK; dp_.kbw = gkb; dp_.wqt = wqt; dp_.rho = rho + p0; dp_.hcoef = hcoef + p0; dp_.targets = a->targets + p0;
-    dp_.dx_ld = a->dx_ld; dp_.Vp = S.Vp; dp_.ldx = S.ldx; dp_.Np = S.Np; dp_.dq = S.dq; dp_.RT = RTp; dp_.CT = CTd;
-    dp_.n_predict = K; dp_.rows_left = (int)(N - p0 > 0 ? N - p0 : 0);
-    dp_.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); dp_.d = (int)d; dp_.V = (int)Vl; dp_.w_s = (float)a->w_s; dp_.dc = dcp;
-    dp_.part = (float*)(ws + B.off_dxpart);
-    // a panel with fewer than half as many tiles as there are CUs shares each tile's K loop among several workgroups
-    const int tiles = RTp * CTd, kpairs = (int)(S.Vp / BK / 2);
-    int ksplit = tiles * 2 <= 256 ? 256 / tiles : 1;
-    if (ksplit > 8) ksplit = 8;
-    if (ksplit > kpairs) ksplit = kpairs;
-    dp_.ksplit = ksplit;
-    {
-      KernelTimer tm(SCE_K_DX, st);
-      const bool f32 = a->dx_dtype == SCE_F32;
-      const int smem_dx = smem_scaled((int)(S.Vp / BK), SMEM_DX);
-      dp_.dx = f32 ? (void*)((float*)a->dx + p0 * a->dx_ld) : (void*)((bf16_t*)a->dx + p0 * a->dx_ld);
-      if (ksplit == 1) {
-        if (f32) bwd_dx_kernel<float, false><<<map_tile_grid(RTp, CTd), NTHREADS, smem_dx, st>>>(dp_);
-        else bwd_dx_kernel<bf16_t, false><<<map_tile_grid(RTp, CTd), NTHREADS, smem_dx, st>>>(dp_);
-      } else if (dp_.rows > 0) {
-        const int fgrid = (int)(((int64_t)dp_.rows * (d / 4) + 255) / 256);
-        if (f32) {
-          bwd_dx_kernel<float, true><<<map_tile_grid(RTp, CTd * ksplit), NTHREADS, smem_dx, st>>>(dp_);
-          bwd_dx_finish_kernel<float><<<fgrid, 256, 0, st>>>(dp_);
-        } else {
-          bwd_dx_kernel<bf16_t, true><<<map_tile_grid(RTp, CTd * ksplit), NTHREADS, smem_dx, st>>>(dp_);
-          bwd_dx_finish_kernel<bf16_t><<<fgrid, 256, 0, st>>>(dp_);
-        }
+      dx_panel(p0, prow, gorg);
+      const int64_t gathered = p0 + prow - w0;
+      if (gathered + P > Pw || p0 + prow >= S.Np) {      // the transposed scratch is full, or this was the last panel
+        dw_launch(w0, gathered, gorg, p0 + prow >= S.Np);
+        w0 = p0 + prow;
       }
-    }
-
-    const int64_t gathered = p0 + prow - w0;
-    if (gathered + P > Pw || p0 + prow >= S.Np) {      // the transposed scratch is full, or this was the last panel
-      DwParams wp;
-      const int part = launch < nparts ? launch : nparts - 1;
-      wp.xt = xt; wp.ghat_t = ghat_t + ((w0 - gorg) / BK) * BLOCKED_KSTEP; wp.gexp = gexp + (w0 - gorg) / BK; wp.dwacc = (float*)((uint8_t*)dwacc + (size_t)part * B.part_stride);
-      wp.kbn = S.Np / BK; wp.kbw = gkb; wp.kb0 = w0 / BK; wp.Vp = S.Vp;
-      wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(gathered / BK);
-      {
-        KernelTimer tm(SCE_K_DW, st);
-        // When this launch is the only one and its last round of tiles would leave many CUs idle, that round is
-        // shared out along K instead (bwd_dw_tail_kernel): the full rounds run as they are.
-        const DwTailPlan tp = dw_tail_plan(S.dq, S.Vp, gathered);
-        const bool only = w0 == 0 && p0 + prow >= S.Np && launch == 0;
-        if (only && tp.use && B.tail_bytes >= tp.bytes && a->workspace_bytes >= B.off_dwtail + tp.bytes) {
-          const int full = tp.full;
-          tail.buf = (float*)(ws + B.off_dwtail); tail.tile0 = tp.full; tail.ntail = tp.ntail; tail.kp = tp.kp; tail.share = tp.share;
-          if (full > 0) bwd_dw_kernel<false><<<full, NTHREADS, smem_scaled(wp.KT, 0), st>>>(wp);
-          bwd_dw_tail_kernel<<<DW_TAIL_WGS, NTHREADS, smem_scaled(2 * tp.share, 0), st>>>(wp, tail);
-        } else if (launch >= nparts) bwd_dw_kernel<true><<<map_tile_rr_grid(CTd, CTv), NTHREADS, smem_scaled(wp.KT, 0), st>>>(wp);
-        else bwd_dw_kernel<false><<<map_tile_rr_grid(CTd, CTv), NTHREADS, smem_scaled(wp.KT, 0), st>>>(wp);
-      }
-      ++launch;
-      w0 = p0 + prow;
     }
   }
   if (a->norm) {       // dX so far is the gradient of the normalised rows: take it through the norm, in place
