@@ -564,41 +564,45 @@ struct DwTail {
   float* buf;
   int tile0, ntail, kp, share;      // tile0 < 0: no tail (every tile is in the fp32 partial)
 };
+// (grid: workgroups x 2.  A workgroup's range is at most half a tile's K loop long, so it lies in one tile or straddles
+// two: blockIdx.y = 0 takes the part in the first tile, blockIdx.y = 1 the part in the second, if there is one.  One piece
+// per workgroup, with no loop around the main loop: looping over the pieces, the compiler spilled the accumulators.)
 __global__ __launch_bounds__(256) void bwd_dw_tail_kernel(DwParams p, DwTail tl) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int g = blockIdx.x;
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
-  int pos = g * tl.share;
-  const int end = min(tl.ntail * tl.kp, pos + tl.share);
-  uint32_t* lsc = reinterpret_cast<uint32_t*>(smem + SMEM_BYTES);
-  while (pos < end) {
-    // (everything here is uniform, but the divisions leave their results in vector registers: the main loop wants
-    // its addresses in scalar ones)
-    const int tt = __builtin_amdgcn_readfirstlane(pos / tl.kp);
-    const int k0 = pos - tt * tl.kp, k1 = min(tl.kp, k0 + (end - pos)), KD = 2 * (k1 - k0);
-    int rt, ct;
-    tile_from_index(tl.tile0 + tt, p.RT, p.CT, rt, ct);
-    rt = __builtin_amdgcn_readfirstlane(rt); ct = __builtin_amdgcn_readfirstlane(ct);
-    for (int e = t; e < 2 * KD; e += NTHREADS) {
-      const int w = e >= KD, kb = e - w * KD;
-      lsc[e] = p.gexp[(int64_t)(2 * ct + w) * p.kbw + 2 * k0 + kb];
-    }
-    __syncthreads();
-    v16f acc[4][4];
-    mfma_mainloop<false, NoHook, BLOCKED_KSTEP, false, 2>(uniform_ptr(p.xt + ((int64_t)rt * p.kbn + p.kb0 + 2 * k0) * BLOCKED_KSTEP), BK,
-                                                          uniform_ptr(p.ghat_t + ((int64_t)ct * p.kbw + 2 * k0) * BLOCKED_KSTEP), BK,
-                                                          __builtin_amdgcn_readfirstlane(KD), smem, acc, ct & 7, 2 * (rt & 3),
-                                                          __builtin_amdgcn_readfirstlane(wave), NoHook(), 0, 0,
-                                                          lsc + __builtin_amdgcn_readfirstlane(wb) * KD);
-    float* dst0 = tl.buf + (size_t)(g + tt) * 65536 + (wa * 128 + 4 * (lane >> 5)) * 256 + wb * 128 + (lane & 31);
-#pragma unroll
-    for (int b = 0; b < 4; ++b)
-#pragma unroll
-      for (int a = 0; a < 4; ++a)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) dst0[(a * 32 + 8 * (r >> 2) + (r & 3)) * 256 + b * 32] = acc[a][b][r];
-    pos += k1 - k0;
+  const int pos0 = g * tl.share, end = min(tl.ntail * tl.kp, pos0 + tl.share);
+  if (pos0 >= end) return;
+  int tt = pos0 / tl.kp, pos = pos0;
+  if (blockIdx.y == 1) {
+    ++tt; pos = tt * tl.kp;
+    if (pos >= end) return;
   }
+  // (everything here is uniform, but the divisions leave their results in vector registers: the main loop wants
+  // its addresses in scalar ones)
+  tt = __builtin_amdgcn_readfirstlane(tt);
+  const int k0 = __builtin_amdgcn_readfirstlane(pos - tt * tl.kp), k1 = min(tl.kp, k0 + (end - pos)), KD = __builtin_amdgcn_readfirstlane(2 * (k1 - k0));
+  int rt, ct;
+  tile_from_index(tl.tile0 + tt, p.RT, p.CT, rt, ct);
+  rt = __builtin_amdgcn_readfirstlane(rt); ct = __builtin_amdgcn_readfirstlane(ct);
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wa = wave >> 1, wb = wave & 1;
+  uint32_t* lsc = reinterpret_cast<uint32_t*>(smem + SMEM_BYTES);
+  for (int e = t; e < 2 * KD; e += NTHREADS) {
+    const int w = e >= KD, kb = e - w * KD;
+    lsc[e] = p.gexp[(int64_t)(2 * ct + w) * p.kbw + 2 * k0 + kb];
+  }
+  __syncthreads();
+  v16f acc[4][4];
+  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, false, 2>(uniform_ptr(p.xt + ((int64_t)rt * p.kbn + p.kb0 + 2 * k0) * BLOCKED_KSTEP), BK,
+                                                        uniform_ptr(p.ghat_t + ((int64_t)ct * p.kbw + 2 * k0) * BLOCKED_KSTEP), BK,
+                                                        KD, smem, acc, ct & 7, 2 * (rt & 3), __builtin_amdgcn_readfirstlane(wave), NoHook(), 0, 0,
+                                                        lsc + __builtin_amdgcn_readfirstlane(wb) * KD);
+  float* dst0 = tl.buf + (size_t)(g + tt) * 65536 + (wa * 128 + 4 * (lane >> 5)) * 256 + wb * 128 + (lane & 31);
+#pragma unroll
+  for (int b = 0; b < 4; ++b)
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dst0[(a * 32 + 8 * (r >> 2) + (r & 3)) * 256 + b * 32] = acc[a][b][r];
 }
 
 // sort keys: one entry per (offset k, row i): key = target y_{i+k} (V if the pair takes no part; targets at or

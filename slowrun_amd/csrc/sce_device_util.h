@@ -19,6 +19,9 @@ __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {   // round to 
   return (uint16_t)(u >> 16);
 }
 __device__ __forceinline__ float round_to_bf16(float f) { return bf16_bits_to_float(float_to_bf16_bits(f)); }
+// the same value through the hardware conversion (v_cvt_pk_bf16_f32: round to nearest even; a NaN stays a NaN, with
+// whatever payload the hardware gives it)
+__device__ __forceinline__ float round_to_bf16_hw(float f) { return (float)(__bf16)f; }
 
 // two floats -> two e4m3 bytes (low half of the result).  v_cvt_pk_fp8_f32 on gfx950 is OCP
 // e4m3fn, round to nearest even, 464 -> 448 and anything larger -> NaN code: the same rule as

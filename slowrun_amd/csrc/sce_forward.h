@@ -35,8 +35,7 @@ struct FwdParams {
 //   t = tanh(u/cap) = 1 - 2/(E + 1), E = e^{2u/cap};   e^{z - cap} = exp2(c2 / (E + 1)).
 // The column of the maximum is looked up only on the (rare, after the first tiles) occasion that
 // a tile raises a row's running maximum.
-// ROUND: the logits are rounded to bf16 first (bf16 operands: the GEMM of the eager head returns bf16).
-template <bool EDGE, bool ROUND = false>
+template <bool EDGE>
 __device__ __forceinline__ void fwd_epilogue(const v16f (&acc)[4][4], const FwdParams& p, int vbase,
                                              float (&sum)[4], float (&amax)[4], int (&uarg)[4]) {
 #pragma unroll
@@ -47,7 +46,7 @@ __device__ __forceinline__ void fwd_epilogue(const v16f (&acc)[4][4], const FwdP
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int vo = a * 32 + 8 * (r >> 2) + (r & 3);
-        float x = ROUND ? round_to_bf16(acc[a][b][r]) : acc[a][b][r];
+        float x = acc[a][b][r];
         // z - cap = c2 / (1 + e^{2u/cap}) in units of log2: the reciprocal of (1 + e) / c2 gives it in one step
         float pt = fast_exp2(fast_rcp(fmaf(fast_exp2(x * p.k1), p.ic2, p.ic2)));
         if (EDGE) {
@@ -66,7 +65,7 @@ __device__ __forceinline__ void fwd_epilogue(const v16f (&acc)[4][4], const FwdP
 #pragma unroll
           for (int r = 15; r >= 0; --r) {
             const int vo = a * 32 + 8 * (r >> 2) + (r & 3);
-            if ((ROUND ? round_to_bf16(acc[a][b][r]) : acc[a][b][r]) == tmax && (!EDGE || vo < p.V - vbase)) targ = vo;   // descending scan: lowest column wins
+            if (acc[a][b][r] == tmax && (!EDGE || vo < p.V - vbase)) targ = vo;   // descending scan: lowest column wins
           }
         }
         amax[b] = tmax;
@@ -95,7 +94,7 @@ __device__ __forceinline__ bool target_valid(const int64_t* __restrict__ targets
 //        neighbours', out of the 8 bits.
 // STATS: with KNOCK, the row statistics (stat, as in form_dlogits) take the target's share here: e^{z_y - cap} into the
 //        sum, and the running maximum / argmax.
-template <bool STORE, bool KNOCK, bool STATS, int TGT_STRIDE, bool ROUND = false>
+template <bool STORE, bool KNOCK, bool STATS, int TGT_STRIDE>
 __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int* tgt, int n_predict, int col0, int rowbase,
                                                    float sc, float* s_uy_tile, int Np, float* stat, float k1, float ic2, float em2cap) {
   const int lane = lane_id(), half = lane >> 5;
@@ -136,7 +135,7 @@ __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int*
           }
           xk[k] = x;
           // (the lane index is taken anew: an address kept from outside the branch stays live across the main loop and is spilled)
-          if (STORE) s_uy_tile[(int64_t)k * Np + rowbase + b * 32 + (lane_id() & 31)] = ROUND ? round_to_bf16(x) * sc : x * sc;
+          if (STORE) s_uy_tile[(int64_t)k * Np + rowbase + b * 32 + (lane_id() & 31)] = x * sc;
         }
       }
     }
@@ -262,14 +261,23 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
       for (int b = 0; b < 4; ++b) {
         sum[b] = stat[(0 + b) * NTHREADS]; amax[b] = stat[(4 + b) * NTHREADS]; uarg[b] = __float_as_int(stat[(8 + b) * NTHREADS]);
       }
-      if (ct * 256 + 256 > p.V) fwd_epilogue<true, BF16>(acc, p, vbase, sum, amax, uarg);
-      else fwd_epilogue<false, BF16>(acc, p, vbase, sum, amax, uarg);
+      if (BF16) {
+        // the GEMM of the eager head returns bf16: the logits are rounded once, in place, and everything after sees the rounded values
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+          for (int b = 0; b < 4; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = round_to_bf16_hw(acc[a][b][r]);
+      }
+      if (ct * 256 + 256 > p.V) fwd_epilogue<true>(acc, p, vbase, sum, amax, uarg);
+      else fwd_epilogue<false>(acc, p, vbase, sum, amax, uarg);
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         stat[(0 + b) * NTHREADS] = sum[b]; stat[(4 + b) * NTHREADS] = amax[b]; stat[(8 + b) * NTHREADS] = __int_as_float(uarg[b]);
       }
     }
-    if (!EMIT) take_target_logits<true, false, false, 256, BF16>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, nullptr, 0.f, 0.f, 0.f);
+    if (!EMIT) take_target_logits<true, false, false, 256>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, nullptr, 0.f, 0.f, 0.f);
     if (EMIT && ct + 1 < ct1) {
       // every wave has read its part of the staging tile (its stores have their data) before the second K slot fills again
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");

@@ -728,7 +728,7 @@ extern "C" int sce_backward(const sce_args* a) {
         const int full = tp.full;
         tail.buf = (float*)(ws + B.off_dwtail); tail.tile0 = tp.full; tail.ntail = tp.ntail; tail.kp = tp.kp; tail.share = tp.share;
         if (full > 0) bwd_dw_kernel<false><<<full, NTHREADS, smem_scaled(wp.KT, 0), st>>>(wp);
-        bwd_dw_tail_kernel<<<DW_TAIL_WGS, NTHREADS, smem_scaled(2 * tp.share, 0), st>>>(wp, tail);
+        bwd_dw_tail_kernel<<<dim3(DW_TAIL_WGS, 2), NTHREADS, smem_scaled(2 * tp.share, 0), st>>>(wp, tail);
       } else if (launch >= nparts) bwd_dw_kernel<true><<<map_tile_rr_grid(CTd, CTv), NTHREADS, smem_scaled(wp.KT, 0), st>>>(wp);
       else bwd_dw_kernel<false><<<map_tile_rr_grid(CTd, CTv), NTHREADS, smem_scaled(wp.KT, 0), st>>>(wp);
     }
