@@ -135,23 +135,21 @@ __global__ __launch_bounds__(256) void bwd_xt_kernel(const uint8_t* __restrict__
 struct RecomputeParams {
   const uint8_t* xq;     // [Np][dp], already offset to the panel's first row
   const uint8_t* wqt;    // [Vp][dp]
-  uint8_t* ghat_t;       // Vp rows, K = 128 * kbw, blocked
+  uint8_t* ghat_t;       // G of the rows this buffer stands for, tile by tile (kbv blocks of 128 columns per tile of 256 rows)
   uint32_t* gexp;        // [Vp / 128][kbw]
   const int32_t* rowinfo;      // [ROWINFO_PLANES][Np], offset to the panel's first row: boosts and targets (bwd_prep_kernel)
   int64_t Np;
   int n_predict;
   int64_t dp, ldx;             // K extent and row stride of xq / wqt
-  int64_t kbw, kb0;            // ghat_t (blocked): K blocks per tile, K block of this panel's first row
+  int64_t kbw, kb0, kbv;       // blocks of 128 rows in the buffer (row stride of gexp), block of this panel's first row, blocks of 128 columns
   int RT, CT, V;
   float k1, c2;          // as in FwdParams
   const DevConsts* dc;   // non-NULL: k1 comes from here
 };
 
-// Recompute a 256 x 256 logit tile and leave its block-scaled dlogits in G^T.  The tile is assembled in LDS (free
-// once the main loop is done) and leaves the chip as 64 KB of consecutive 16-byte stores.
+// Recompute a 256 x 256 logit tile and leave its block-scaled dlogits in G (16-byte stores straight from the registers).
 constexpr int ROWINFO_PLANES = 5;                      // per row: exponent boost (a float), then the target column of each of 4 offsets (or -1)
-constexpr int SMEM_RECOMPUTE = SMEM_BYTES + 4 * ROWINFO_PLANES * 512;      // two K slots (the staging tile reuses them) + the row data of 128 rows per wave
-static_assert(STG_BYTES <= SMEM_BYTES, "the staging tile must fit the K slots");
+constexpr int SMEM_RECOMPUTE = SMEM_BYTES + 4 * ROWINFO_PLANES * 512;      // two K slots + the row data of 128 rows per wave
 
 __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p_in) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -190,15 +188,15 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p_in
   const int* tgt = reinterpret_cast<const int*>(smem + SMEM_BYTES) + wave * (ROWINFO_PLANES * 128) + 128;
   take_target_logits<false, true, false, 128>(acc, tgt, p.n_predict, ct * 256 + wa * 128, 0, 0.f, nullptr, 0, nullptr, 0.f, 0.f, 0.f);
   uint32_t ew;
-  if (vlim < 256) ew = form_dlogits<true, false, 32, 32>(acc, p.k1, p.c2, vlim, 0, smem, wa, wb, nullptr, lam);
-  else ew = form_dlogits<false, false, 32, 32>(acc, p.k1, p.c2, vlim, 0, smem, wa, wb, nullptr, lam);
-  store_dlogits_quadrant(smem, p.ghat_t + ((int64_t)ct * p.kbw + p.kb0 + 2 * rt + wb) * BLOCKED_KSTEP + wa * 128 * BK, wa, wb);
+  uint8_t* gq = const_cast<uint8_t*>(uniform_ptr(p.ghat_t + ((p.kb0 / 2 + rt) * p.kbv + 2 * ct + wa) * BLOCKED_KSTEP + wb * 128 * BK));      // the wave's quadrant of G
+  if (vlim < 256) ew = form_dlogits<true, false, 32, 32>(acc, p.k1, p.c2, vlim, 0, gq, wa, wb, nullptr, lam);
+  else ew = form_dlogits<false, false, 32, 32>(acc, p.k1, p.c2, vlim, 0, gq, wa, wb, nullptr, lam);
   if (lane_id() == 0) p.gexp[(int64_t)(2 * ct + wa) * p.kbw + p.kb0 + 2 * rt + wb] = ew;
 }
 
 struct DxParams {
   const uint8_t* wq;      // dq rows, K = Vp, tile by tile: A side (rows j)
-  const uint8_t* ghat_t;  // G^T, blocked; already at the K block of the panel's first row    B side (rows i of the panel)
+  const uint8_t* ghat_t;  // G, tile by tile (rows i, K = v); already at the tile of the panel's first row    B side (rows i of the panel)
   const uint32_t* gexp;   // its block exponents [Vp / 128][kbw], likewise at the panel's first row
   const uint8_t* wqt;     // [Vp][dp]   for the one-hot gather
   const float* rho;       // offset to the panel
@@ -207,7 +205,7 @@ struct DxParams {
   void* dx;               // offset to the panel's first row
   float* part;            // [ksplit][RT * 256][dq] fp32 partial sums (ksplit > 1 only)
   int64_t dx_ld, Vp, ldx, Np, dq;        // Vp: K extent; ldx: row stride of wqt
-  int64_t kbw;                           // K blocks (of 128 rows i) per v tile of ghat_t
+  int64_t kbw;                           // blocks of 128 rows i that gexp counts per block of 128 columns
   int RT, CT, rows, d, V;  // rows: valid rows in this panel
   int n_predict, rows_left; // rows_left: N - (first row of the panel), bounds the target look-ahead
   int ksplit;              // the K loop (V) is cut into this many parts, one workgroup each
@@ -284,13 +282,11 @@ __global__ __launch_bounds__(256) void bwd_dx_kernel(DxParams p_in) {
   }
   __syncthreads();
   v16f acc[4][4];
-  // B = G^T: K (v) is the slow index there.  The 128 v rows of a K block are half a v tile; the 256 panel rows of this
-  // tile are the two 128-byte pieces of i blocks 2 rt and 2 rt + 1 (BLOCKED_KSTEP apart).
-  const int64_t bpair = p.kbw * BLOCKED_KSTEP;                     // from one v tile (two K blocks) to the next
-  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, true, 1>(p.wq + ((int64_t)ct * (p.Vp / BK) + k0 / BK) * BLOCKED_KSTEP, BK,
-                                                       p.ghat_t + 2 * (int64_t)rt * BLOCKED_KSTEP + (k0 / (2 * BK)) * bpair, BLOCKED_KSTEP, KD, smem, acc,
-                                                       2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave), NoHook(), 128 * BK, bpair,
-                                                       lsc + __builtin_amdgcn_readfirstlane(wb) * KD);
+  // both operands tile by tile with K = v: W_q rows j, G rows i
+  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, false, 1>(p.wq + ((int64_t)ct * (p.Vp / BK) + k0 / BK) * BLOCKED_KSTEP, BK,
+                                                        p.ghat_t + ((int64_t)rt * (p.Vp / BK) + k0 / BK) * BLOCKED_KSTEP, BK, KD, smem, acc,
+                                                        2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave), NoHook(), 0, 0,
+                                                        lsc + __builtin_amdgcn_readfirstlane(wb) * KD);
   const int jbase = ct * 256 + wa * 128 + 4 * (lane >> 5);
   T* dx = reinterpret_cast<T*>(p.dx);
   if (!SPLIT && p.n_predict > 1 && ((reinterpret_cast<uintptr_t>(p.dx) | (uintptr_t)(p.dx_ld * (int64_t)sizeof(T))) & 15) == 0) {
@@ -508,10 +504,11 @@ __global__ __launch_bounds__(256) void bwd_dx_finish_kernel(DxParams p_in) {
 
 struct DwParams {
   const uint8_t* xt;      // dq rows, K = Np, blocked                             A side (rows j)
-  const uint8_t* ghat_t;  // Vp rows, blocked, already at the first K block of this launch          B side (rows v)
+  const uint8_t* ghat_t;  // G, tile by tile (rows i, K = v), already at the tile of this launch's first row      B side (rows v, through the transposing read)
   const uint32_t* gexp;   // its block exponents [Vp / 128][kbw], likewise
   float* dwacc;           // [dq][Vp] fp32
-  int64_t kbn, kbw, kb0, Vp;   // K blocks per tile of xt and of ghat_t; first K block of xt in this launch; row length of dwacc
+  int64_t kbn, kbw, kb0, Vp;   // K blocks per tile of xt; blocks of 128 rows that gexp counts; first K block of xt in this launch; row length of dwacc
+  int64_t kbv;                 // blocks of 128 columns per tile of 256 rows of G
   int RT, CT, KT;
 };
 
@@ -530,9 +527,11 @@ __global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
   }
   __syncthreads();
   v16f acc[4][4];
-  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, false, 2>(p.xt + ((int64_t)rt * p.kbn + p.kb0) * BLOCKED_KSTEP, BK, p.ghat_t + (int64_t)ct * p.kbw * BLOCKED_KSTEP, BK, p.KT,
-                                                        smem, acc, ct & 7, 2 * (rt & 3), __builtin_amdgcn_readfirstlane(wave), NoHook(), 0, 0,
-                                                        lsc + __builtin_amdgcn_readfirstlane(wb) * p.KT);
+  // B = G with K (rows i) as the slow index: the 128 rows of a K block are half a tile of G, the 256 columns of this dW
+  // tile its column blocks 2 ct and 2 ct + 1 (BLOCKED_KSTEP apart); from one tile of G to the next kbv blocks
+  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, true, 2>(p.xt + ((int64_t)rt * p.kbn + p.kb0) * BLOCKED_KSTEP, BK, p.ghat_t + (int64_t)(2 * ct) * BLOCKED_KSTEP, BLOCKED_KSTEP, p.KT,
+                                                       smem, acc, ct & 7, 2 * (rt & 3), __builtin_amdgcn_readfirstlane(wave), NoHook(), 128 * BK, p.kbv * BLOCKED_KSTEP,
+                                                       lsc + __builtin_amdgcn_readfirstlane(wb) * p.KT);
   const int jbase = rt * 256 + wa * 128 + 4 * (lane >> 5);
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
@@ -549,12 +548,6 @@ __global__ __launch_bounds__(256) void bwd_dw_kernel(DwParams p) {
   }
 }
 
-// a pointer that is the same in every lane, moved to scalar registers
-__device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* q) {
-  const uint64_t u = (uint64_t)(uintptr_t)q;
-  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)u), hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(u >> 32));
-  return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
-}
 // The tiles of the last, partly filled round of dW (tile0 .. tile0 + ntail - 1 of the round-robin order), shared out
 // along K: a tile's K loop is kp pairs of K blocks long, all of them together W = ntail * kp pairs, and workgroup g takes
 // pairs [g share, (g + 1) share) of that line -- the end of one tile and the beginning of the next, when its range
@@ -592,10 +585,10 @@ __global__ __launch_bounds__(256) void bwd_dw_tail_kernel(DwParams p, DwTail tl)
   }
   __syncthreads();
   v16f acc[4][4];
-  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, false, 2>(uniform_ptr(p.xt + ((int64_t)rt * p.kbn + p.kb0 + 2 * k0) * BLOCKED_KSTEP), BK,
-                                                        uniform_ptr(p.ghat_t + ((int64_t)ct * p.kbw + 2 * k0) * BLOCKED_KSTEP), BK,
-                                                        KD, smem, acc, ct & 7, 2 * (rt & 3), __builtin_amdgcn_readfirstlane(wave), NoHook(), 0, 0,
-                                                        lsc + __builtin_amdgcn_readfirstlane(wb) * KD);
+  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, true, 2>(uniform_ptr(p.xt + ((int64_t)rt * p.kbn + p.kb0 + 2 * k0) * BLOCKED_KSTEP), BK,
+                                                       uniform_ptr(p.ghat_t + ((int64_t)k0 * p.kbv + 2 * ct) * BLOCKED_KSTEP), BLOCKED_KSTEP,
+                                                       KD, smem, acc, ct & 7, 2 * (rt & 3), __builtin_amdgcn_readfirstlane(wave), NoHook(), 128 * BK, p.kbv * BLOCKED_KSTEP,
+                                                       lsc + __builtin_amdgcn_readfirstlane(wb) * KD);
   float* dst0 = tl.buf + (size_t)(g + tt) * 65536 + (wa * 128 + 4 * (lane >> 5)) * 256 + wb * 128 + (lane & 31);
 #pragma unroll
   for (int b = 0; b < 4; ++b)

@@ -135,11 +135,10 @@ __global__ __launch_bounds__(256) void floor_dx_kernel(DxParams p, float* __rest
   }
   __syncthreads();
   v16f acc[4][4];
-  const int64_t bpair = p.kbw * BLOCKED_KSTEP;
-  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, true, 1>(p.wq + (int64_t)ct * (p.Vp / BK) * BLOCKED_KSTEP, BK,
-                                                       p.ghat_t + 2 * (int64_t)rt * BLOCKED_KSTEP, BLOCKED_KSTEP, KD, smem, acc,
-                                                       2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave), NoHook(), 128 * BK, bpair,
-                                                       lsc + __builtin_amdgcn_readfirstlane(wb) * KD);
+  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, false, 1>(p.wq + (int64_t)ct * (p.Vp / BK) * BLOCKED_KSTEP, BK,
+                                                        p.ghat_t + (int64_t)rt * (p.Vp / BK) * BLOCKED_KSTEP, BK, KD, smem, acc,
+                                                        2 * (rt & 3), ct & 7, __builtin_amdgcn_readfirstlane(wave), NoHook(), 0, 0,
+                                                        lsc + __builtin_amdgcn_readfirstlane(wb) * KD);
   out[(int64_t)blockIdx.x * 256 + threadIdx.x] = acc_sum(acc);
   floor_clock(clk, c0, r0);
 }
@@ -157,9 +156,9 @@ __global__ __launch_bounds__(256) void floor_dw_kernel(DwParams p, float* __rest
   }
   __syncthreads();
   v16f acc[4][4];
-  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, false, 2>(p.xt + ((int64_t)rt * p.kbn + p.kb0) * BLOCKED_KSTEP, BK, p.ghat_t + (int64_t)ct * p.kbw * BLOCKED_KSTEP, BK, p.KT,
-                                                        smem, acc, ct & 7, 2 * (rt & 3), __builtin_amdgcn_readfirstlane(wave), NoHook(), 0, 0,
-                                                        lsc + __builtin_amdgcn_readfirstlane(wb) * p.KT);
+  mfma_mainloop<false, NoHook, BLOCKED_KSTEP, true, 2>(p.xt + ((int64_t)rt * p.kbn + p.kb0) * BLOCKED_KSTEP, BK, p.ghat_t + (int64_t)(2 * ct) * BLOCKED_KSTEP, BLOCKED_KSTEP, p.KT,
+                                                       smem, acc, ct & 7, 2 * (rt & 3), __builtin_amdgcn_readfirstlane(wave), NoHook(), 128 * BK, p.kbv * BLOCKED_KSTEP,
+                                                       lsc + __builtin_amdgcn_readfirstlane(wb) * p.KT);
   out[(int64_t)blockIdx.x * 256 + threadIdx.x] = acc_sum(acc);
   floor_clock(clk, c0, r0);
 }

@@ -77,7 +77,7 @@ static inline SavedLayout saved_layout(int64_t N, int64_t d, int64_t V, int n_pr
   L.w_total = o;
   L.total = L.x_total + L.w_total;
   o = 0;
-  L.rel_g = take((size_t)L.Vp * L.Np);                          // G^T, Vp rows, K = Np, tile by tile
+  L.rel_g = take((size_t)L.Vp * L.Np);                          // G, Np rows, K = Vp, tile by tile
   L.rel_gexp = take((size_t)(L.Vp / 128) * (L.Np / 128) * 4);   // its block exponents
   L.g_total = o;
   return L;

@@ -127,4 +127,11 @@ __device__ __forceinline__ bool map_tile_rr(int bid, int RT, int CT, int& rt, in
 }
 static inline int map_tile_rr_grid(int RT, int CT) { return 256 * ((RT * CT + 255) / 256); }
 
+// a pointer that is the same in every lane, moved to scalar registers
+__device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* q) {
+  const uint64_t u = (uint64_t)(uintptr_t)q;
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)u), hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(u >> 32));
+  return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+
 }  // namespace sce

@@ -21,21 +21,16 @@ namespace sce {
 // the row's logits (fwd_sample_kernel) and undone exactly in rho_i.  The block exponent is taken after the boost, so
 // a poor estimate costs precision, never range.
 //
-// Layout: G^T, tile by tile ([v tile][K block of 128 rows i][256 v][128 i] bytes): the B operand of dW as it lies,
-// and of dX through the transposing LDS read.  Exponents: one dword per (128 v, 128 i), byte c for rows [32 c, 32 c + 32),
-// as gexp[v / 128][i / 128].
+// Layout: G, tile by tile ([tile of 256 rows i][block of 128 columns v][256 i][128 v] bytes): the B operand of dX as it
+// lies (rows i, K = v), and of dW (rows v, K = i) through the transposing LDS read.  Exponents: one dword per
+// (128 v, 128 i), byte c for rows [32 c, 32 c + 32), as gexp[v / 128][i / 128].
 //
-// One wave turns its 128 (v) x 128 (i) quadrant of a finished logit tile into its quadrant of the staging tile TT
-// ([256 v][STG_PITCH], rows i contiguous) in LDS and returns the dword of exponents of its four 32-row blocks.  The
-// transposition happens in registers: the four lanes of a quad hold four consecutive rows of the same four
-// columns, and two quad-permute + byte-permute steps turn that 4 x 4 byte block around.
+// One wave turns its 128 (v) x 128 (i) quadrant of a finished logit tile into its quadrant of G and returns the dword
+// of exponents of its four 32-row blocks.  A lane holds, of one row i, the columns 8 q + 4 h + (0..3) of every group of
+// 32 (q = 0..3, h = its half-wave): the two lanes of a row swap two of their four words (v_permlane32_swap) and then
+// hold 16 consecutive columns each, which go out as one 16-byte store.  No LDS is involved.
 // STATS: the forward pass's row statistics as well (sum of e^{z - cap}, largest raw logit and its column), kept in
 // `stat` (LDS, 12 floats per lane: [sum, max, argmax][4 row blocks], NTHREADS apart).
-// 256 + 32: 16-byte aligned, and a row is 72 dwords, 8 banks on from the row before: the dword writes of a wave (the 4 lanes
-// of a quad write 4 consecutive rows, its 8 quads consecutive dwords, the upper half-wave 4 rows on) then fall on
-// 32 h + 8 k + j, all 64 banks once.
-constexpr int STG_PITCH = 288;
-constexpr int STG_BYTES = 256 * STG_PITCH;                   // 73728
 
 // Maximum over the 64 lanes, in every lane.  The lane exchanges are LDS-crossbar swizzles with the pattern in the
 // instruction (xor 1 .. 16 within a half-wave), and one ds_bpermute across the halves whose address comes from
@@ -65,18 +60,17 @@ __device__ __forceinline__ float wave_max_dpp(float v) {
 // lam (LDS, wave-uniform base; per row block LAM_STRIDE floats apart, one float for each of LAM_LANES lanes): the row's
 // exponent boost (see fwd_sample_kernel).
 // want_argmax (uniform, STATS only): see the lookup of the maximum's column below.
+// gq: the wave's quadrant of G (128 rows i of 128 bytes, contiguous).
 template <bool EDGE, bool STATS, int LAM_STRIDE = NTHREADS, int LAM_LANES = 64>
 __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float k1, float c2, int vlim, int vabs0,
-                                                 uint8_t* TT, int wa, int wb, float* stat, const float* lam, bool want_argmax = true) {
+                                                 uint8_t* __restrict__ gq, int wa, int wb, float* stat, const float* lam, bool want_argmax = true) {
   const int lane = lane_id();
   const int vloc0 = wa * 128 + 4 * (lane >> 5);       // column (within the tile) of accumulator register 0 of block a = 0
-  const int k = lane & 3;
-  const uint32_t sel1 = (k & 1) ? 0x03070105u : 0x06020400u;
-  const uint32_t sel2 = (k & 2) ? 0x03020706u : 0x05040100u;
   uint32_t expword = 0;
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
-    const int iloc = wb * 128 + b * 32 + (lane & 31);        // row within the tile
+    __builtin_amdgcn_sched_barrier(0);      // the next row block's accumulator reads stay behind this one's work: moved up, they do not fit the registers
+    uint8_t* grow = gq + (b * 32 + (lane_id() & 31)) * BK + 16 * (lane_id() >> 5);      // the lane's row, its half of each 32 columns
     // the block's largest logit fixes its exponent: D * 2^s <= 2^(lg + s) <= 446 with lg = log2 e^{zmax - cap}
     float tmax = -INFINITY;
 #pragma unroll
@@ -123,17 +117,14 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
         for (int m = g0; m < g0 + NB; ++m) gg[m] *= rr[m] - rr[m] * rr[m];
         __builtin_amdgcn_sched_barrier(0);
       }
+      // words d[q] = columns 8 q + 4 h .. + 3 of this group of 32.  After the two swaps the lower half-wave holds
+      // (d0, d0', d1, d1') = columns 0..15 and the upper one (d2, d2', d3, d3') = columns 16..31 (x' = the other lane's x).
+      uint32_t d[4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int vloc = vloc0 + a * 32 + 8 * q;
-        const uint32_t w = cvt4_e4m3(gg[4 * q], gg[4 * q + 1], gg[4 * q + 2], gg[4 * q + 3]);
-        // 4 x 4 byte transpose inside the quad: lane k ends up with column vloc + k, rows (iloc & ~3) .. +3
-        const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xB1, 0xF, 0xF, true);     // lane ^ 1
-        const uint32_t x = __builtin_amdgcn_perm(p1, w, sel1);
-        const uint32_t p2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, true);     // lane ^ 2
-        const uint32_t yv = __builtin_amdgcn_perm(p2, x, sel2);
-        *reinterpret_cast<uint32_t*>(TT + (vloc + k) * STG_PITCH + (iloc & ~3)) = yv;
-      }
+      for (int q = 0; q < 4; ++q) d[q] = cvt4_e4m3(gg[4 * q], gg[4 * q + 1], gg[4 * q + 2], gg[4 * q + 3]);
+      const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+      const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+      *reinterpret_cast<v4i*>(grow + a * 32) = (v4i){(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
     }
     if (STATS) {
       stat[(0 + b) * NTHREADS] += ssum * fast_exp2(-cs);
@@ -163,18 +154,6 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
     }
   }
   return expword;
-}
-
-// The wave's quadrant of the staging tile (128 columns v x 128 rows i) is one contiguous 16 KB run of G^T: out in
-// 16-byte stores.  A wave reads only what it wrote itself, so no barrier is needed between forming and storing.
-__device__ __forceinline__ void store_dlogits_quadrant(const uint8_t* TT, uint8_t* gcol, int wa, int wb) {
-  const int lane = lane_id();
-  const uint8_t* tq = TT + wa * 128 * STG_PITCH + wb * 128;
-#pragma unroll
-  for (int n = 0; n < 16; ++n) {
-    const int cidx = lane + 64 * n, row = cidx >> 3, col = (cidx & 7) * 16;
-    *reinterpret_cast<v4i*>(gcol + row * BK + col) = *reinterpret_cast<const v4i*>(tq + row * STG_PITCH + col);
-  }
 }
 
 }  // namespace sce

@@ -14,12 +14,12 @@ struct FwdParams {
   float4* partials;        // [S][Np]: sum exp(z - cap), max u, argmax u (bits), unused
   const int64_t* targets;  // (N,)
   float* s_uy;             // [n_predict][Np]: raw logit u at the target of (offset, row), written by the workgroup that meets it
-  uint8_t* ghat_t;         // EMIT: G^T, all Np rows (K blocks per v tile: kbw)
+  uint8_t* ghat_t;         // EMIT: G, all Np rows, tile by tile (kbv blocks of 128 columns per tile of 256 rows)
   uint32_t* gexp;          // EMIT: its block exponents [Vp / 128][kbw]
   const float* lam;        // EMIT: exponent boost of every row
   int64_t ignore_index;
   int64_t dp, ldx;         // K extent and row stride of xq / wqt
-  int64_t kbw;
+  int64_t kbw, kbv;        // blocks of 128 rows (the exponents' row stride) and of 128 columns
   int N, V, Np, RT, CT, S, n_predict;      // V: columns that take part; CT: column tiles walked (EMIT: all of Vp / 256)
   float sc;                // x_s * w_s
   float k1;                // x_s * w_s * 2 log2(e) / cap : exp2(acc * k1) = e^{2u/cap}
@@ -190,17 +190,15 @@ __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct,
   }
 }
 
-// LDS of the forward kernel: the two K slots; with EMIT the staging tile of the dlogits in the second slot (reaching
-// 4 KB beyond it); the row statistics of the workgroup's walk (12 values per lane, and the boosts of its rows: kept in registers they are spilled
-// around the main loop, and the reload -- a vector memory load -- makes the epilogue wait for the tile loads that were
-// just put in flight for the next tile); the targets of the workgroup's 256 rows.
-constexpr int FWD_STAGE_OFF = SLOT_BYTES;
+// LDS of the forward kernel: the two K slots; the row statistics of the workgroup's walk (12 values per lane, and the boosts of
+// its rows: kept in registers they are spilled around the main loop, and the reload -- a vector memory load -- makes the
+// epilogue wait for the tile loads that were just put in flight for the next tile); the targets of the workgroup's 256 rows.
 constexpr int FWD_STAT_OFF = SMEM_MAX - 4096 - 16 * 4 * NTHREADS;      // 12 statistics and the boosts of the lane's 4 rows
 constexpr int FWD_TGT_OFF = SMEM_MAX - 4096;
 constexpr int SMEM_FWD = SMEM_MAX;
-static_assert(FWD_STAGE_OFF + STG_BYTES <= FWD_STAT_OFF, "staging tile and row statistics overlap");
+static_assert(SMEM_BYTES <= FWD_STAT_OFF, "K slots and row statistics overlap");
 
-// EMIT: the epilogue also leaves the block-scaled dlogits of the tile in G^T (see form_dlogits), for a backward pass
+// EMIT: the epilogue also leaves the block-scaled dlogits of the tile in G (see form_dlogits), for a backward pass
 // that does not compute the logits again.
 // BF16 (without EMIT): bf16 operands, logits rounded to bf16 as the eager head's GEMM returns them (forward only).
 template <bool EMIT, bool BF16 = false>
@@ -233,26 +231,23 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
   const int KT = (int)(p.dp / BK);
   // of the workgroups that start together on this XCD, those with the same split share the W tiles, those with the same rt the X rows
   const int rot_a = 2 * (rt & 3), rot_b = s & 7;
-  // the first K blocks of the next tile travel while the epilogue of this one runs (it does not touch the K slots;
-  // with EMIT it uses the second one, so only the first block travels and the rest follows after the epilogue)
+  // the first K blocks of the next tile travel while the epilogue of this one runs (it does not touch the K slots)
   if (ct0 < ct1) mfma_prefetch(p.wqt + (int64_t)ct0 * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
   for (int ct = ct0; ct < ct1; ++ct) {
-    mfma_mainloop<true, NoHook, BK, false, 0, BF16>(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, Bg, p.ldx, KT, smem, acc, rot_a, rot_b, wave,
-                                                    NoHook(), 0, 0, nullptr, EMIT && ct > ct0);
-    const uint8_t* Anext = p.wqt + (int64_t)(ct + 1) * 256 * p.ldx;
-    if (ct + 1 < ct1) mfma_prefetch<EMIT ? 1 : 3>(Anext, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
+    mfma_mainloop<true, NoHook, BK, false, 0, BF16>(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, Bg, p.ldx, KT, smem, acc, rot_a, rot_b, wave);
+    if (ct + 1 < ct1) mfma_prefetch(p.wqt + (int64_t)(ct + 1) * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
     float* stat = reinterpret_cast<float*>(smem + FWD_STAT_OFF) + wave * 64 + lane_id();
     const int vbase = ct * 256 + wa * 128 + 4 * (lane_id() >> 5);
     const int* tgt = reinterpret_cast<const int*>(smem + FWD_TGT_OFF) + wb * 128;
     if (EMIT) {
       take_target_logits<true, true, true, 256>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2, p.em2cap);
       const int vlim = p.V - ct * 256;
-      uint8_t* TT = smem + FWD_STAGE_OFF;
+      // the wave's quadrant of G: tile of rows rt, block of columns 2 ct + wa, rows 128 wb on
+      uint8_t* gq = p.ghat_t + ((int64_t)rt * p.kbv + 2 * ct + wa) * BLOCKED_KSTEP + wb * 128 * BK;
       uint32_t ew;
       const float* lam = reinterpret_cast<const float*>(smem + FWD_STAT_OFF) + 12 * NTHREADS + wave * 64;
-      if (vlim < 256) ew = form_dlogits<true, true>(acc, p.k1, p.c2, vlim, vbase, TT, wa, wb, stat, lam, p.want_argmax != 0);
-      else ew = form_dlogits<false, true>(acc, p.k1, p.c2, vlim, vbase, TT, wa, wb, stat, lam, p.want_argmax != 0);
-      store_dlogits_quadrant(TT, p.ghat_t + ((int64_t)ct * p.kbw + 2 * rt + wb) * BLOCKED_KSTEP + wa * 128 * BK, wa, wb);
+      if (vlim < 256) ew = form_dlogits<true, true>(acc, p.k1, p.c2, vlim, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0);
+      else ew = form_dlogits<false, true>(acc, p.k1, p.c2, vlim, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0);
       if (lane_id() == 0) p.gexp[(int64_t)(2 * ct + wa) * p.kbw + 2 * rt + wb] = ew;
     } else {
       float sum[4], amax[4];
@@ -278,13 +273,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
       }
     }
     if (!EMIT) take_target_logits<true, false, false, 256>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, nullptr, 0.f, 0.f, 0.f);
-    if (EMIT && ct + 1 < ct1) {
-      // every wave has read its part of the staging tile (its stores have their data) before the second K slot fills again
-      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      mfma_prefetch<2>(Anext, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
-    }
   }
-  if (EMIT) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");     // the staging tile gives way to the reduction below
   float sum[4], amax[4];
   int uarg[4];
   const int lane = lane_id();

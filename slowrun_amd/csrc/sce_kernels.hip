@@ -9,7 +9,7 @@
 //             fwd_kernel: 256x256 logit tiles on v_mfma_f32_32x32x64_f8f6f4; the epilogue keeps per-row
 //             sum exp(z - cap), the target logits and (on request) max/argmax of u; the logits never leave
 //             the chip.  With dlogits_from_forward it also leaves D = (1 - t^2) exp(z - cap) as e4m3 bytes
-//             with one power-of-two exponent per 32 rows x 128 columns (G^T, tile by tile), the targets'
+//             with one power-of-two exponent per 32 rows x 128 columns (G, tile by tile), the targets'
 //             entries zero.  Partials per (row, V-split) -> combine.
 //   backward: the dlogits as forward left them, or formed again panel by panel from recomputed logit tiles
 //             (bwd_recompute_kernel, same format); dX = rho_row * D W_q^T and dW = (rho X_q)^T D run on the
@@ -499,7 +499,7 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
   FwdParams p;
   p.xq = xq; p.wqt = wqt; p.partials = (float4*)ws;
   p.targets = a->targets; p.ignore_index = a->ignore_index; p.n_predict = a->shape.n_predict; p.s_uy = (float*)(sv + S.off_zy);
-  p.ghat_t = emit ? gbase + S.rel_g : nullptr; p.gexp = emit ? (uint32_t*)(gbase + S.rel_gexp) : nullptr; p.kbw = S.Np / BK;
+  p.ghat_t = emit ? gbase + S.rel_g : nullptr; p.gexp = emit ? (uint32_t*)(gbase + S.rel_gexp) : nullptr; p.kbw = S.Np / BK; p.kbv = S.Vp / BK;
   p.dp = S.dp; p.ldx = S.ldx; p.N = (int)N; p.V = (int)Vl; p.Np = (int)S.Np; p.RT = RT; p.CT = CTw; p.S = nsplit;
   p.sc = bf16ops ? 1.0f : (float)a->x_s * (float)a->w_s; p.k1 = p.sc * 2.0f * LOG2E / a->cap; p.c2 = -2.0f * a->cap * LOG2E; p.ic2 = 1.0f / p.c2; p.em2cap = expf(-2.0f * a->cap);
   p.dc = bf16ops ? nullptr : dcp;
@@ -679,7 +679,7 @@ extern "C" int sce_backward(const sce_args* a) {
   // dX of the rows [p0, p0 + prow) (a multiple of 256), the dlogits buffer standing for rows from gorg on
   auto dx_params = [&](int64_t p0, int64_t prow, int64_t gorg) {
     DxParams q;
-    q.wq = wq; q.ghat_t = ghat_t + ((p0 - gorg) / BK) * BLOCKED_KSTEP; q.gexp = gexp + (p0 - gorg) / BK; q.kbw = gkb; q.wqt = wqt; q.rho = rho + p0; q.hcoef = hcoef + p0; q.targets = a->targets + p0;
+    q.wq = wq; q.ghat_t = ghat_t + ((p0 - gorg) / 256) * (S.Vp / BK) * BLOCKED_KSTEP; q.gexp = gexp + (p0 - gorg) / BK; q.kbw = gkb; q.wqt = wqt; q.rho = rho + p0; q.hcoef = hcoef + p0; q.targets = a->targets + p0;
     q.dx_ld = a->dx_ld; q.Vp = S.Vp; q.ldx = S.ldx; q.Np = S.Np; q.dq = S.dq; q.RT = (int)(prow / 256); q.CT = CTd;
     q.n_predict = K; q.rows_left = (int)(N - p0 > 0 ? N - p0 : 0);
     q.rows = (int)((N - p0 < prow) ? (N - p0 > 0 ? N - p0 : 0) : prow); q.d = (int)d; q.V = (int)Vl; q.w_s = (float)a->w_s; q.dc = dcp;
@@ -715,8 +715,8 @@ extern "C" int sce_backward(const sce_args* a) {
   auto dw_launch = [&](int64_t w0, int64_t gathered, int64_t gorg, bool last) {
     DwParams wp;
     const int part = launch < nparts ? launch : nparts - 1;
-    wp.xt = xt; wp.ghat_t = ghat_t + ((w0 - gorg) / BK) * BLOCKED_KSTEP; wp.gexp = gexp + (w0 - gorg) / BK; wp.dwacc = (float*)((uint8_t*)dwacc + (size_t)part * B.part_stride);
-    wp.kbn = S.Np / BK; wp.kbw = gkb; wp.kb0 = w0 / BK; wp.Vp = S.Vp;
+    wp.xt = xt; wp.ghat_t = ghat_t + ((w0 - gorg) / 256) * (S.Vp / BK) * BLOCKED_KSTEP; wp.gexp = gexp + (w0 - gorg) / BK; wp.dwacc = (float*)((uint8_t*)dwacc + (size_t)part * B.part_stride);
+    wp.kbn = S.Np / BK; wp.kbw = gkb; wp.kb0 = w0 / BK; wp.Vp = S.Vp; wp.kbv = S.Vp / BK;
     wp.RT = CTd; wp.CT = CTv; wp.KT = (int)(gathered / BK);
     {
       KernelTimer tm(SCE_K_DW, st);
@@ -750,7 +750,7 @@ extern "C" int sce_backward(const sce_args* a) {
       const int64_t gorg = w0;                                    // the row that K block 0 of the dlogits buffer stands for
       RecomputeParams rp;
       rp.xq = xq + p0 * S.ldx; rp.wqt = wqt; rp.ghat_t = ghat_t; rp.gexp = gexp; rp.rowinfo = rowinfo + p0; rp.Np = S.Np; rp.n_predict = K;
-      rp.dp = S.dp; rp.ldx = S.ldx; rp.kbw = gkb; rp.kb0 = (p0 - gorg) / BK; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2; rp.dc = dcp;
+      rp.dp = S.dp; rp.ldx = S.ldx; rp.kbw = gkb; rp.kbv = S.Vp / BK; rp.kb0 = (p0 - gorg) / BK; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2; rp.dc = dcp;
       {
         KernelTimer tm(SCE_K_RECOMPUTE, st);
         bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_RECOMPUTE, st>>>(rp);
@@ -923,13 +923,13 @@ extern "C" int sce_bench_floor(const sce_args* a, int32_t which, int32_t reps, v
       for (int64_t p0 = 0; p0 < S.Np; p0 += P) {
         const int64_t prow = (S.Np - p0 < P) ? (S.Np - p0) : P;
         DxParams p = {};
-        p.wq = wq; p.ghat_t = ghat_t + (p0 / BK) * BLOCKED_KSTEP; p.gexp = gexp + p0 / BK; p.kbw = S.Np / BK; p.Vp = S.Vp;
+        p.wq = wq; p.ghat_t = ghat_t + (p0 / 256) * (S.Vp / BK) * BLOCKED_KSTEP; p.gexp = gexp + p0 / BK; p.kbw = S.Np / BK; p.Vp = S.Vp;
         p.RT = (int)(prow / 256); p.CT = CTd;
         floor_dx_kernel<<<map_tile_grid(p.RT, CTd), NTHREADS, smem_scaled((int)(S.Vp / BK), 0), st>>>(p, out, clk);
       }
     } else {
       DwParams p = {};
-      p.xt = (const uint8_t*)a->workspace + B.off_xt; p.ghat_t = ghat_t; p.gexp = gexp; p.kbn = S.Np / BK; p.kbw = S.Np / BK; p.kb0 = 0; p.Vp = S.Vp;
+      p.xt = (const uint8_t*)a->workspace + B.off_xt; p.ghat_t = ghat_t; p.gexp = gexp; p.kbn = S.Np / BK; p.kbw = S.Np / BK; p.kb0 = 0; p.Vp = S.Vp; p.kbv = S.Vp / BK;
       p.RT = CTd; p.CT = CTv; p.KT = (int)(S.Np / BK);
       floor_dw_kernel<<<map_tile_rr_grid(CTd, CTv), NTHREADS, smem_scaled(p.KT, 0), st>>>(p, out, clk);
     }

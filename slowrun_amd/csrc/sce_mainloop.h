@@ -154,7 +154,7 @@ struct NoHook { __device__ __forceinline__ void operator()(int) const {} };
 // The exponents of a tile wait in LDS behind the two K slots, one dword per K block for each half (wb) of the B rows:
 //   SCALE = 1: byte b of the dword of K block k belongs to the wave's B rows [32 b, 32 b + 32) (dX: B = dlogits, K = v);
 //   SCALE = 2: byte c of the dword of K block k belongs to K values [32 c, 32 c + 32) of that block, for all of the
-//              wave's 128 B rows (dW: B = dlogits^T, K = i).
+//              wave's 128 B rows (dW: B = the columns of the dlogits, K = i, TRB).
 // The A operand goes in with exponent 127 (factor 1).  lds_scale points at the wave's KD dwords.
 template <int OPB>
 __device__ __forceinline__ v16f mfma_fp8_scaled(const v8i& a, const v8i& b, const v16f& c, int sa, int sb) {
@@ -169,9 +169,6 @@ __device__ __forceinline__ v16f mfma_fp8_scaled_sel(int opb, const v8i& a, const
   }
 }
 
-// stores_between (PREFETCHED only, uniform): the caller issued at least 16 vector memory stores between its prefetch of
-// K block 0 and its 8 loads of K block 1 (mfma_prefetch<1>, the stores, mfma_prefetch<2>); they are younger than
-// block 0, so the first wait may leave them in flight.
 // BF16: the operands are bf16 (64 K values per 128-byte block) and each step is two v_mfma_f32_32x32x16_bf16, on the
 // first and the second 16 bytes of the lanes' fragments; everything else -- loads, LDS, the schedule in bytes -- is the same.
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
@@ -185,8 +182,7 @@ template <bool PREFETCHED = false, class Hook = NoHook, int KSTEP = BK, bool TRB
 __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, int64_t lda,
                                               const uint8_t* __restrict__ Bg, int64_t ldb, int KD,
                                               uint8_t* smem, v16f (&acc)[4][4], int rot_a, int rot_b, int wave, Hook&& hook = NoHook(),
-                                              int64_t bk1_arg = 0, int64_t bk2_arg = 0, const uint32_t* lds_scale = nullptr,
-                                              bool stores_between = false) {
+                                              int64_t bk1_arg = 0, int64_t bk2_arg = 0, const uint32_t* lds_scale = nullptr) {
   const int lane = lane_id();
   const int wa = wave >> 1, wb = wave & 1;
   const int64_t bk1 = TRB ? bk1_arg : (int64_t)KSTEP, bk2 = TRB ? bk2_arg : (int64_t)(2 * KSTEP);
@@ -204,11 +200,13 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
       // each of the group's 8 rows: 8 consecutive K values of its own N.  Four reads give the lane its 32 K values.
       // Group g = lane / 16 holds N chunk 2 b + (g & 1) and K half g / 2; the chunks of a row are XOR-swizzled by
       // (K row & 7) = j >> 1 (the loader stores them so).
+      // Which 32 of the sub-step's 64 K rows a lane takes: registers 4 u .. 4 u + 3 hold rows 32 h + 16 u .. + 15, or, where the
+      // exponent changes along K (SCALE = 2, see below), rows 32 u + 16 h .. + 15 -- the same choice as for the other operand.
       const int b = n - 4, g = lane >> 4, j = lane & 15;
-      const uint8_t* s = smem + slot * SLOT_BYTES + TM * BK + wb * 128 * BK + (64 * half + 32 * (g >> 1) + (j >> 1)) * BK +
-                         (((2 * b + (g & 1)) ^ (j >> 1)) << 4) + 8 * (j & 1);
-      const v2i r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)(s + (2 * u) * 8 * BK));
-      const v2i r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)(s + (2 * u + 1) * 8 * BK));
+      const int krow = 64 * half + (SCALE == 2 ? 32 * u + 16 * (g >> 1) : 32 * (g >> 1) + 16 * u) + (j >> 1);
+      const uint8_t* s = smem + slot * SLOT_BYTES + TM * BK + wb * 128 * BK + krow * BK + (((2 * b + (g & 1)) ^ (j >> 1)) << 4) + 8 * (j & 1);
+      const v2i r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)(s));
+      const v2i r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)(s + 8 * BK));
       q = (v4i){r0[0], r0[1], r1[0], r1[1]};
     } else {
       // Which 32 of the sub-step's 64 K bytes a lane takes does not matter as long as both operands agree -- except
@@ -234,9 +232,9 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
 #pragma unroll
     for (int n = 0; n < AHEAD_LOADS; ++n) ld.template issue<1>(n, Ag + KSTEP, Bg + bk1);
   }
-  // K block 0 has landed once at most the loads of block 1 (and the 16 stores a caller put between the two) are in flight
-  if (PREFETCHED && stores_between) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(AHEAD_LOADS + 16) : "memory");
-  else asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(AHEAD_LOADS) : "memory");
+  // K block 0 has landed once at most the loads of block 1 are in flight (vector memory operations that a caller issued
+  // after its prefetch -- stores of an epilogue -- are younger still: the wait then covers block 1 as well, no more)
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(AHEAD_LOADS) : "memory");
   v8i fa[2][4], fb[2][4];
   runits(0, 0, 0, 16, fa[0], fb[0]);
   // block scales of the current pair of K blocks and of the next one (read one pair ahead)
