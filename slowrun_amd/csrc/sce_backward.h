@@ -182,15 +182,25 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p_in
     }
   }
   v16f acc[4][4];
-  mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 2 * (rt & 3), ct & 7, wave);
+  // (as in the forward kernel: the last pair's MFMAs of row blocks 1 - 3 ride along with the epilogues of row blocks 0 and 1)
+  mfma_mainloop<false, NoHook, BK, false, 0, false, true>(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 2 * (rt & 3), ct & 7, wave);
+  DeferredTail deferred(smem, wa, wb);
+  auto tail = [&](int b, int k) { deferred(acc, b, k); };
   const int vlim = p.V - ct * 256;           // columns >= vlim of this tile do not exist
+  const bool ragged = vlim < 256;
   const float* lam = reinterpret_cast<const float*>(smem + SMEM_BYTES) + wave * (ROWINFO_PLANES * 128);     // row block b: 32 floats on
   const int* tgt = reinterpret_cast<const int*>(smem + SMEM_BYTES) + wave * (ROWINFO_PLANES * 128) + 128;
-  take_target_logits<false, true, false, 128>(acc, tgt, p.n_predict, ct * 256 + wa * 128, 0, 0.f, nullptr, 0, nullptr, 0.f, 0.f, 0.f);
-  uint32_t ew;
   uint8_t* gq = const_cast<uint8_t*>(uniform_ptr(p.ghat_t + ((p.kb0 / 2 + rt) * p.kbv + 2 * ct + wa) * BLOCKED_KSTEP + wb * 128 * BK));      // the wave's quadrant of G
-  if (vlim < 256) ew = form_dlogits<true, false, 32, 32>(acc, p.k1, p.c2, vlim, 0, gq, wa, wb, nullptr, lam);
-  else ew = form_dlogits<false, false, 32, 32>(acc, p.k1, p.c2, vlim, 0, gq, wa, wb, nullptr, lam);
+  const int col0 = ct * 256 + wa * 128;
+  if (ragged) strike_columns_beyond<0, 1>(acc, vlim, wa);
+  take_target_logits<false, true, false, 128, 0, 1>(acc, tgt, p.n_predict, col0, 0, 0.f, nullptr, 0, nullptr, 0.f, 0.f, 0.f);
+  uint32_t ew = form_dlogits<false, false, 32, 32, 0, 1>(acc, p.k1, p.c2, vlim, 0, gq, wa, wb, nullptr, lam, false, tail);
+  if (ragged) strike_columns_beyond<1, 2>(acc, vlim, wa);
+  take_target_logits<false, true, false, 128, 1, 2>(acc, tgt, p.n_predict, col0, 0, 0.f, nullptr, 0, nullptr, 0.f, 0.f, 0.f);
+  ew |= form_dlogits<false, false, 32, 32, 1, 2>(acc, p.k1, p.c2, vlim, 0, gq, wa, wb, nullptr, lam, false, tail);
+  if (ragged) strike_columns_beyond<2, 4>(acc, vlim, wa);
+  take_target_logits<false, true, false, 128, 2, 4>(acc, tgt, p.n_predict, col0, 0, 0.f, nullptr, 0, nullptr, 0.f, 0.f, 0.f);
+  ew |= form_dlogits<false, false, 32, 32, 2, 4>(acc, p.k1, p.c2, vlim, 0, gq, wa, wb, nullptr, lam, false);
   if (lane_id() == 0) p.gexp[(int64_t)(2 * ct + wa) * p.kbw + p.kb0 + 2 * rt + wb] = ew;
 }
 

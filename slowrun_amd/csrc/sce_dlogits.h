@@ -57,18 +57,46 @@ __device__ __forceinline__ float wave_max_dpp(float v) {
   return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
 }
 
+// The other way to deal with a tile that reaches beyond the vocabulary (columns >= vlim of the tile do not exist): their
+// accumulators are set to -inf before the epilogue, which then needs no EDGE variant -- such a logit reads as z = -cap, its
+// stored value is exactly 0, it cannot be a block's maximum, and what it adds to the row sum, e^{-2 cap} a piece, is
+// taken out of `stat` here (a caller without row statistics passes none).  Row blocks [B0, B1).
+template <int B0, int B1>
+__device__ __forceinline__ void strike_columns_beyond(v16f (&acc)[4][4], int vlim, int wa, float* stat = nullptr, float em2cap = 0.f) {
+  const int vloc0 = wa * 128 + 4 * (lane_id() >> 5);
+  int cnt = 0;
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const bool out = vloc0 + a * 32 + 8 * (r >> 2) + (r & 3) >= vlim;
+      cnt += out ? 1 : 0;
+#pragma unroll
+      for (int b = B0; b < B1; ++b) acc[a][b][r] = out ? -INFINITY : acc[a][b][r];
+    }
+  if (stat) {
+#pragma unroll
+    for (int b = B0; b < B1; ++b) stat[(0 + b) * NTHREADS] -= (float)cnt * em2cap;
+  }
+}
+
 // lam (LDS, wave-uniform base; per row block LAM_STRIDE floats apart, one float for each of LAM_LANES lanes): the row's
 // exponent boost (see fwd_sample_kernel).
 // want_argmax (uniform, STATS only): see the lookup of the maximum's column below.
 // gq: the wave's quadrant of G (128 rows i of 128 bytes, contiguous).
-template <bool EDGE, bool STATS, int LAM_STRIDE = NTHREADS, int LAM_LANES = 64>
+// B0, B1: the row blocks [B0, B1) only (the returned dword has their bytes).
+// hook(b, k), k = 0..31: called between the stages of row block b's arithmetic (four to a batch of eight values): a place
+// for a caller's matrix instructions on other accumulators.
+template <bool EDGE, bool STATS, int LAM_STRIDE = NTHREADS, int LAM_LANES = 64, int B0 = 0, int B1 = 4, class Hook = NoHook>
 __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float k1, float c2, int vlim, int vabs0,
-                                                 uint8_t* __restrict__ gq, int wa, int wb, float* stat, const float* lam, bool want_argmax = true) {
+                                                 uint8_t* __restrict__ gq, int wa, int wb, float* stat, const float* lam, bool want_argmax = true,
+                                                 Hook&& hook = NoHook()) {
+  constexpr bool HOOKED = !std::is_same<typename std::decay<Hook>::type, NoHook>::value;
   const int lane = lane_id();
   const int vloc0 = wa * 128 + 4 * (lane >> 5);       // column (within the tile) of accumulator register 0 of block a = 0
   uint32_t expword = 0;
 #pragma unroll
-  for (int b = 0; b < 4; ++b) {
+  for (int b = B0; b < B1; ++b) {
     __builtin_amdgcn_sched_barrier(0);      // the next row block's accumulator reads stay behind this one's work: moved up, they do not fit the registers
     uint8_t* grow = gq + (b * 32 + (lane_id() & 31)) * BK + 16 * (lane_id() >> 5);      // the lane's row, its half of each 32 columns
     // the block's largest logit fixes its exponent: D * 2^s <= 2^(lg + s) <= 446 with lg = log2 e^{zmax - cap}
@@ -99,12 +127,15 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
 #pragma unroll
         for (int m = g0; m < g0 + NB; ++m) rr[m] = fast_exp2(acc[a][b][m] * k1);
         __builtin_amdgcn_sched_barrier(0);
+        if (HOOKED) { hook(b, 4 * (2 * a + g0 / NB)); __builtin_amdgcn_sched_barrier(0); }
 #pragma unroll
         for (int m = g0; m < g0 + NB; ++m) rr[m] = fast_rcp(rr[m] + 1.0f);
         __builtin_amdgcn_sched_barrier(0);
+        if (HOOKED) { hook(b, 4 * (2 * a + g0 / NB) + 1); __builtin_amdgcn_sched_barrier(0); }
 #pragma unroll
         for (int m = g0; m < g0 + NB; ++m) gg[m] = fast_exp2(fmaf(c2, rr[m], cs));
         __builtin_amdgcn_sched_barrier(0);
+        if (HOOKED) { hook(b, 4 * (2 * a + g0 / NB) + 2); __builtin_amdgcn_sched_barrier(0); }
         if (EDGE) {
 #pragma unroll
           for (int m = g0; m < g0 + NB; ++m) gg[m] = (vloc0 + a * 32 + 8 * (m >> 2) + (m & 3) >= vlim) ? 0.f : gg[m];
@@ -116,6 +147,7 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
 #pragma unroll
         for (int m = g0; m < g0 + NB; ++m) gg[m] *= rr[m] - rr[m] * rr[m];
         __builtin_amdgcn_sched_barrier(0);
+        if (HOOKED) { hook(b, 4 * (2 * a + g0 / NB) + 3); __builtin_amdgcn_sched_barrier(0); }
       }
       // words d[q] = columns 8 q + 4 h .. + 3 of this group of 32.  After the two swaps the lower half-wave holds
       // (d0, d0', d1, d1') = columns 0..15 and the upper one (d2, d2', d3, d3') = columns 16..31 (x' = the other lane's x).
@@ -134,7 +166,7 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
       // some lane of the 64 does in nearly every tile of a walk of a few dozen: a caller that does not ask for the argmax
       // is spared it.  (A flag at run time, not a template parameter: without the lookup in the code the register
       // allocation of the rest changes, and accumulators end up in scratch memory.)
-      if (want_argmax && __builtin_amdgcn_ballot_w64(tmax >= amax) != 0) {
+      if (want_argmax && __builtin_amdgcn_ballot_w64(tmax >= amax && tmax != -INFINITY) != 0) {
         if (tmax >= amax) {
           int targ = 0x7fffffff;
 #pragma unroll

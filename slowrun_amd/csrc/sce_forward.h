@@ -92,14 +92,15 @@ __device__ __forceinline__ bool target_valid(const int64_t* __restrict__ targets
 //        no part in the stored dlogits (its column is handled in fp32, see bwd_prep_kernel) and must not set the
 //        exponent of its block either -- a row the model is sure of would push its own other columns, and its
 //        neighbours', out of the 8 bits.
+// B0, B1: the row blocks [B0, B1) only.
 // STATS: with KNOCK, the row statistics (stat, as in form_dlogits) take the target's share here: e^{z_y - cap} into the
 //        sum, and the running maximum / argmax.
-template <bool STORE, bool KNOCK, bool STATS, int TGT_STRIDE>
+template <bool STORE, bool KNOCK, bool STATS, int TGT_STRIDE, int B0 = 0, int B1 = 4>
 __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int* tgt, int n_predict, int col0, int rowbase,
                                                    float sc, float* s_uy_tile, int Np, float* stat, float k1, float ic2, float em2cap) {
   const int lane = lane_id(), half = lane >> 5;
 #pragma unroll
-  for (int b = 0; b < 4; ++b) {
+  for (int b = B0; b < B1; ++b) {
     const int row = b * 32 + (lane & 31);
     float xk[4] = {0.f, 0.f, 0.f, 0.f};
     for (int k = 0; k < n_predict; ++k) {
@@ -234,20 +235,41 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
   // the first K blocks of the next tile travel while the epilogue of this one runs (it does not touch the K slots)
   if (ct0 < ct1) mfma_prefetch(p.wqt + (int64_t)ct0 * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
   for (int ct = ct0; ct < ct1; ++ct) {
-    mfma_mainloop<true, NoHook, BK, false, 0, BF16>(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, Bg, p.ldx, KT, smem, acc, rot_a, rot_b, wave);
-    if (ct + 1 < ct1) mfma_prefetch(p.wqt + (int64_t)(ct + 1) * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
+    if (EMIT) mfma_mainloop<true, NoHook, BK, false, 0, false, true>(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, Bg, p.ldx, KT, smem, acc, rot_a, rot_b, wave);
+    else mfma_mainloop<true, NoHook, BK, false, 0, BF16>(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, Bg, p.ldx, KT, smem, acc, rot_a, rot_b, wave);
+    auto prefetch = [&]() {
+      if (ct + 1 < ct1) mfma_prefetch(p.wqt + (int64_t)(ct + 1) * 256 * p.ldx, p.ldx, Bg, p.ldx, smem, rot_a, rot_b, wave);
+    };
+    if (!EMIT) prefetch();
     float* stat = reinterpret_cast<float*>(smem + FWD_STAT_OFF) + wave * 64 + lane_id();
     const int vbase = ct * 256 + wa * 128 + 4 * (lane_id() >> 5);
     const int* tgt = reinterpret_cast<const int*>(smem + FWD_TGT_OFF) + wb * 128;
     if (EMIT) {
-      take_target_logits<true, true, true, 256>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2, p.em2cap);
+      // The main loop has left 48 of the 64 MFMAs of its last pair of K blocks undone, those of row blocks 1 - 3; the pair
+      // is still in LDS.  They are issued one at a time between the stages of the epilogues of row blocks 0 and 1, where
+      // the matrix pipe would stand idle: during block 0's the 32 of blocks 1 and 2 (one at each of its 32 stage
+      // boundaries), during block 1's the 16 of block 3.  Only then are the slots free for the next tile's first K blocks.
+      DeferredTail deferred(smem, wa, wb);
+      auto tail = [&](int b, int k) { deferred(acc, b, k); };
       const int vlim = p.V - ct * 256;
       // the wave's quadrant of G: tile of rows rt, block of columns 2 ct + wa, rows 128 wb on
       uint8_t* gq = p.ghat_t + ((int64_t)rt * p.kbv + 2 * ct + wa) * BLOCKED_KSTEP + wb * 128 * BK;
-      uint32_t ew;
       const float* lam = reinterpret_cast<const float*>(smem + FWD_STAT_OFF) + 12 * NTHREADS + wave * 64;
-      if (vlim < 256) ew = form_dlogits<true, true>(acc, p.k1, p.c2, vlim, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0);
-      else ew = form_dlogits<false, true>(acc, p.k1, p.c2, vlim, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0);
+      const int col0 = ct * 256 + wa * 128, row0 = rt * 256 + wb * 128;
+      // (one code path for the epilogue: with a second one for the last tile of the vocabulary, each with its MFMAs, the
+      // accumulators are spilled; columns that do not exist are struck out of the finished accumulators instead)
+      const bool ragged = vlim < 256;
+      if (ragged) strike_columns_beyond<0, 1>(acc, vlim, wa, stat, p.em2cap);
+      take_target_logits<true, true, true, 256, 0, 1>(acc, tgt, p.n_predict, col0, row0, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2, p.em2cap);
+      uint32_t ew = form_dlogits<false, true, NTHREADS, 64, 0, 1>(acc, p.k1, p.c2, vlim, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, tail);
+      if (ragged) strike_columns_beyond<1, 2>(acc, vlim, wa, stat, p.em2cap);
+      take_target_logits<true, true, true, 256, 1, 2>(acc, tgt, p.n_predict, col0, row0, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2, p.em2cap);
+      ew |= form_dlogits<false, true, NTHREADS, 64, 1, 2>(acc, p.k1, p.c2, vlim, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, tail);
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // every wave has read its last fragment
+      prefetch();
+      if (ragged) strike_columns_beyond<2, 4>(acc, vlim, wa, stat, p.em2cap);
+      take_target_logits<true, true, true, 256, 2, 4>(acc, tgt, p.n_predict, col0, row0, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2, p.em2cap);
+      ew |= form_dlogits<false, true, NTHREADS, 64, 2, 4>(acc, p.k1, p.c2, vlim, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0);
       if (lane_id() == 0) p.gexp[(int64_t)(2 * ct + wa) * p.kbw + 2 * rt + wb] = ew;
     } else {
       float sum[4], amax[4];

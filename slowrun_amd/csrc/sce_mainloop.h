@@ -140,7 +140,10 @@ __device__ __forceinline__ void mfma_prefetch(const uint8_t* __restrict__ Ag, in
 
 // lda, ldb: row strides in bytes, multiples of 16, at most 2^24; KD = K / 128, even, >= 2;
 // rot_a, rot_b in [0, 8), uniform over the workgroup; wave: index of the wavefront in the workgroup (scalar).
-struct NoHook { __device__ __forceinline__ void operator()(int) const {} };
+struct NoHook {
+  __device__ __forceinline__ void operator()(int) const {}
+  __device__ __forceinline__ void operator()(int, int) const {}
+};
 
 // `hook(i)` is called after MFMA i (0..63) of every pair of K blocks: a place for vector ALU work that
 // does not depend on the accumulators (it runs while the matrix pipe is busy).
@@ -178,11 +181,16 @@ __device__ __forceinline__ v16f mfma_bf16_pair(const v8i& a, const v8i& b, v16f 
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a1), __builtin_bit_cast(v8bf, b1), c, 0, 0, 0);
 }
 
-template <bool PREFETCHED = false, class Hook = NoHook, int KSTEP = BK, bool TRB = false, int SCALE = 0, bool BF16 = false>
+// DEFER (plain fp8 only): of the last pair of K blocks only the MFMAs of B block 0 (accumulators acc[.][0]) are
+// issued; the other 48 are left to the caller, who finds the pair in the two LDS slots on return (lds_fragment) and
+// issues them (mfma_tail) between the vector instructions of its epilogue of the finished accumulators, where the
+// matrix pipe would otherwise stand idle.  Nothing may be loaded into the slots until that is done.
+template <bool PREFETCHED = false, class Hook = NoHook, int KSTEP = BK, bool TRB = false, int SCALE = 0, bool BF16 = false, bool DEFER = false>
 __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, int64_t lda,
                                               const uint8_t* __restrict__ Bg, int64_t ldb, int KD,
                                               uint8_t* smem, v16f (&acc)[4][4], int rot_a, int rot_b, int wave, Hook&& hook = NoHook(),
                                               int64_t bk1_arg = 0, int64_t bk2_arg = 0, const uint32_t* lds_scale = nullptr) {
+  static_assert(!DEFER || (!BF16 && SCALE == 0 && !TRB), "DEFER is for the plain fp8 loop");
   const int lane = lane_id();
   const int wa = wave >> 1, wb = wave & 1;
   const int64_t bk1 = TRB ? bk1_arg : (int64_t)KSTEP, bk2 = TRB ? bk2_arg : (int64_t)(2 * KSTEP);
@@ -291,7 +299,8 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
         }
       }
       const int sub = s >> 4, i = s & 15;
-      if (first && BLK == 0 && sub == 0) mm0(i); else mm(BLK, sub, i);
+      if (DEFER && !has2 && (i & 3) != 0) {}      // last pair, B blocks 1 - 3: the caller's
+      else if (first && BLK == 0 && sub == 0) mm0(i); else mm(BLK, sub, i);
       hook(32 * BLK + s);
       if (!(first && BLK == 0)) runits(BLK, 0, UNITS_N0 + ksum(KS.c0, s), KS.c0[s], fa[0], fb[0]);      // (the first block's came with the prologue)
       runits(BLK, 1, ksum(KS.r1, s), KS.r1[s], fa[1], fb[1]);
@@ -315,6 +324,14 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
   };
   const int P = KD >> 1;
   if (P == 1) {
+    if (DEFER) {       // the only pair is the last one: what it leaves undone starts from zero
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 1; b < 4; ++b)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+    }
     pair(true, false);
   } else {
     pair(true, true);
@@ -330,5 +347,66 @@ __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, in
   // all LDS reads of this tile are complete in every wave before the caller reuses the buffer
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
+
+// Reader of the fragments of the pair of K blocks in the two LDS slots, as the plain fp8 main loop reads them; the lane's
+// part of the addresses is computed once (lb[half][u]: the lane's row and the swizzled 16-byte chunks 2 h + u of the
+// 64-byte half `half` of a K block).
+struct TailReader {
+  const uint8_t* lb[2][2];
+  int wa, wb;
+  __device__ __forceinline__ TailReader(const uint8_t* smem, int wa_, int wb_) : wa(wa_), wb(wb_) {
+    const int lane = lane_id(), r = lane & 31, h = lane >> 5, sw = (r & 7) ^ ((r >> 3) & 1);
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int c0 = ((4 * half + 2 * h) ^ sw) * 16;
+      lb[half][0] = smem + r * BK + c0; lb[half][1] = smem + r * BK + (c0 ^ 16);
+    }
+  }
+  // fragment n (0 - 3: A block n, 4 - 7: B block n - 4) of sub-step `step` (0 - 3: K block step / 2, its half step % 2)
+  __device__ __forceinline__ v8i operator()(int step, int n) const {
+    const int off = (step >> 1) * SLOT_BYTES + (n < 4 ? wa * 128 * BK + n * 32 * BK : TM * BK + wb * 128 * BK + (n - 4) * 32 * BK);
+    const v4i q0 = *reinterpret_cast<const v4i*>(lb[step & 1][0] + off), q1 = *reinterpret_cast<const v4i*>(lb[step & 1][1] + off);
+    return (v8i){q0[0], q0[1], q0[2], q0[3], q1[0], q1[1], q1[2], q1[3]};
+  }
+};
+// The 48 MFMAs that a DEFER main loop has left undone, handed out one call at a time: a caller's epilogue of row block
+// 0 calls (acc, 0, k), k = 0..31, between the stages of its arithmetic and gets the 32 MFMAs of row blocks 1 and 2, one a
+// call; its epilogue of row block 1 calls (acc, 1, k), k = 0..31, and gets the 16 of row block 3 at every other call.
+// After that the LDS slots are free.  Every fragment is read two calls before its first use, into registers that the
+// MFMAs in between do not use: the A fragments alternate between fa[0] and fa[1], the B fragments of a sub-step between
+// fb[0] and fb[1].
+struct DeferredTail {
+  TailReader frag;
+  v8i fa[2], fb[2][2];
+  __device__ __forceinline__ DeferredTail(const uint8_t* smem, int wa, int wb) : frag(smem, wa, wb) {
+    fa[0] = frag(0, 0); fb[0][0] = frag(0, 5); fb[0][1] = frag(0, 6);
+  }
+  static __device__ __forceinline__ void mfma(const v8i& a, const v8i& b, v16f& c) {
+    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+  }
+  __device__ __forceinline__ void operator()(v16f (&acc)[4][4], int b, int k) {
+    if (b == 0) {
+      // MFMA k of 32: sub-step k / 8, A block (k % 8) / 2, row block 1 + k % 2
+      const int s = k >> 3, a = (k & 7) >> 1;
+      mfma(fa[a & 1], fb[s & 1][k & 1], acc[a][1 + (k & 1)]);
+      const int k2 = k + 2, s2 = k2 >> 3, a2 = (k2 & 7) >> 1;       // what MFMA k + 2 needs
+      if (k2 < 32) {
+        if ((k2 & 1) == 0) fa[a2 & 1] = frag(s2, a2);
+        if ((k2 & 7) == 0) { fb[s2 & 1][0] = frag(s2, 5); fb[s2 & 1][1] = frag(s2, 6); }
+      } else if (k2 == 32) {                                      // the first of row block 3's
+        fa[0] = frag(0, 0); fb[0][0] = frag(0, 7);
+      }
+    } else if (b == 1 && (k & 1)) {
+      // MFMA m = k / 2 of 16: sub-step m / 4, A block m % 4, row block 3
+      const int m = k >> 1, s = m >> 2, a = m & 3;
+      mfma(fa[a & 1], fb[s & 1][0], acc[a][3]);
+      const int m2 = m + 1, s2 = m2 >> 2, a2 = m2 & 3;
+      if (m2 < 16) {
+        fa[a2 & 1] = frag(s2, a2);
+        if (a2 == 0) fb[s2 & 1][0] = frag(s2, 7);
+      }
+    }
+  }
+};
 
 }  // namespace sce
