@@ -194,13 +194,13 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p_in
   const int col0 = ct * 256 + wa * 128;
   if (ragged) strike_columns_beyond<0, 1>(acc, vlim, wa);
   take_target_logits<false, true, false, 128, 0, 1>(acc, tgt, p.n_predict, col0, 0, 0.f, nullptr, 0, nullptr, 0.f, 0.f, 0.f);
-  uint32_t ew = form_dlogits<false, false, 32, 32, 0, 1>(acc, p.k1, p.c2, vlim, 0, gq, wa, wb, nullptr, lam, false, tail);
+  uint32_t ew = form_dlogits<false, 32, 32, 0, 1>(acc, p.k1, p.c2, 0, gq, wa, wb, nullptr, lam, false, tail);
   if (ragged) strike_columns_beyond<1, 2>(acc, vlim, wa);
   take_target_logits<false, true, false, 128, 1, 2>(acc, tgt, p.n_predict, col0, 0, 0.f, nullptr, 0, nullptr, 0.f, 0.f, 0.f);
-  ew |= form_dlogits<false, false, 32, 32, 1, 2>(acc, p.k1, p.c2, vlim, 0, gq, wa, wb, nullptr, lam, false, tail);
+  ew |= form_dlogits<false, 32, 32, 1, 2>(acc, p.k1, p.c2, 0, gq, wa, wb, nullptr, lam, false, tail);
   if (ragged) strike_columns_beyond<2, 4>(acc, vlim, wa);
   take_target_logits<false, true, false, 128, 2, 4>(acc, tgt, p.n_predict, col0, 0, 0.f, nullptr, 0, nullptr, 0.f, 0.f, 0.f);
-  ew |= form_dlogits<false, false, 32, 32, 2, 4>(acc, p.k1, p.c2, vlim, 0, gq, wa, wb, nullptr, lam, false);
+  ew |= form_dlogits<false, 32, 32, 2, 4>(acc, p.k1, p.c2, 0, gq, wa, wb, nullptr, lam, false);
   if (lane_id() == 0) p.gexp[(int64_t)(2 * ct + wa) * p.kbw + p.kb0 + 2 * rt + wb] = ew;
 }
 

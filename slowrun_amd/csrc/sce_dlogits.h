@@ -57,8 +57,9 @@ __device__ __forceinline__ float wave_max_dpp(float v) {
   return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
 }
 
-// The other way to deal with a tile that reaches beyond the vocabulary (columns >= vlim of the tile do not exist): their
-// accumulators are set to -inf before the epilogue, which then needs no EDGE variant -- such a logit reads as z = -cap, its
+// A tile that reaches beyond the vocabulary (columns >= vlim of the tile do not exist): their accumulators are set to
+// -inf before the epilogue, which then needs no masking variant (two copies of it, each with the MFMAs that ride along,
+// make the compiler spill accumulators) -- such a logit reads as z = -cap, its
 // stored value is exactly 0, it cannot be a block's maximum, and what it adds to the row sum, e^{-2 cap} a piece, is
 // taken out of `stat` here (a caller without row statistics passes none).  Row blocks [B0, B1).
 template <int B0, int B1>
@@ -87,13 +88,11 @@ __device__ __forceinline__ void strike_columns_beyond(v16f (&acc)[4][4], int vli
 // B0, B1: the row blocks [B0, B1) only (the returned dword has their bytes).
 // hook(b, k), k = 0..31: called between the stages of row block b's arithmetic (four to a batch of eight values): a place
 // for a caller's matrix instructions on other accumulators.
-template <bool EDGE, bool STATS, int LAM_STRIDE = NTHREADS, int LAM_LANES = 64, int B0 = 0, int B1 = 4, class Hook = NoHook>
-__device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float k1, float c2, int vlim, int vabs0,
+template <bool STATS, int LAM_STRIDE = NTHREADS, int LAM_LANES = 64, int B0 = 0, int B1 = 4, class Hook = NoHook>
+__device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float k1, float c2, int vabs0,
                                                  uint8_t* __restrict__ gq, int wa, int wb, float* stat, const float* lam, bool want_argmax = true,
                                                  Hook&& hook = NoHook()) {
   constexpr bool HOOKED = !std::is_same<typename std::decay<Hook>::type, NoHook>::value;
-  const int lane = lane_id();
-  const int vloc0 = wa * 128 + 4 * (lane >> 5);       // column (within the tile) of accumulator register 0 of block a = 0
   uint32_t expword = 0;
 #pragma unroll
   for (int b = B0; b < B1; ++b) {
@@ -105,9 +104,7 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
     for (int a = 0; a < 4; ++a)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        float x = acc[a][b][r];
-        if (EDGE && vloc0 + a * 32 + 8 * (r >> 2) + (r & 3) >= vlim) x = -INFINITY;
-        tmax = fmaxf(tmax, x);
+        tmax = fmaxf(tmax, acc[a][b][r]);
       }
     const float lamb = lam[b * LAM_STRIDE + (lane_id() & (LAM_LANES - 1))];      // (index taken anew: see lane_id)
     const float lg = wave_max_dpp(fmaf(c2, fast_rcp(1.0f + fast_exp2(tmax * k1)), lamb));      // over the block: log2 of the largest boosted e^{z - cap}
@@ -136,10 +133,6 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
         for (int m = g0; m < g0 + NB; ++m) gg[m] = fast_exp2(fmaf(c2, rr[m], cs));
         __builtin_amdgcn_sched_barrier(0);
         if (HOOKED) { hook(b, 4 * (2 * a + g0 / NB) + 2); __builtin_amdgcn_sched_barrier(0); }
-        if (EDGE) {
-#pragma unroll
-          for (int m = g0; m < g0 + NB; ++m) gg[m] = (vloc0 + a * 32 + 8 * (m >> 2) + (m & 3) >= vlim) ? 0.f : gg[m];
-        }
         if (STATS) {
 #pragma unroll
           for (int m = g0; m < g0 + NB; ++m) ssum += gg[m];
@@ -174,7 +167,7 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
 #pragma unroll
             for (int r = 15; r >= 0; --r) {
               const int vo = a * 32 + 8 * (r >> 2) + (r & 3);
-              if (acc[a][b][r] == tmax && (!EDGE || vloc0 + vo < vlim)) targ = vo;   // descending scan: lowest column wins
+              if (acc[a][b][r] == tmax) targ = vo;   // descending scan: lowest column wins
             }
           }
           if (tmax > amax || (targ != 0x7fffffff && vabs0 + targ < __float_as_int(stat[(8 + b) * NTHREADS]))) {

@@ -261,15 +261,15 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
       const bool ragged = vlim < 256;
       if (ragged) strike_columns_beyond<0, 1>(acc, vlim, wa, stat, p.em2cap);
       take_target_logits<true, true, true, 256, 0, 1>(acc, tgt, p.n_predict, col0, row0, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2, p.em2cap);
-      uint32_t ew = form_dlogits<false, true, NTHREADS, 64, 0, 1>(acc, p.k1, p.c2, vlim, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, tail);
+      uint32_t ew = form_dlogits<true, NTHREADS, 64, 0, 1>(acc, p.k1, p.c2, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, tail);
       if (ragged) strike_columns_beyond<1, 2>(acc, vlim, wa, stat, p.em2cap);
       take_target_logits<true, true, true, 256, 1, 2>(acc, tgt, p.n_predict, col0, row0, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2, p.em2cap);
-      ew |= form_dlogits<false, true, NTHREADS, 64, 1, 2>(acc, p.k1, p.c2, vlim, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, tail);
+      ew |= form_dlogits<true, NTHREADS, 64, 1, 2>(acc, p.k1, p.c2, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, tail);
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // every wave has read its last fragment
       prefetch();
       if (ragged) strike_columns_beyond<2, 4>(acc, vlim, wa, stat, p.em2cap);
       take_target_logits<true, true, true, 256, 2, 4>(acc, tgt, p.n_predict, col0, row0, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2, p.em2cap);
-      ew |= form_dlogits<false, true, NTHREADS, 64, 2, 4>(acc, p.k1, p.c2, vlim, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0);
+      ew |= form_dlogits<true, NTHREADS, 64, 2, 4>(acc, p.k1, p.c2, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0);
       if (lane_id() == 0) p.gexp[(int64_t)(2 * ct + wa) * p.kbw + 2 * rt + wb] = ew;
     } else {
       float sum[4], amax[4];
