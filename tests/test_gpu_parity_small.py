@@ -477,6 +477,22 @@ def test_ragged_and_tiny_shapes(N, d, V, keep):
     print(N, d, V, reduction, rep)
 
 
+@pytest.mark.parametrize("V", [1019, 900, 257])
+@pytest.mark.parametrize("keep", [False, True])
+def test_negative_logits_beside_columns_that_do_not_exist(V, keep):
+    """Every logit below zero, in a vocabulary that ends inside a tile (inside a group of 32 columns, inside the second
+    128-column half, one column into a tile): the columns a tile has beyond the vocabulary come out of the zero padding
+    of W as logit 0, above every real one -- they must win neither the argmax nor a block's exponent, and add nothing
+    to the row sums."""
+    inp = _small("irregular", 300, 64, V)
+    inp.x = inp.x.abs()
+    inp.w = -inp.w.abs()
+    ours = pu.run_ours(inp, "mean", keep_dlogits=keep)
+    ref = pu.run_oracle(inp, ours, "mean")
+    assert int(ours["argmax"].max()) < V
+    print(V, keep, pu.check_parity(ours, ref, "mean"))
+
+
 def test_fused_norm_with_multi_token_prediction_and_eval_head():
     """The fused norm composes with the other options: multi-token prediction in training, the vocabulary slice in
     evaluation.  Reference: the same calls on torch's own rms_norm output (bit-identical to the fused norm for bf16)."""
