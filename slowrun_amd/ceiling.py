@@ -8,7 +8,9 @@ shader clock.  This report puts numbers beside that peak, each from a short run 
   2. the library's main loop alone (global -> LDS -> MFMA, no epilogue) on the three GEMM shapes of the headline
      workload, on random and on all-zero operands;
   3. the vendor library's fp8 GEMM (torch._scaled_mm -> hipBLASLt) on the same shapes;
-  4. the shader clock and package power that rocm-smi reports while the main loop runs flat out.
+  4. the three big kernels of a step and their main loops alone on the step's own operands;
+  5. the socket power (sysfs) and the shader clock (rocm-smi) while the main loop runs flat out, on random and on
+     all-zero operands.
 
 Prints a plain-text report (and one JSON line at the end).  Nothing here is on the product path.
 """
@@ -78,32 +80,48 @@ def _hipblaslt(M, N, K, dev, reps=5):
     return 2.0 * M * N * K * reps / (e0.elapsed_time(e1) * 1e-3) * 1e-12, None
 
 
-def _smi_sample():
+def _hwmon():
+    """The GPU's power sensor in sysfs (socket power in microwatts, and its cap), if the box exposes one."""
+    import glob
+    for f in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")):
+        try:
+            open(f).read()
+            return f
+        except OSError:
+            continue
+    return None
+
+
+def _power_w(sensor):
     try:
-        out = subprocess.run(["rocm-smi", "--showclocks", "--showpower", "--json"], capture_output=True, text=True, timeout=10).stdout
+        return round(int(open(sensor).read()) * 1e-6)
+    except (OSError, ValueError, TypeError):
+        return None
+
+
+def _smi_sample(sensor=None):
+    try:
+        out = subprocess.run(["rocm-smi", "--showclocks", "--json"], capture_output=True, text=True, timeout=10).stdout
         card = next(iter(json.loads(out).values()))
     except Exception:                            # noqa: BLE001
         return None
     sclk = next((v for k, v in card.items() if "sclk" in k.lower()), None)
-    power = next((v for k, v in card.items() if "power" in k.lower() and "socket" in k.lower()), None) or \
-        next((v for k, v in card.items() if "power" in k.lower()), None)
-    return {"sclk": sclk, "power": power}
+    return {"sclk": sclk, "power_w": _power_w(sensor)}
 
 
-def _under_load(scratch, seconds=4.0):
-    """rocm-smi readings while the main loop runs on random operands."""
+def _under_load(scratch, kind, sensor, seconds=4.0):
+    """Socket power (sysfs) and rocm-smi's shader clock while the main loop runs on `kind` operands."""
     dev = scratch.device
-    a, b = _operand(8192, 8192, "random", dev), _operand(8192, 8192, "random", dev)
+    a, b = _operand(8192, 8192, kind, dev), _operand(8192, 8192, kind, dev)
     samples, stop = [], threading.Event()
 
     def poll():
         while not stop.is_set():
-            smp = _smi_sample()
+            smp = _smi_sample(sensor)
             if smp:
                 samples.append(smp)
             time.sleep(0.3)
 
-    idle = _smi_sample()
     th = threading.Thread(target=poll)
     th.start()
     tf, mhz = C.c_double(), C.c_double()
@@ -115,10 +133,10 @@ def _under_load(scratch, seconds=4.0):
         rates.append((tf.value, mhz.value))
     stop.set()
     th.join()
-    return idle, samples, rates
+    return samples, rates
 
 
-def _floor(workload, scratch, reps=5):
+def _floor(workload, scratch, reps=5, sensor=None):
     """One forward (dlogits kept) + backward of `workload`, timed per kernel kind by the library's events; then the main loops
     of the three big kernels alone (sce_bench_floor) on the buffers those calls left, and on all-zero buffers of the same
     sizes.  Returns {kind: {kernel_ms, floor_ms, floor_mhz, floor_zero_ms, floor_zero_mhz}}."""
@@ -185,6 +203,34 @@ def _floor(workload, scratch, reps=5):
     tot_k, tot_f = sum(out[k]["kernel_ms"] for k in kinds), sum(out[k]["floor_ms"] for k in kinds)
     print(f"   sum: kernels {tot_k:.3f} ms, main loops alone {tot_f:.3f} ms = {3 * flops / tot_f * 1e-9 / PEAK_FP8_TFLOPS * 100:.1f} % of peak "
           "for a step that did nothing else")
+    power = None
+    if sensor:                                   # last, so that the timings above are of a part as cool as bench.py finds it: socket power while steps run back to back
+        pw, stop = [], threading.Event()
+
+        def poll():
+            while not stop.is_set():
+                pw.append(_power_w(sensor))
+                time.sleep(0.05)
+
+        th = threading.Thread(target=poll)
+        th.start()
+        t0, nsteps = time.time(), 0
+        torch.cuda.synchronize()
+        while time.time() - t0 < 3.0:
+            for _ in range(10):
+                step()
+            torch.cuda.synchronize()
+            nsteps += 10
+        sustained_ms = (time.time() - t0) * 1e3 / nsteps
+        stop.set()
+        th.join()
+        pw = [v for v in pw[len(pw) // 4:] if v is not None]          # the first quarter is the ramp
+        if pw:
+            power = {"mean_w": round(sum(pw) / len(pw)), "max_w": max(pw), "min_w": min(pw), "steps": nsteps, "ms_per_step": round(sustained_ms, 3)}
+    if power:
+        out["step_power"] = power
+        print(f"   socket power while {power['steps']} such steps run back to back ({power['ms_per_step']} ms each by the host's clock): "
+              f"mean {power['mean_w']} W, {power['min_w']} - {power['max_w']} W")
     del saved, fws, bws
     return out
 
@@ -223,17 +269,27 @@ def main():
         rep["hipblaslt"][name.split()[0]] = None if tf is None else round(tf, 1)
         print(f"   {name:24s} " + (f"{tf:7.1f} TFLOP/s" if tf is not None else f"not available: {err}"))
     print("\n4. the three big kernels of a step and their main loops alone, on the step's own operand buffers (limited_2p7b: N = 65536, d = 2560, V = 50304)")
-    rep["floor"] = _floor("limited_2p7b", scratch)
+    sensor = None if args.no_smi else _hwmon()
+    rep["floor"] = _floor("limited_2p7b", scratch, sensor=sensor)
     if not args.no_smi:
-        print("\n5. rocm-smi while the main loop runs (8192^3, random operands)")
-        idle, samples, rates = _under_load(scratch)
-        rep["smi"] = {"idle": idle, "under_load": samples[:: max(1, len(samples) // 6)]}
-        rep["under_load"] = {"tflops": [round(r[0], 1) for r in rates][:: max(1, len(rates) // 6)],
-                             "shader_mhz": [round(r[1]) for r in rates][:: max(1, len(rates) // 6)]}
+        cap = None
+        if sensor:
+            try:
+                cap = round(int(open(sensor.replace("power1_input", "power1_cap")).read()) * 1e-6)
+            except (OSError, ValueError):
+                pass
+        print(f"\n5. socket power (sysfs hwmon, cap {cap} W) and rocm-smi's shader clock while the main loop runs (8192^3)")
+        idle = _smi_sample(sensor)
         print(f"   idle: {idle}")
-        for smp in rep["smi"]["under_load"]:
-            print(f"   load: {smp}")
-        print(f"   main loop meanwhile: {rep['under_load']['tflops']} TFLOP/s at {rep['under_load']['shader_mhz']} MHz (in-kernel)")
+        rep["smi"] = {"cap_w": cap, "idle": idle}
+        for kind in ("random", "zero"):
+            samples, rates = _under_load(scratch, kind, sensor)
+            pick = lambda v: v[:: max(1, len(v) // 6)]
+            rep["smi"][kind] = {"samples": pick(samples), "tflops": pick([round(r[0], 1) for r in rates]), "shader_mhz": pick([round(r[1]) for r in rates])}
+            print(f"   {kind} operands:")
+            for smp in rep["smi"][kind]["samples"]:
+                print(f"      {smp}")
+            print(f"      main loop meanwhile: {rep['smi'][kind]['tflops']} TFLOP/s at {rep['smi'][kind]['shader_mhz']} MHz (in-kernel)")
     print("\n" + json.dumps(rep))
 
 
