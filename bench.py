@@ -66,6 +66,53 @@ def cpu_baseline(inp, rows, threads):
     return rows / dt, dt
 
 
+class SocketPower:
+    """The GPU's socket power (the hwmon sensor in sysfs, microwatts) sampled from a thread while something runs; every
+    figure is None where the box has no such sensor."""
+
+    def __init__(self, period=0.02):
+        import glob
+        self.path = next((f for f in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")) if self._read(f)), None)
+        self.period, self.samples, self._stop, self._th = period, [], None, None
+
+    @staticmethod
+    def _read(path):
+        try:
+            return int(open(path).read()) * 1e-6
+        except (OSError, ValueError):
+            return None
+
+    def __enter__(self):
+        import threading
+        if self.path:
+            self._stop = threading.Event()
+
+            def poll():
+                while not self._stop.is_set():
+                    v = self._read(self.path)
+                    if v is not None:
+                        self.samples.append(v)
+                    time.sleep(self.period)
+
+            self._th = threading.Thread(target=poll)
+            self._th.start()
+        return self
+
+    def __exit__(self, *exc):
+        if self._th:
+            self._stop.set()
+            self._th.join()
+
+    def report(self):
+        if not self.path or not self.samples:
+            return None
+        body = self.samples[len(self.samples) // 4:]          # the first quarter is the ramp
+        cap = self._read(self.path.replace("power1_input", "power1_cap"))
+        return {"sensor": "hwmon power1_input (socket)", "cap_w": None if cap is None else round(cap), "mean_w": round(sum(body) / len(body)),
+                "max_w": round(max(body)), "samples": len(body),
+                "during": "the pass with the per-kernel timers that follows the timed region (same steps)"}
+
+
 def timed(step, steps, warmup=2):
     """ms per step over exactly `steps` steps, HIP events on torch's current stream (where the library launches)."""
     import torch
@@ -203,9 +250,10 @@ def main():
     ms_total = e0.elapsed_time(e1)
     # second pass of the same steps with the library's per-kernel HIP events switched on (roofline figures only)
     _lib.timing_enable(True)
-    for _ in range(args.steps):
-        out = step()
-    torch.cuda.synchronize()
+    with SocketPower() as power:
+        for _ in range(args.steps):
+            out = step()
+        torch.cuda.synchronize()
     kt = _lib.timing_read()
     _lib.timing_enable(False)
     ms_per_step = ms_total / args.steps
@@ -258,6 +306,7 @@ def main():
         "wall_s_timed_region": round(wall, 3),
         "roofline": roofline,
         "kernels": kernels,
+        "socket_power": power.report(),
         "other": other,
     }
     if not args.no_cpu_baseline:
