@@ -375,37 +375,102 @@ struct TailReader {
 // After that the LDS slots are free.  Every fragment is read two calls before its first use, into registers that the
 // MFMAs in between do not use: the A fragments alternate between fa[0] and fa[1], the B fragments of a sub-step between
 // fb[0] and fb[1].
+//
+// What a call does is a table, tail_op(b, k), that the device code follows and that tail_schedule_ok() replays at
+// compile time: every one of the 48 (sub-step, A block, row block) products is issued exactly once, in ascending
+// sub-step order for each accumulator block (the order the main loop itself would have used), from registers that
+// hold the right fragments, each read at least two calls earlier.
+struct TailRead { int kind, i, j, step, n; };       // register (kind 0: fa[i]; kind 1: fb[i][j]) <- fragment n of sub-step `step`
+struct TailOp {
+  bool mfma;                                         // acc[a][rb] += fa[fa_i] x fb[fb_i][fb_j] (sub-step `step`)
+  int step, a, rb, fa_i, fb_i, fb_j;
+  int nreads;
+  TailRead reads[3];
+};
+constexpr int TAIL_CALLS = 32;                       // calls per row block epilogue (8 batches of 4 stages)
+constexpr TailOp tail_prologue() {                   // before the first call
+  return TailOp{false, 0, 0, 0, 0, 0, 0, 3, {{0, 0, 0, 0, 0}, {1, 0, 0, 0, 5}, {1, 0, 1, 0, 6}}};
+}
+constexpr TailOp tail_op(int b, int k) {
+  TailOp op{false, 0, 0, 0, 0, 0, 0, 0, {{0, 0, 0, 0, 0}, {0, 0, 0, 0, 0}, {0, 0, 0, 0, 0}}};
+  if (b == 0) {
+    // MFMA k of 32: sub-step k / 8, A block (k % 8) / 2, row block 1 + k % 2
+    const int s = k >> 3, a = (k & 7) >> 1;
+    op.mfma = true; op.step = s; op.a = a; op.rb = 1 + (k & 1); op.fa_i = a & 1; op.fb_i = s & 1; op.fb_j = k & 1;
+    const int k2 = k + 2, s2 = k2 >> 3, a2 = (k2 & 7) >> 1;       // what MFMA k + 2 needs
+    if (k2 < 32) {
+      if ((k2 & 1) == 0) op.reads[op.nreads++] = TailRead{0, a2 & 1, 0, s2, a2};
+      if ((k2 & 7) == 0) {
+        op.reads[op.nreads++] = TailRead{1, s2 & 1, 0, s2, 5};
+        op.reads[op.nreads++] = TailRead{1, s2 & 1, 1, s2, 6};
+      }
+    } else if (k2 == 32) {                                        // the first of row block 3's
+      op.reads[op.nreads++] = TailRead{0, 0, 0, 0, 0};
+      op.reads[op.nreads++] = TailRead{1, 0, 0, 0, 7};
+    }
+  } else if (b == 1 && (k & 1)) {
+    // MFMA m = k / 2 of 16: sub-step m / 4, A block m % 4, row block 3
+    const int m = k >> 1, s = m >> 2, a = m & 3;
+    op.mfma = true; op.step = s; op.a = a; op.rb = 3; op.fa_i = a & 1; op.fb_i = s & 1; op.fb_j = 0;
+    const int m2 = m + 1, s2 = m2 >> 2, a2 = m2 & 3;
+    if (m2 < 16) {
+      op.reads[op.nreads++] = TailRead{0, a2 & 1, 0, s2, a2};
+      if (a2 == 0) op.reads[op.nreads++] = TailRead{1, s2 & 1, 0, s2, 7};
+    }
+  }
+  return op;
+}
+constexpr bool tail_schedule_ok() {
+  int fa_frag[2] = {-1, -1}, fa_when[2] = {0, 0};            // which fragment (8 * step + n) a register holds, and since which call
+  int fb_frag[2][2] = {{-1, -1}, {-1, -1}}, fb_when[2][2] = {{0, 0}, {0, 0}};
+  int done[4][4][4] = {};                                     // [step][a][rb]
+  int next_step[4][4] = {};                                   // [a][rb]: the sub-step this accumulator block expects next
+  int call = 0;
+  auto apply = [&](const TailOp& op) {
+    for (int q = 0; q < op.nreads; ++q) {
+      const TailRead& r = op.reads[q];
+      if (r.kind == 0) { fa_frag[r.i] = 8 * r.step + r.n; fa_when[r.i] = call; }
+      else { fb_frag[r.i][r.j] = 8 * r.step + r.n; fb_when[r.i][r.j] = call; }
+    }
+  };
+  apply(tail_prologue());
+  call = 2;                                                   // the prologue's reads have had the time before the first call
+  for (int b = 0; b < 2; ++b)
+    for (int k = 0; k < TAIL_CALLS; ++k, ++call) {
+      const TailOp op = tail_op(b, k);
+      if (op.mfma) {
+        if (fa_frag[op.fa_i] != 8 * op.step + op.a || fb_frag[op.fb_i][op.fb_j] != 8 * op.step + 4 + op.rb) return false;
+        if (call - fa_when[op.fa_i] < 2 || call - fb_when[op.fb_i][op.fb_j] < 2) return false;
+        if (next_step[op.a][op.rb] != op.step) return false;
+        ++next_step[op.a][op.rb];
+        ++done[op.step][op.a][op.rb];
+      }
+      apply(op);
+    }
+  for (int s = 0; s < 4; ++s)
+    for (int a = 0; a < 4; ++a)
+      for (int rb = 1; rb < 4; ++rb)
+        if (done[s][a][rb] != 1) return false;
+  return true;
+}
+static_assert(tail_schedule_ok(), "the deferred MFMAs: some product missing, doubled, out of order, or fed from the wrong registers");
+
 struct DeferredTail {
   TailReader frag;
   v8i fa[2], fb[2][2];
-  __device__ __forceinline__ DeferredTail(const uint8_t* smem, int wa, int wb) : frag(smem, wa, wb) {
-    fa[0] = frag(0, 0); fb[0][0] = frag(0, 5); fb[0][1] = frag(0, 6);
+  __device__ __forceinline__ void read(const TailOp& op) {
+#pragma unroll
+    for (int q = 0; q < 3; ++q)
+      if (q < op.nreads) {
+        const TailRead& r = op.reads[q];
+        if (r.kind == 0) fa[r.i] = frag(r.step, r.n); else fb[r.i][r.j] = frag(r.step, r.n);
+      }
   }
-  static __device__ __forceinline__ void mfma(const v8i& a, const v8i& b, v16f& c) {
-    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
-  }
+  __device__ __forceinline__ DeferredTail(const uint8_t* smem, int wa, int wb) : frag(smem, wa, wb) { read(tail_prologue()); }
   __device__ __forceinline__ void operator()(v16f (&acc)[4][4], int b, int k) {
-    if (b == 0) {
-      // MFMA k of 32: sub-step k / 8, A block (k % 8) / 2, row block 1 + k % 2
-      const int s = k >> 3, a = (k & 7) >> 1;
-      mfma(fa[a & 1], fb[s & 1][k & 1], acc[a][1 + (k & 1)]);
-      const int k2 = k + 2, s2 = k2 >> 3, a2 = (k2 & 7) >> 1;       // what MFMA k + 2 needs
-      if (k2 < 32) {
-        if ((k2 & 1) == 0) fa[a2 & 1] = frag(s2, a2);
-        if ((k2 & 7) == 0) { fb[s2 & 1][0] = frag(s2, 5); fb[s2 & 1][1] = frag(s2, 6); }
-      } else if (k2 == 32) {                                      // the first of row block 3's
-        fa[0] = frag(0, 0); fb[0][0] = frag(0, 7);
-      }
-    } else if (b == 1 && (k & 1)) {
-      // MFMA m = k / 2 of 16: sub-step m / 4, A block m % 4, row block 3
-      const int m = k >> 1, s = m >> 2, a = m & 3;
-      mfma(fa[a & 1], fb[s & 1][0], acc[a][3]);
-      const int m2 = m + 1, s2 = m2 >> 2, a2 = m2 & 3;
-      if (m2 < 16) {
-        fa[a2 & 1] = frag(s2, a2);
-        if (a2 == 0) fb[s2 & 1][0] = frag(s2, 7);
-      }
-    }
+    const TailOp op = tail_op(b, k);
+    if (op.mfma) acc[op.a][op.rb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[op.fa_i], fb[op.fb_i][op.fb_j], acc[op.a][op.rb], 0, 0, 0, 0, 0, 0);
+    read(op);
   }
 };
 
