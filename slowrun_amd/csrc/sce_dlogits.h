@@ -19,7 +19,8 @@ namespace sce {
 // D near 0.05 next to D near e^{-cap}), and 8 bits cannot hold both at one exponent.  So each row also has a boost of
 // its own, D_iv 2^{lam_i} is what is stored, with lam_i an integer estimated before the forward pass from a sample of
 // the row's logits (fwd_sample_kernel) and undone exactly in rho_i.  The block exponent is taken after the boost, so
-// a poor estimate costs precision, never range.
+// a poor estimate costs precision, never range: the row's own when it is too low, its block-mates' when it is too high
+// (hence the limit on it there).
 //
 // Layout: G, tile by tile ([tile of 256 rows i][block of 128 columns v][256 i][128 v] bytes): the B operand of dX as it
 // lies (rows i, K = v), and of dW (rows v, K = i) through the transposing LDS read.  Exponents: one dword per

@@ -145,7 +145,12 @@ __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int*
 
 // The exponent boost of every row, from one tile of its logits (256 columns from the middle of the vocabulary):
 // lam_i = floor(-log2 m_i), m_i the smallest of the means of e^{z - cap} over 16 groups of 16 columns -- the smallest,
-// so that a few peaks inside the sample (a target, say) do not pass for the level of the row.  One workgroup per row tile.
+// so that a few peaks inside the sample do not pass for the level of the row -- but no more than lifts the largest
+// sampled value (the row's own targets aside: they are not stored) to 2^BOOST_SPREAD.  The limit is for rows whose
+// logits saturate the cap: their e^{z - cap} is either 1 or e^{-2 cap}, a group without a positive column makes the
+// "level" 2^-40, and a boost of that size would let the row's saturated columns set the exponent of every block it
+// is in and push the 31 rows that share those blocks out of the 8 bits.  One workgroup per row tile.
+constexpr float BOOST_SPREAD = 10.f;
 __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct, float* __restrict__ lam_out) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   FwdParams p = p_in;
@@ -156,35 +161,46 @@ __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct,
   mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 0, 0, wave);
   const int lane = lane_id();
   const int vlim = p.V - ct * 256, vloc0 = wa * 128 + 4 * (lane >> 5);
-  float gmin[4];
+  float gmin[4], gmax[4];
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
-    gmin[b] = INFINITY;
+    gmin[b] = INFINITY; gmax[b] = 0.f;
+    // the row's targets, as columns of this tile (far outside it when there is none)
+    const int row = rt * 256 + wb * 128 + b * 32 + (lane & 31);
+    int ty[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      ty[k] = (k < p.n_predict && target_valid(p.targets, p.ignore_index, row + k, p.N, p.V) && row < p.N) ? (int)p.targets[row + k] - ct * 256 : -1;
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
       float sum = 0.f, cnt = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const float pt = fast_exp2(fast_rcp(fmaf(fast_exp2(acc[a][b][r] * p.k1), p.ic2, p.ic2)));
-        const bool live = vloc0 + a * 32 + 8 * (r >> 2) + (r & 3) < vlim;
+        const int vo = vloc0 + a * 32 + 8 * (r >> 2) + (r & 3);
+        const bool live = vo < vlim;
         sum += live ? pt : 0.f;
         cnt += live ? 1.f : 0.f;
+        const bool target = vo == ty[0] || vo == ty[1] || vo == ty[2] || vo == ty[3];
+        gmax[b] = (live && !target) ? fmaxf(gmax[b], pt) : gmax[b];
       }
       if (cnt > 0.f) gmin[b] = fminf(gmin[b], sum / cnt);
     }
     gmin[b] = fminf(gmin[b], __shfl_xor(gmin[b], 32));
+    gmax[b] = fmaxf(gmax[b], __shfl_xor(gmax[b], 32));
   }
   float* red = reinterpret_cast<float*>(smem);          // free: the main loop has ended in every wave
   if (wa == 1 && lane < 32) {
 #pragma unroll
-    for (int b = 0; b < 4; ++b) red[wb * 128 + b * 32 + lane] = gmin[b];
+    for (int b = 0; b < 4; ++b) { red[wb * 128 + b * 32 + lane] = gmin[b]; red[256 + wb * 128 + b * 32 + lane] = gmax[b]; }
   }
   __syncthreads();
   if (wa == 0 && lane < 32) {
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-      const float m = fminf(gmin[b], red[wb * 128 + b * 32 + lane]);
+      const float m = fminf(gmin[b], red[wb * 128 + b * 32 + lane]), top = fmaxf(gmax[b], red[256 + wb * 128 + b * 32 + lane]);
       float l = floorf(-log2f(m));
+      if (top > 0.f) l = fminf(l, floorf(-log2f(top)) + BOOST_SPREAD);      // (top == 0: the sample held nothing but the row's targets)
       l = l > 0.f ? (l < 120.f ? l : 120.f) : 0.f;           // also: NaN -> 0
       lam_out[rt * 256 + wb * 128 + b * 32 + lane] = l;
     }
