@@ -493,6 +493,19 @@ def test_negative_logits_beside_columns_that_do_not_exist(V, keep):
     print(V, keep, pu.check_parity(ours, ref, "mean"))
 
 
+@pytest.mark.parametrize("N,d,V,keep,reduction", [(3518, 560, 9364, True, "none"), (4216, 832, 131, True, "mean"), (5549, 576, 133, False, "mean"),
+                                                  (3183, 560, 290, True, "none"), (1267, 544, 8807, False, "none")])
+def test_saturating_rows_with_an_unlucky_sample(N, d, V, keep, reduction):
+    """Shapes (found by random search) in which one of the workload's few rows with 50-fold activations -- logits that
+    saturate the cap -- has a group of 16 sampled columns without a positive one: taken at its word, the sample makes
+    the row's level 2^-40, and with that boost the row sets the exponent of every block it is in; the 31 rows that
+    share those blocks then lose their mantissa bits (dX off by 3 to 14 % of the largest entry).  The boost is limited."""
+    inp = _small("irregular", N, d, V)
+    ours = pu.run_ours(inp, reduction, keep_dlogits=keep)
+    ref = pu.run_oracle(inp, ours, reduction)
+    print(N, d, V, keep, reduction, pu.check_parity(ours, ref, reduction))
+
+
 def test_fused_norm_with_multi_token_prediction_and_eval_head():
     """The fused norm composes with the other options: multi-token prediction in training, the vocabulary slice in
     evaluation.  Reference: the same calls on torch's own rms_norm output (bit-identical to the fused norm for bf16)."""
