@@ -156,7 +156,8 @@ def softcapped_ce_mtp(x, w, targets, mtp_weights, x_s=None, w_s=None, cap=15.0,
     shifted = []
     for k in range(K):
         t = torch.full((N,), IGNORE_INDEX, dtype=torch.int64, device=dev)
-        t[: N - k] = targets[k:]
+        if k < N:                      # (fewer rows than offsets: the later offsets have no row to point at)
+            t[: N - k] = targets[k:]
         shifted.append(t)
     wleaf = wq.detach().clone().requires_grad_(want_grads)
     losses = torch.empty(N, dtype=dtype, device=dev)

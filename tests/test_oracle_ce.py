@@ -223,6 +223,17 @@ def test_mtp_single_offset_is_plain_path():
     assert torch.equal(a["loss"], c["loss"]) and torch.equal(a["dx"], c["dx"]) and torch.equal(a["dw"], c["dw"])
 
 
+def test_mtp_with_fewer_rows_than_offsets():
+    """One or two rows and four offsets: the offsets beyond the last row take no part, so the result is that of the
+    offsets that have a row."""
+    x, w, y = _tiny(seed=13)
+    x, w = x.float(), w.float()
+    for n in (1, 2):
+        a = eager.softcapped_ce_mtp(x[:n], w, y[:n], [1.0, 0.5, 0.25, 0.125], cap=15.0)
+        b = eager.softcapped_ce_mtp(x[:n], w, y[:n], [1.0, 0.5][:n], cap=15.0)
+        assert torch.equal(a["loss"], b["loss"]) and torch.equal(a["dx"], b["dx"]) and torch.equal(a["dw"], b["dw"])
+
+
 def test_mtp_reference_kernel_formula_on_valid_targets():
     # tiny/cuda_kernels.py:226-240: loss_i = sum_k w_k (lse_i - z[i, y_{i+k}]) for i + k < N
     x, w, y = _tiny(seed=13, ignore=False)
