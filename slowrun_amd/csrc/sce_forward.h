@@ -169,8 +169,13 @@ __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct,
     const int row = rt * 256 + wb * 128 + b * 32 + (lane & 31);
     int ty[4];
 #pragma unroll
-    for (int k = 0; k < 4; ++k)
-      ty[k] = (k < p.n_predict && target_valid(p.targets, p.ignore_index, row + k, p.N, p.V) && row < p.N) ? (int)p.targets[row + k] - ct * 256 : -1;
+    for (int k = 0; k < 4; ++k) {
+      ty[k] = -1;
+      if (k < p.n_predict && row + k < p.N) {
+        const int64_t y = p.targets[row + k];
+        if (y != p.ignore_index && y >= 0 && y < p.V) ty[k] = (int)y - ct * 256;
+      }
+    }
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
       float sum = 0.f, cnt = 0.f;
