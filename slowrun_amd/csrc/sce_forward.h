@@ -151,30 +151,45 @@ __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int*
 // "level" 2^-40, and a boost of that size would let the row's saturated columns set the exponent of every block it
 // is in and push the 31 rows that share those blocks out of the 8 bits.  One workgroup per row tile.
 constexpr float BOOST_SPREAD = 10.f;
+constexpr int SMEM_SAMPLE = SMEM_BYTES + 4 * 256 * 4;      // the K slots and the targets of the tile's rows
 __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct, float* __restrict__ lam_out) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   FwdParams p = p_in;
   if (p.dc) { p.sc = p.dc->sc; p.k1 = p.dc->k1; }
   const int rt = blockIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wa = wave >> 1, wb = wave & 1;
+  // the targets of the tile's rows are fetched before the main loop, which hides the wait (four per thread), and laid out
+  // in LDS behind the K slots after it, as columns of this tile (-1: none), for the lanes that own the rows
+  int* tgt = reinterpret_cast<int*>(smem + SMEM_BYTES);          // [4 offsets][256 rows]
+  int64_t yraw[4];                                               // thread t fetches entries t, t + 256, ...: offset k of row t
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int row = rt * 256 + (int)threadIdx.x;
+    yraw[k] = (k < p.n_predict && row + k < p.N) ? p.targets[row + k] : p.ignore_index;
+  }
   v16f acc[4][4];
   mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 0, 0, wave);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int64_t y = yraw[k];
+    tgt[k * 256 + threadIdx.x] = (y != p.ignore_index && y >= 0 && y < p.V) ? (int)y - ct * 256 : -1;
+  }
+  __syncthreads();
   const int lane = lane_id();
   const int vlim = p.V - ct * 256, vloc0 = wa * 128 + 4 * (lane >> 5);
   float gmin[4], gmax[4];
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
     gmin[b] = INFINITY; gmax[b] = 0.f;
-    // the row's targets, as columns of this tile (far outside it when there is none)
-    const int row = rt * 256 + wb * 128 + b * 32 + (lane & 31);
     int ty[4];
 #pragma unroll
+    for (int k = 0; k < 4; ++k) ty[k] = tgt[k * 256 + wb * 128 + b * 32 + (lane_id() & 31)];
+    // which of the lane's 64 values of this row are targets: bit 16 a + r (the value's place as in take_target_logits)
+    unsigned long long excl = 0;
+#pragma unroll
     for (int k = 0; k < 4; ++k) {
-      ty[k] = -1;
-      if (k < p.n_predict && row + k < p.N) {
-        const int64_t y = p.targets[row + k];
-        if (y != p.ignore_index && y >= 0 && y < p.V) ty[k] = (int)y - ct * 256;
-      }
+      const int rel = ty[k] - wa * 128;
+      if ((unsigned)rel < 128u && ((rel >> 2) & 1) == (lane >> 5)) excl |= 1ull << ((rel >> 5) * 16 + ((rel >> 3) & 3) * 4 + (rel & 3));
     }
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
@@ -182,12 +197,10 @@ __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct,
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const float pt = fast_exp2(fast_rcp(fmaf(fast_exp2(acc[a][b][r] * p.k1), p.ic2, p.ic2)));
-        const int vo = vloc0 + a * 32 + 8 * (r >> 2) + (r & 3);
-        const bool live = vo < vlim;
+        const bool live = vloc0 + a * 32 + 8 * (r >> 2) + (r & 3) < vlim;
         sum += live ? pt : 0.f;
         cnt += live ? 1.f : 0.f;
-        const bool target = vo == ty[0] || vo == ty[1] || vo == ty[2] || vo == ty[3];
-        gmax[b] = (live && !target) ? fmaxf(gmax[b], pt) : gmax[b];
+        gmax[b] = (live && !((excl >> (16 * a + r)) & 1)) ? fmaxf(gmax[b], pt) : gmax[b];
       }
       if (cnt > 0.f) gmin[b] = fminf(gmin[b], sum / cnt);
     }

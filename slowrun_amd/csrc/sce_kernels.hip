@@ -140,7 +140,7 @@ static int check_device(int dev) {
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
-      HIP_TRY(hipFuncSetAttribute((const void*)fwd_sample_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES));
+      HIP_TRY(hipFuncSetAttribute((const void*)fwd_sample_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_SAMPLE));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_recompute_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_RECOMPUTE));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
@@ -510,7 +510,7 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
     KernelTimer tm(SCE_K_QUANT, st);
     float* lam = (float*)(sv + S.off_lam);
     p.lam = lam;
-    if (!bf16ops) fwd_sample_kernel<<<RT, NTHREADS, SMEM_BYTES, st>>>(p, CT / 2, lam);
+    if (!bf16ops) fwd_sample_kernel<<<RT, NTHREADS, SMEM_SAMPLE, st>>>(p, CT / 2, lam);
   }
   {
     KernelTimer tm(SCE_K_FWD, st);
