@@ -32,8 +32,15 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__
   // its state does not fit this call, and every gradient comes out NaN rather than silently wrong
   const CallMode fm = *reinterpret_cast<const CallMode*>(reinterpret_cast<const uint8_t*>(hdr) + HDR_MODE_OFF);
   const bool mismatch = fm.emit != mode.emit || fm.vocab_limit != mode.vocab_limit || fm.n_predict != mode.n_predict || fm.cap_bits != mode.cap_bits;
+  // The row's exponent boost.  A forward pass that emitted the dlogits had to estimate it from a sample of the row
+  // (fwd_sample_kernel).  When the dlogits are formed again here in backward, the row's sum S = e^{lse - cap} is known, and
+  // the boost is what makes the stored value the probability itself, D 2^lam = p (1 - t^2) 2^f with 0 <= f < 1: rows
+  // that share a block are then weighed by what their entries contribute, whatever the shapes of their distributions.
+  float lam_i = 0.f;
+  if (i < N) lam_i = rowinfo ? floorf((cap - s_lse[i]) * LOG2E) : lam[i];
+  if (!(lam_i >= -64.f && lam_i <= 120.f)) lam_i = 0.f;      // (ignored rows have no lse to speak of)
   if (rowinfo && i < Np) {          // what the recompute kernel wants to know of a row: its boost and its target columns
-    rowinfo[i] = __float_as_int(i < N ? lam[i] : 0.f);
+    rowinfo[i] = __float_as_int(lam_i);
     for (int k = 0; k < 4; ++k)
       rowinfo[(int64_t)(1 + k) * Np + i] = (k < n_predict && i < N && target_valid(targets, ignore_index, i + k, N, V)) ? (int)targets[i + k] : -1;
   }
@@ -59,7 +66,7 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__
         for (int k2 = 0; k2 < k; ++k2) first = first && !(ok[k2] && yk[k2] == yk[k]);
         h[k] = g * (1.0f - ty * ty) * (wk - (first ? sw * expf(zy - lse) : 0.f));
       }
-      r = ldexpf(g * sw * expf(cap - lse), -(int)lam[i]);      // the stored dlogits carry the row's boost 2^lam
+      r = ldexpf(g * sw * expf(cap - lse), -(int)lam_i);      // the stored dlogits carry the row's boost 2^lam
     }
   }
   if (mismatch && i < N) {

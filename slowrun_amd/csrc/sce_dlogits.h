@@ -17,8 +17,9 @@ namespace sce {
 // dX and dW GEMMs apply the exponents inside the matrix instruction (mfma_mainloop, SCALE).
 // Rows of very different temperature may share a block (a row whose logits saturate the cap next to ordinary ones:
 // D near 0.05 next to D near e^{-cap}), and 8 bits cannot hold both at one exponent.  So each row also has a boost of
-// its own, D_iv 2^{lam_i} is what is stored, with lam_i an integer estimated before the forward pass from a sample of
-// the row's logits (fwd_sample_kernel) and undone exactly in rho_i.  The block exponent is taken after the boost, so
+// its own, D_iv 2^{lam_i} is what is stored, with lam_i an integer -- estimated before a forward pass that emits the
+// dlogits from a sample of the row's logits (fwd_sample_kernel), taken from the row's sum when backward forms them
+// (bwd_prep_kernel) -- and undone exactly in rho_i.  The block exponent is taken after the boost, so
 // a poor estimate costs precision, never range: the row's own when it is too low, its block-mates' when it is too high
 // (hence the limit on it there).
 //
@@ -109,7 +110,7 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
       }
     const float lamb = lam[b * LAM_STRIDE + (lane_id() & (LAM_LANES - 1))];      // (index taken anew: see lane_id)
     const float lg = wave_max_dpp(fmaf(c2, fast_rcp(1.0f + fast_exp2(tmax * k1)), lamb));      // over the block: log2 of the largest boosted e^{z - cap}
-    const float sb = floorf(8.8f - lg);                       // between -120 and 8 + 2 cap log2(e) <= 124 (cap <= 40, boost <= 120)
+    const float sb = fminf(floorf(8.8f - lg), 126.f);         // from -112 (boost <= 120) to 8 + 2 cap log2(e) - boost, held to what the exponent byte has
     const float cs = sb + 2.0f + lamb;                        // the 4 of 4 r (1 - r) and the row's boost ride along
     expword |= (uint32_t)(127 - (int)sb) << (8 * b);
     float ssum = 0.f;

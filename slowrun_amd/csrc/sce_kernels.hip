@@ -506,11 +506,12 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
   p.want_argmax = a->argmax != nullptr;
   const int grid = 8 * nsplit * ((RT + 7) / 8);
   {
-    // the exponent boosts of the rows, from the tile in the middle of the vocabulary (kept for backward in either mode)
+    // the exponent boosts of the rows, estimated from the tile in the middle of the vocabulary: only for a forward pass
+    // that emits the dlogits (a backward pass that forms them again knows the rows' sums and takes the boosts from those)
     KernelTimer tm(SCE_K_QUANT, st);
     float* lam = (float*)(sv + S.off_lam);
     p.lam = lam;
-    if (!bf16ops) fwd_sample_kernel<<<RT, NTHREADS, SMEM_SAMPLE, st>>>(p, CT / 2, lam);
+    if (!bf16ops && emit) fwd_sample_kernel<<<RT, NTHREADS, SMEM_SAMPLE, st>>>(p, CT / 2, lam);
   }
   {
     KernelTimer tm(SCE_K_FWD, st);
