@@ -143,54 +143,52 @@ __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int*
   }
 }
 
-// The exponent boost of every row, from one tile of its logits (256 columns from the middle of the vocabulary):
-// lam_i = floor(-log2 m_i), m_i the smallest of the means of e^{z - cap} over 16 groups of 16 columns -- the smallest,
-// so that a few peaks inside the sample do not pass for the level of the row -- but no more than lifts the largest
-// sampled value (the row's own targets aside: they are not stored) to 2^BOOST_SPREAD.  The limit is for rows whose
-// logits saturate the cap: their e^{z - cap} is either 1 or e^{-2 cap}, a group without a positive column makes the
-// "level" 2^-40, and a boost of that size would let the row's saturated columns set the exponent of every block it
-// is in and push the 31 rows that share those blocks out of the 8 bits.  One workgroup per row tile.
-constexpr float BOOST_SPREAD = 10.f;
-constexpr int SMEM_SAMPLE = SMEM_BYTES + 4 * 256 * 4;      // the K slots and the targets of the tile's rows
+// The exponent boost of every row: lam_i = floor(-log2 S^_i), S^_i an estimate of the row's sum S_i = sum_v e^{z_iv - cap}
+// made before the forward kernel starts, so that the stored value D 2^lam is close to the row's probabilities
+// (times 1 - t^2) whatever the level of its logits.  Two tiles of logits go into it (one workgroup per row tile):
+//   * 256 columns from the middle of the vocabulary, for the level of the row's bulk: V times m_i, the smallest of the
+//     means of e^{z - cap} over 16 groups of 16 columns (the smallest, so that a few peaks inside the sample do not
+//     pass for the level of the row);
+//   * the 256 columns that are the targets of the tile's own rows (the rows of W^T gathered by the tile loader): the
+//     row's own target -- where a confident row that is right has most of its sum -- and the tokens around it in the
+//     text, where a language model's rows tend to have their other peaks.
+// Every single e^{z - cap} is a lower bound of the sum, so S^_i = max(V m_i, largest value seen in either tile).  What
+// the estimate cannot see is a peak in a column that is in neither tile: such a row is boosted too far by the share
+// of that peak in its sum (see form_dlogits for what that costs the rows that share its blocks).
+// A row that has no valid target at all takes no part in the backward pass (its weight is zero): it gets the lowest
+// boost, so that whatever its logits hold cannot set the exponent of a block.
+constexpr int SMEM_SAMPLE = SMEM_BYTES + 2 * 256 * 4;      // the K slots, the gathered rows, the rows without a target
 __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct, float* __restrict__ lam_out) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   FwdParams p = p_in;
   if (p.dc) { p.sc = p.dc->sc; p.k1 = p.dc->k1; }
   const int rt = blockIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wa = wave >> 1, wb = wave & 1;
-  // the targets of the tile's rows are fetched before the main loop, which hides the wait (four per thread), and laid out
-  // in LDS behind the K slots after it, as columns of this tile (-1: none), for the lanes that own the rows
-  int* tgt = reinterpret_cast<int*>(smem + SMEM_BYTES);          // [4 offsets][256 rows]
-  int64_t yraw[4];                                               // thread t fetches entries t, t + 256, ...: offset k of row t
+  // the targets of the thread's row are fetched before the first main loop, which hides the wait
+  int* rows = reinterpret_cast<int*>(smem + SMEM_BYTES);         // [256]: the row of W^T that column j of the second tile is
+  int* dead = rows + 256;                                        // [256]: row j has no valid target
+  int64_t yraw[4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
     const int row = rt * 256 + (int)threadIdx.x;
-    yraw[k] = (k < p.n_predict && row + k < p.N) ? p.targets[row + k] : p.ignore_index;
+    yraw[k] = (k < p.n_predict && row + k < p.N && row < p.N) ? p.targets[row + k] : p.ignore_index;
   }
   v16f acc[4][4];
   mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 0, 0, wave);
+  // (a row without a target stands in with column 0: any column of the vocabulary gives a valid lower bound)
+  {
+    bool any = false;
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const int64_t y = yraw[k];
-    tgt[k * 256 + threadIdx.x] = (y != p.ignore_index && y >= 0 && y < p.V) ? (int)y - ct * 256 : -1;
+    for (int k = 0; k < 4; ++k) any = any || (yraw[k] != p.ignore_index && yraw[k] >= 0 && yraw[k] < p.V);
+    rows[threadIdx.x] = (yraw[0] != p.ignore_index && yraw[0] >= 0 && yraw[0] < p.V) ? (int)yraw[0] : 0;
+    dead[threadIdx.x] = !any;
   }
-  __syncthreads();
   const int lane = lane_id();
   const int vlim = p.V - ct * 256, vloc0 = wa * 128 + 4 * (lane >> 5);
-  float gmin[4], gmax[4];
+  float gmin[4], top[4];                                         // top: the largest logit seen (in the accumulator's units)
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
-    gmin[b] = INFINITY; gmax[b] = 0.f;
-    int ty[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) ty[k] = tgt[k * 256 + wb * 128 + b * 32 + (lane_id() & 31)];
-    // which of the lane's 64 values of this row are targets: bit 16 a + r (the value's place as in take_target_logits)
-    unsigned long long excl = 0;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int rel = ty[k] - wa * 128;
-      if ((unsigned)rel < 128u && ((rel >> 2) & 1) == (lane >> 5)) excl |= 1ull << ((rel >> 5) * 16 + ((rel >> 3) & 3) * 4 + (rel & 3));
-    }
+    gmin[b] = INFINITY; top[b] = -INFINITY;
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
       float sum = 0.f, cnt = 0.f;
@@ -200,27 +198,41 @@ __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct,
         const bool live = vloc0 + a * 32 + 8 * (r >> 2) + (r & 3) < vlim;
         sum += live ? pt : 0.f;
         cnt += live ? 1.f : 0.f;
-        gmax[b] = (live && !((excl >> (16 * a + r)) & 1)) ? fmaxf(gmax[b], pt) : gmax[b];
+        top[b] = live ? fmaxf(top[b], acc[a][b][r]) : top[b];
       }
       if (cnt > 0.f) gmin[b] = fminf(gmin[b], sum / cnt);
     }
+  }
+  // the gathered tile, unless its offsets would not fit the loader's 32 bits
+  if ((int64_t)p.V * p.ldx < (int64_t)1 << 32) {
+    __syncthreads();
+    mfma_mainloop(p.wqt, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 0, 0, wave, NoHook(), 0, 0, nullptr, rows);
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) top[b] = fmaxf(top[b], acc[a][b][r]);
+  }
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
     gmin[b] = fminf(gmin[b], __shfl_xor(gmin[b], 32));
-    gmax[b] = fmaxf(gmax[b], __shfl_xor(gmax[b], 32));
+    top[b] = fmaxf(top[b], __shfl_xor(top[b], 32));
   }
   float* red = reinterpret_cast<float*>(smem);          // free: the main loop has ended in every wave
   if (wa == 1 && lane < 32) {
 #pragma unroll
-    for (int b = 0; b < 4; ++b) { red[wb * 128 + b * 32 + lane] = gmin[b]; red[256 + wb * 128 + b * 32 + lane] = gmax[b]; }
+    for (int b = 0; b < 4; ++b) { red[wb * 128 + b * 32 + lane] = gmin[b]; red[256 + wb * 128 + b * 32 + lane] = top[b]; }
   }
   __syncthreads();
   if (wa == 0 && lane < 32) {
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-      const float m = fminf(gmin[b], red[wb * 128 + b * 32 + lane]), top = fmaxf(gmax[b], red[256 + wb * 128 + b * 32 + lane]);
-      float l = floorf(-log2f(m));
-      if (top > 0.f) l = fminf(l, floorf(-log2f(top)) + BOOST_SPREAD);      // (top == 0: the sample held nothing but the row's targets)
-      l = l > 0.f ? (l < 120.f ? l : 120.f) : 0.f;           // also: NaN -> 0
-      lam_out[rt * 256 + wb * 128 + b * 32 + lane] = l;
+      const float m = fminf(gmin[b], red[wb * 128 + b * 32 + lane]), u = fmaxf(top[b], red[256 + wb * 128 + b * 32 + lane]);
+      const float peak = fast_exp2(fast_rcp(fmaf(fast_exp2(u * p.k1), p.ic2, p.ic2)));       // (u = -inf: e^{-2 cap})
+      float l = floorf(-log2f(fmaxf((float)p.V * m, peak)));
+      l = l > -64.f ? (l < 120.f ? l : 120.f) : -64.f;
+      lam_out[rt * 256 + wb * 128 + b * 32 + lane] = dead[wb * 128 + b * 32 + lane] ? -64.f : (l == l ? l : 0.f);
     }
   }
 }

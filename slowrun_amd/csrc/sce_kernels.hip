@@ -506,7 +506,7 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
   p.want_argmax = a->argmax != nullptr;
   const int grid = 8 * nsplit * ((RT + 7) / 8);
   {
-    // the exponent boosts of the rows, estimated from the tile in the middle of the vocabulary: only for a forward pass
+    // the exponent boosts of the rows, estimated from two tiles of their logits: only for a forward pass
     // that emits the dlogits (a backward pass that forms them again knows the rows' sums and takes the boosts from those)
     KernelTimer tm(SCE_K_QUANT, st);
     float* lam = (float*)(sv + S.off_lam);

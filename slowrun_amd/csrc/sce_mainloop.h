@@ -94,7 +94,9 @@ struct TileLoads {
   uint32_t vo[16];    // per-lane byte offset of load n; even n: A, odd n: B
   uint32_t lds[16];   // LDS address of load n in slot 0 (wave-uniform)
   // load n of an operand covers the 8-row chunk (n / 2 + rot) % 8 of the wave's 64 rows
-  __device__ __forceinline__ TileLoads(int64_t lda, int64_t ldb, uint8_t* smem, int rot_a, int rot_b, int wave) {
+  // a_rows (LDS, or null): row r of the A tile is row a_rows[r] of the array at Ag instead of row r -- a gather; the
+  // offsets stay 32-bit, so (largest index + 1) * lda must be below 2^32
+  __device__ __forceinline__ TileLoads(int64_t lda, int64_t ldb, uint8_t* smem, int rot_a, int rot_b, int wave, const int* a_rows = nullptr) {
     const int lane = lane_id();
     const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
     // one wave instruction covers 8 rows x 128 B; a wave fills rows [64 w, 64 w + 64) of A and of B
@@ -104,7 +106,7 @@ struct TileLoads {
       const int ca = (n + rot_a) & 7, cb = (n + rot_b) & 7;
       const int rowa = wave * 64 + ca * 8 + lr, rowb = wave * 64 + cb * 8 + lr;
       const int swa = (rowa & 7) ^ ((rowa >> 3) & 1), swb = (rowb & 7) ^ ((rowb >> 3) & 1);
-      vo[2 * n] = (uint32_t)(rowa * lda + ((pc ^ swa) * 16));
+      vo[2 * n] = (uint32_t)((a_rows ? a_rows[rowa] : rowa) * lda + ((pc ^ swa) * 16));
       if (TRB) vo[2 * n + 1] = (uint32_t)((rowb >> 7) * ldb + (rowb & 127) * BK + ((pc ^ (rowb & 7)) * 16));
       else vo[2 * n + 1] = (uint32_t)(rowb * ldb + ((pc ^ swb) * 16));
       lds[2 * n] = lds0 + wave * 64 * BK + ca * 8 * BK;
@@ -189,12 +191,13 @@ template <bool PREFETCHED = false, class Hook = NoHook, int KSTEP = BK, bool TRB
 __device__ __forceinline__ void mfma_mainloop(const uint8_t* __restrict__ Ag, int64_t lda,
                                               const uint8_t* __restrict__ Bg, int64_t ldb, int KD,
                                               uint8_t* smem, v16f (&acc)[4][4], int rot_a, int rot_b, int wave, Hook&& hook = NoHook(),
-                                              int64_t bk1_arg = 0, int64_t bk2_arg = 0, const uint32_t* lds_scale = nullptr) {
+                                              int64_t bk1_arg = 0, int64_t bk2_arg = 0, const uint32_t* lds_scale = nullptr,
+                                              const int* a_rows = nullptr) {
   static_assert(!DEFER || (!BF16 && SCALE == 0 && !TRB), "DEFER is for the plain fp8 loop");
   const int lane = lane_id();
   const int wa = wave >> 1, wb = wave & 1;
   const int64_t bk1 = TRB ? bk1_arg : (int64_t)KSTEP, bk2 = TRB ? bk2_arg : (int64_t)(2 * KSTEP);
-  const TileLoads<TRB> ld(lda, ldb, smem, rot_a, rot_b, wave);
+  const TileLoads<TRB> ld(lda, ldb, smem, rot_a, rot_b, wave, a_rows);
   // fragments: lane reads row l%32 of a 32-row block, 32 bytes of K at (l/32)*32 within the sub-step
   const int r = lane & 31, h = lane >> 5;
   const int sw = (r & 7) ^ ((r >> 3) & 1);

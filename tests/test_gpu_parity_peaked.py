@@ -144,3 +144,46 @@ def test_peaked_rows_at_the_headline_width(keep):
     print(rep)
     assert rep["mean_py"] > 0.2 and rep["sure_rows"] > 1000
     assert float(rr.median()) < 1e-2 and float(rr.max()) < 5e-2, rep
+
+
+def make_language_like(N, d, V, conf_max, seed=1, cap=15.0):
+    """Logits shaped like a language model's: a Zipfian unigram bias (log p ~ -log rank, the frequent tokens anywhere
+    in the vocabulary) that every row follows with its own strength conf_i ~ U(0, conf_max), carried by hidden unit
+    0, on top of random logits; the targets are drawn from the rows' own distributions (a calibrated model).  The
+    rows' peaks are then in the same few columns, at very different heights, and most of them are not the target."""
+    g = torch.Generator().manual_seed(seed)
+    bias = -torch.log(torch.arange(1, V + 1, dtype=torch.float32))[torch.randperm(V, generator=g)]
+    x = torch.randn(N, d, generator=g) * 0.3
+    w = torch.randn(d, V, generator=g) * d ** -0.5
+    x[:, 0] = torch.rand(N, generator=g) * conf_max
+    w[0, :] = bias
+    p = torch.softmax(cap * torch.tanh(x @ w / cap), dim=1)
+    y = torch.multinomial(p, 1, generator=g)[:, 0]
+    return configs.HeadInputs("language_like", x, w, y, float(x.abs().max()) / 448.0, float(w.abs().max()) / 448.0, cap)
+
+
+@pytest.mark.parametrize("keep", [False, True])
+@pytest.mark.parametrize("conf_max", [1.0, 3.0])
+def test_rows_of_mixed_confidence_with_peaks_in_the_same_columns(conf_max, keep):
+    """What the rows' exponent boost is for: rows whose sums differ by many powers of two share the blocks of the
+    frequent tokens' columns.  A boost that follows the level of a row's bulk instead of its sum puts the peaks of
+    the confident rows 2^17 above the unconfident rows' values in those blocks and costs the latter ten percent and
+    more of their dX; with the boost from the row's sum (the backward pass that forms the dlogits again) or from its
+    estimate (the forward pass that emits them: the row's own target and its neighbours' are among the sampled
+    columns) every row keeps its precision."""
+    N, d, V = 4096, 256, 8192
+    inp = make_language_like(N, d, V, conf_max)
+    go = torch.full((N,), 1.0 / N, device="cuda")
+    ours = pu.run_ours(inp, "none", x_dtype=torch.float32, w_dtype=torch.float32, grad_output=go, keep_dlogits=keep)
+    ref = pu.run_oracle(inp, ours, "none", grad_output=go)
+    # dW of a calibrated model cancels in expectation (the targets are drawn from p): what is left is of the size of
+    # the sampling noise, against which the rounding of S p to e4m3 shows -- the largest entry is held to one
+    # rounding step (2^-4), the direction to the stated cosine
+    rep = pu.check_parity(ours, ref, "none", grad_maxrel=0.0625)
+    rr = per_row_rel(ours["dx"], ref["dx"])
+    rep["dx_maxrel"], rep["row_rel_99"], rep["row_rel_max"] = pu.maxrel(ours["dx"].float(), ref["dx"]), float(rr.quantile(0.99)), float(rr.max())
+    rep["max_py"] = float(torch.exp(-ref["losses"]).max())
+    print(rep)
+    assert rep["dx_maxrel"] < 5e-3 and rep["row_rel_99"] < 4e-2 and rep["row_rel_max"] < 6e-2, rep
+    if conf_max >= 3.0:
+        assert rep["max_py"] > 0.8           # the case is what it claims to be
