@@ -34,10 +34,10 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__
   const bool mismatch = fm.emit != mode.emit || fm.vocab_limit != mode.vocab_limit || fm.n_predict != mode.n_predict || fm.cap_bits != mode.cap_bits;
   // The row's exponent boost.  A forward pass that emitted the dlogits had to estimate the row's sum from a sample of
   // the row (fwd_sample_kernel).  When the dlogits are formed again here in backward, the sum S = e^{lse - cap} is known, and
-  // the boost is what makes the stored value the probability itself, D 2^lam = p (1 - t^2) 2^f with 0 <= f < 1: rows
+  // the boost is what makes the stored value the probability itself, D 2^lam = p (1 - t^2): rows
   // that share a block are then weighed by what their entries contribute, whatever the shapes of their distributions.
   float lam_i = 0.f;
-  if (i < N) lam_i = rowinfo ? floorf((cap - s_lse[i]) * LOG2E) : lam[i];
+  if (i < N) lam_i = rowinfo ? (cap - s_lse[i]) * LOG2E : lam[i];
   if (!(lam_i >= -64.f && lam_i <= 120.f)) lam_i = 0.f;      // (ignored rows have no lse to speak of)
   if (rowinfo && i < Np) {          // what the recompute kernel wants to know of a row: its boost and its target columns
     rowinfo[i] = __float_as_int(lam_i);
@@ -66,7 +66,10 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__
         for (int k2 = 0; k2 < k; ++k2) first = first && !(ok[k2] && yk[k2] == yk[k]);
         h[k] = g * (1.0f - ty * ty) * (wk - (first ? sw * expf(zy - lse) : 0.f));
       }
-      r = ldexpf(g * sw * expf(cap - lse), -(int)lam_i);      // the stored dlogits carry the row's boost 2^lam
+      // the stored dlogits carry the row's boost 2^lam: an integer from the forward pass that emitted them, the real
+      // (cap - lse) log2(e) here -- then rho_i 2^-lam_i is g_i times the row's weights and nothing else, the same number for
+      // nearly every row of a mean-reduced loss, and the scaled X that dW multiplies with is X_q itself: no second rounding
+      r = rowinfo ? g * sw * expf(cap - lse - lam_i * 0.6931471805599453f) : ldexpf(g * sw * expf(cap - lse), -(int)lam_i);
     }
   }
   if (mismatch && i < N) {

@@ -17,13 +17,13 @@ namespace sce {
 // dX and dW GEMMs apply the exponents inside the matrix instruction (mfma_mainloop, SCALE).
 // Rows of very different temperature may share a block (a row whose logits saturate the cap next to ordinary ones:
 // D near 0.05 next to D near e^{-cap}), and 8 bits cannot hold both at one exponent.  So each row also has a boost of
-// its own, D_iv 2^{lam_i} is what is stored, with the integer lam_i = floor(-log2 S_i), S_i = sum_v e^{z_iv - cap} the
-// row's sum -- known when backward forms the dlogits (bwd_prep_kernel), estimated from two tiles of the row's logits
-// before a forward pass that emits them (fwd_sample_kernel) -- and undone exactly in rho_i.  What is stored is then
-// the row's probabilities, p_iv (1 - t^2) 2^f with 0 <= f < 1, and rows that share a block are weighed by what their
-// entries contribute.  The block exponent is taken after the boost, so a poor estimate costs precision, never range:
-// an estimate of the sum that is too low boosts the row too far, and the 31 rows that share its blocks lose bits
-// where its peaks are.
+// its own, D_iv 2^{lam_i} is what is stored, with lam_i = -log2 S_i, S_i = sum_v e^{z_iv - cap} the row's sum -- known
+// when backward forms the dlogits (bwd_prep_kernel), estimated from two tiles of the row's logits and rounded down to an
+// integer before a forward pass that emits them (fwd_sample_kernel) -- and undone in rho_i.  What is stored is then
+// the row's probabilities, p_iv (1 - t^2) (times 2^f, 0 <= f < 1, for the integer), and rows that share a block are
+// weighed by what their entries contribute.  The block exponent is taken after the boost, so a poor estimate costs
+// precision, never range: an estimate of the sum that is too low boosts the row too far, and the 31 rows that share
+// its blocks lose bits where its peaks are.
 //
 // Layout: G, tile by tile ([tile of 256 rows i][block of 128 columns v][256 i][128 v] bytes): the B operand of dX as it
 // lies (rows i, K = v), and of dW (rows v, K = i) through the transposing LDS read.  Exponents: one dword per
