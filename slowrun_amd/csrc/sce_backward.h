@@ -33,7 +33,7 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__
   const CallMode fm = *reinterpret_cast<const CallMode*>(reinterpret_cast<const uint8_t*>(hdr) + HDR_MODE_OFF);
   const bool mismatch = fm.emit != mode.emit || fm.vocab_limit != mode.vocab_limit || fm.n_predict != mode.n_predict || fm.cap_bits != mode.cap_bits;
   // The row's exponent boost.  A forward pass that emitted the dlogits had to estimate the row's sum from a sample of
-  // the row (fwd_sample_kernel).  When the dlogits are formed again here in backward, the sum S = e^{lse - cap} is known, and
+  // the row (fwd_sample_kernel).  When the dlogits are formed again here in backward, the sum Z = e^{lse - cap} is known, and
   // the boost is what makes the stored value the probability itself, D 2^lam = p (1 - t^2): rows
   // that share a block are then weighed by what their entries contribute, whatever the shapes of their distributions.
   float lam_i = 0.f;

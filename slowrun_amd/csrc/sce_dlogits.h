@@ -17,7 +17,7 @@ namespace sce {
 // dX and dW GEMMs apply the exponents inside the matrix instruction (mfma_mainloop, SCALE).
 // Rows of very different temperature may share a block (a row whose logits saturate the cap next to ordinary ones:
 // D near 0.05 next to D near e^{-cap}), and 8 bits cannot hold both at one exponent.  So each row also has a boost of
-// its own, D_iv 2^{lam_i} is what is stored, with lam_i = -log2 S_i, S_i = sum_v e^{z_iv - cap} the row's sum -- known
+// its own, D_iv 2^{lam_i} is what is stored, with lam_i = -log2 Z_i, Z_i = sum_v e^{z_iv - cap} the row's softmax sum -- known
 // when backward forms the dlogits (bwd_prep_kernel), estimated from two tiles of the row's logits and rounded down to an
 // integer before a forward pass that emits them (fwd_sample_kernel) -- and undone in rho_i.  What is stored is then
 // the row's probabilities, p_iv (1 - t^2) (times 2^f, 0 <= f < 1, for the integer), and rows that share a block are

@@ -143,7 +143,7 @@ __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int*
   }
 }
 
-// The exponent boost of every row: lam_i = floor(-log2 S^_i), S^_i an estimate of the row's sum S_i = sum_v e^{z_iv - cap}
+// The exponent boost of every row: lam_i = floor(-log2 Z^_i), Z^_i an estimate of the row's softmax sum Z_i = sum_v e^{z_iv - cap}
 // made before the forward kernel starts, so that the stored value D 2^lam is close to the row's probabilities
 // (times 1 - t^2) whatever the level of its logits.  Two tiles of logits go into it (one workgroup per row tile):
 //   * 256 columns from the middle of the vocabulary, for the level of the row's bulk: V times m_i, the smallest of the
@@ -152,7 +152,7 @@ __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int*
 //   * the 256 columns that are the targets of the tile's own rows (the rows of W^T gathered by the tile loader): the
 //     row's own target -- where a confident row that is right has most of its sum -- and the tokens around it in the
 //     text, where a language model's rows tend to have their other peaks.
-// Every single e^{z - cap} is a lower bound of the sum, so S^_i = max(V m_i, largest value seen in either tile).  What
+// Every single e^{z - cap} is a lower bound of the sum, so Z^_i = max(V m_i, largest value seen in either tile).  What
 // the estimate cannot see is a peak in a column that is in neither tile: such a row is boosted too far by the share
 // of that peak in its sum (see form_dlogits for what that costs the rows that share its blocks).
 // A row that has no valid target at all takes no part in the backward pass (its weight is zero): it gets the lowest
