@@ -243,6 +243,15 @@ int sce_bench_gemm(const void* A, const void* B, int64_t M, int64_t N, int64_t K
 int sce_bench_floor(const sce_args* args, int32_t which, int32_t reps, void* scratch, size_t scratch_bytes, double* ms_per_pass,
                     double* shader_mhz);
 
+/* ---- test aid (no counterpart in the reference) --------------------------------------------
+ * A forward pass with dlogits_from_forward computes its target logits ahead of the forward kernel, from a tile of gathered
+ * rows of the quantised W, while W_q^T is smaller than 4 GiB (the reach of that tile's 32-bit offsets), and inside the
+ * forward kernel, out of its accumulators, beyond.  This sets the size in bytes from which the second way is taken
+ * (0 or less: back to 4 GiB), so that a test can run it at a size it can afford.  Process-wide; returns the previous
+ * value.  The results of the two ways are the same bit for bit in the losses and within the tolerances in the
+ * gradients (the target entries of a block take part in nothing either way). */
+int64_t sce_test_set_gather_limit(int64_t bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -15,7 +15,8 @@ SCE_VERSION = 4
 
 EXPORTS = ("sce_version", "sce_last_error", "sce_sizes_for", "sce_quantize_e4m3", "sce_quantize_e4m3_dev", "sce_amax_scale",
            "sce_transpose_bytes",
-           "sce_forward", "sce_forward_noalloc", "sce_backward", "sce_timing_enable", "sce_timing_read", "sce_bench_mfma", "sce_bench_gemm", "sce_bench_floor")
+           "sce_forward", "sce_forward_noalloc", "sce_backward", "sce_timing_enable", "sce_timing_read", "sce_bench_mfma", "sce_bench_gemm", "sce_bench_floor",
+           "sce_test_set_gather_limit")
 
 KERNEL_KINDS = ("quantize", "fwd", "fwd_reduce", "bwd_prep", "recompute", "dx", "dw", "dw_final")
 
@@ -82,6 +83,8 @@ def lib():
         L.sce_bench_gemm.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_size_t,
                                      C.c_int32, C.c_void_p, C.POINTER(C.c_double), C.POINTER(C.c_double)]
         L.sce_bench_floor.argtypes = [C.POINTER(SceArgs), C.c_int32, C.c_int32, C.c_void_p, C.c_size_t, C.POINTER(C.c_double), C.POINTER(C.c_double)]
+        L.sce_test_set_gather_limit.restype = C.c_int64
+        L.sce_test_set_gather_limit.argtypes = [C.c_int64]
         L.sce_timing_enable.argtypes = [C.c_int]
         L.sce_timing_read.argtypes = [C.POINTER(SceTiming)]
         if L.sce_version() != SCE_VERSION:

@@ -92,10 +92,13 @@ __device__ __forceinline__ void strike_columns_beyond(v16f (&acc)[4][4], int vli
 // B0, B1: the row blocks [B0, B1) only (the returned dword has their bytes).
 // hook(b, k), k = 0..31: called between the stages of row block b's arithmetic (four to a batch of eight values): a place
 // for a caller's matrix instructions on other accumulators.
-template <bool STATS, int LAM_STRIDE = NTHREADS, int LAM_LANES = 64, int B0 = 0, int B1 = 4, class Hook = NoHook>
+// EXCL: the lane's values of row block b hold a target logit that is still in the accumulators (it has not been knocked
+// out; its byte of G is cleared afterwards), known by its value: the accumulator times `sc` equals xc[b] (NaN: none).  It
+// takes no part in the block's exponent -- the lane offers its second largest value when the largest is that one.
+template <bool STATS, int LAM_STRIDE = NTHREADS, int LAM_LANES = 64, int B0 = 0, int B1 = 4, class Hook = NoHook, bool EXCL = false>
 __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float k1, float c2, int vabs0,
                                                  uint8_t* __restrict__ gq, int wa, int wb, float* stat, const float* lam, bool want_argmax = true,
-                                                 Hook&& hook = NoHook()) {
+                                                 Hook&& hook = NoHook(), const float* xc = nullptr, float sc = 0.f) {
   constexpr bool HOOKED = !std::is_same<typename std::decay<Hook>::type, NoHook>::value;
   uint32_t expword = 0;
 #pragma unroll
@@ -110,8 +113,22 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
       for (int r = 0; r < 16; ++r) {
         tmax = fmaxf(tmax, acc[a][b][r]);
       }
+    float texp = tmax;
+    if (EXCL) {
+      // some lane's largest value is its row's target (seldom, unless the rows are sure of their targets): that lane
+      // offers the largest of the others
+      const bool is_target = tmax * sc == xc[b];
+      if (__builtin_amdgcn_ballot_w64(is_target) != 0) {
+        float tsec = -INFINITY;
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) tsec = fmaxf(tsec, acc[a][b][r] == tmax ? -INFINITY : acc[a][b][r]);
+        texp = is_target ? tsec : tmax;
+      }
+    }
     const float lamb = lam[b * LAM_STRIDE + (lane_id() & (LAM_LANES - 1))];      // (index taken anew: see lane_id)
-    const float lg = wave_max_dpp(fmaf(c2, fast_rcp(1.0f + fast_exp2(tmax * k1)), lamb));      // over the block: log2 of the largest boosted e^{z - cap}
+    const float lg = wave_max_dpp(fmaf(c2, fast_rcp(1.0f + fast_exp2(texp * k1)), lamb));      // over the block: log2 of the largest boosted e^{z - cap}
     const float sb = fminf(floorf(8.8f - lg), 126.f);         // from -112 (boost <= 120) to 8 + 2 cap log2(e) - boost, held to what the exponent byte has
     const float cs = sb + 2.0f + lamb;                        // the 4 of 4 r (1 - r) and the row's boost ride along
     expword |= (uint32_t)(127 - (int)sb) << (8 * b);

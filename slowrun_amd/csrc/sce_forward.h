@@ -157,16 +157,32 @@ __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int*
 // of that peak in its sum (see form_dlogits for what that costs the rows that share its blocks).
 // A row that has no valid target at all takes no part in the backward pass (its weight is zero): it gets the lowest
 // boost, so that whatever its logits hold cannot set the exponent of a block.
-constexpr int SMEM_SAMPLE = SMEM_BYTES + 2 * 256 * 4;      // the K slots, the gathered rows, the rows without a target
+//
+// GATHER = false: the first tile only (the gathered rows' offsets would not fit the loader's 32 bits: W_q^T of 4 GiB or more).
+// GATHER = true also leaves the target logits of the tile's rows in s_uy, for the forward kernel that follows: u[i, y_{i+k}]
+// is element (i, i + k) of the gathered tile, computed by the same instructions in the same order as the forward
+// kernel will compute it (bit for bit: that kernel recognises the entry by its value).  The offsets k >= 1 of the
+// tile's last rows point at targets of the next tile's rows: those (at most three) ride as the last columns of the
+// first tile, in place of the sampled columns there.
+constexpr int SMEM_SAMPLE = SMEM_BYTES + 2 * 256 * 4 + 8 * 256 * 4;      // the K slots, the gathered rows, the rows without a target, the first tile's results
+template <bool GATHER>
 __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct, float* __restrict__ lam_out) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   FwdParams p = p_in;
   if (p.dc) { p.sc = p.dc->sc; p.k1 = p.dc->k1; }
   const int rt = blockIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wa = wave >> 1, wb = wave & 1;
-  // the targets of the thread's row are fetched before the first main loop, which hides the wait
-  int* rows = reinterpret_cast<int*>(smem + SMEM_BYTES);         // [256]: the row of W^T that column j of the second tile is
+  int* rows = reinterpret_cast<int*>(smem + SMEM_BYTES);         // [256]: the row of W^T that column j of a tile is
   int* dead = rows + 256;                                        // [256]: row j has no valid target
+  const int ntail = GATHER ? p.n_predict - 1 : 0;                // columns 256 - ntail .. 255 of the first tile: the next rows' targets
+  auto column_of = [&](int64_t y) { return (y != p.ignore_index && y >= 0 && y < p.V) ? (int)y : 0; };
+  if (GATHER) {
+    // (a row without a target stands in with column 0: any column of the vocabulary gives a valid lower bound of the sum)
+    const int t = threadIdx.x, j = t - (256 - ntail), row = rt * 256 + 256 + j;
+    rows[t] = j < 0 ? ct * 256 + t : column_of(row < p.N ? p.targets[row] : p.ignore_index);
+    __syncthreads();
+  }
+  // the targets of the thread's row are fetched before the first main loop, which hides the wait
   int64_t yraw[4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
@@ -174,17 +190,28 @@ __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct,
     yraw[k] = (k < p.n_predict && row + k < p.N && row < p.N) ? p.targets[row + k] : p.ignore_index;
   }
   v16f acc[4][4];
-  mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 0, 0, wave);
-  // (a row without a target stands in with column 0: any column of the vocabulary gives a valid lower bound)
+  if (GATHER) mfma_mainloop(p.wqt, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 0, 0, wave, NoHook(), 0, 0, nullptr, rows);
+  else mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 0, 0, wave);
   {
     bool any = false;
 #pragma unroll
     for (int k = 0; k < 4; ++k) any = any || (yraw[k] != p.ignore_index && yraw[k] >= 0 && yraw[k] < p.V);
-    rows[threadIdx.x] = (yraw[0] != p.ignore_index && yraw[0] >= 0 && yraw[0] < p.V) ? (int)yraw[0] : 0;
+    rows[threadIdx.x] = column_of(yraw[0]);
     dead[threadIdx.x] = !any;
   }
   const int lane = lane_id();
-  const int vlim = p.V - ct * 256, vloc0 = wa * 128 + 4 * (lane >> 5);
+  if (GATHER) {
+    // columns 252 .. 255 are registers 12 .. 15 of A block 3 in the upper half-wave of the waves with wa = 1; rows 224 .. 255
+    // are B block 3 of the waves with wb = 1
+    const int i = 224 + (lane & 31);
+    const bool mine = wave == 3 && lane >= 32;
+#pragma unroll
+    for (int r = 12; r < 16; ++r) {
+      const int k = 256 + (252 + (r & 3) - (256 - ntail)) - i;       // the offset of row i that this column serves
+      if (mine && 252 + (r & 3) >= 256 - ntail && k >= 1 && k < p.n_predict) p.s_uy[(int64_t)k * p.Np + rt * 256 + i] = acc[3][3][r] * p.sc;
+    }
+  }
+  const int vlim = min(p.V - ct * 256, 256 - ntail), vloc0 = wa * 128 + 4 * (lane >> 5);
   float gmin[4], top[4];                                         // top: the largest logit seen (in the accumulator's units)
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
@@ -203,16 +230,40 @@ __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct,
       if (cnt > 0.f) gmin[b] = fminf(gmin[b], sum / cnt);
     }
   }
-  // the gathered tile, unless its offsets would not fit the loader's 32 bits
-  if ((int64_t)p.V * p.ldx < (int64_t)1 << 32) {
+  if (GATHER && p.n_predict > 0) {      // (a condition the compiler cannot decide: merged into one block, the code of the two main loops is spilled)
+    // the first tile's results wait in LDS: there is no register for them in the main loop
+    float* keep = reinterpret_cast<float*>(smem + SMEM_BYTES + 2048) + threadIdx.x;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) { keep[b * 256] = gmin[b]; keep[(4 + b) * 256] = top[b]; }
     __syncthreads();
     mfma_mainloop(p.wqt, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 0, 0, wave, NoHook(), 0, 0, nullptr, rows);
+    keep = reinterpret_cast<float*>(smem + SMEM_BYTES + 2048) + wave * 64 + lane_id();
+#pragma unroll
+    for (int b = 0; b < 4; ++b) { gmin[b] = keep[b * 256]; top[b] = keep[(4 + b) * 256]; }
 #pragma unroll
     for (int b = 0; b < 4; ++b)
 #pragma unroll
       for (int a = 0; a < 4; ++a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) top[b] = fmaxf(top[b], acc[a][b][r]);
+    // The band 0 <= column - row < n_predict lies in the 32 x 32 blocks on the diagonal and right of it: blocks (a, b) with
+    // a - b = 0 or 1 of the waves with wa = wb, block (0, 3) of the wave with wa = 1, wb = 0.  (Stores under a lane
+    // condition, no branches around the accumulators.)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int a = b; a < 5; ++a) {
+        if (a > b + 1 && !(a == 4 && b == 3)) continue;
+        const int aa = a & 3;                                    // (a = 4: A block 0 of the waves one to the right)
+        const bool mine = a < 4 ? wa == wb : (wa == 1 && wb == 0);
+        const int i = wb * 128 + b * 32 + (lane_id() & 31);      // (the lane index taken anew: what is prepared before the main loop is spilled across it)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int k = wa * 128 + aa * 32 + 8 * (r >> 2) + 4 * (lane_id() >> 5) + (r & 3) - i;
+          if (mine && k >= 0 && k < p.n_predict) p.s_uy[(int64_t)k * p.Np + rt * 256 + i] = acc[aa][b][r] * p.sc;
+        }
+        __builtin_amdgcn_sched_barrier(0);      // (one block's accumulators at a time: all of them moved up front do not fit the registers)
+      }
   }
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
@@ -237,19 +288,37 @@ __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct,
   }
 }
 
+// The target entries of the dlogits that a forward pass has emitted are set to zero: they take no part in D (their
+// share goes into the one-hot coefficient in fp32, see bwd_prep_kernel).  One thread per row.
+__global__ __launch_bounds__(256) void fwd_knock_kernel(uint8_t* __restrict__ ghat, int64_t kbv, const int64_t* __restrict__ targets,
+                                                       int64_t ignore_index, int N, int V, int n_predict) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= N) return;
+  for (int k = 0; k < n_predict; ++k) {
+    if (!target_valid(targets, ignore_index, i + k, N, V)) continue;
+    const int64_t y = targets[i + k];
+    ghat[((int64_t)(i >> 8) * kbv + (y >> 7)) * BLOCKED_KSTEP + (i & 255) * BK + (y & 127)] = 0;
+  }
+}
+
 // LDS of the forward kernel: the two K slots; the row statistics of the workgroup's walk (12 values per lane, and the boosts of
 // its rows: kept in registers they are spilled around the main loop, and the reload -- a vector memory load -- makes the
 // epilogue wait for the tile loads that were just put in flight for the next tile); the targets of the workgroup's 256 rows.
 constexpr int FWD_STAT_OFF = SMEM_MAX - 4096 - 16 * 4 * NTHREADS;      // 12 statistics and the boosts of the lane's 4 rows
 constexpr int FWD_TGT_OFF = SMEM_MAX - 4096;
+constexpr int FWD_UY_OFF = FWD_STAT_OFF - 4096;                        // PRE: the target logits of the rows, laid out like the targets
 constexpr int SMEM_FWD = SMEM_MAX;
-static_assert(SMEM_BYTES <= FWD_STAT_OFF, "K slots and row statistics overlap");
+static_assert(SMEM_BYTES <= FWD_UY_OFF, "K slots and row data overlap");
 
 // EMIT: the epilogue also leaves the block-scaled dlogits of the tile in G (see form_dlogits), for a backward pass
 // that does not compute the logits again.
 // BF16 (without EMIT): bf16 operands, logits rounded to bf16 as the eager head's GEMM returns them (forward only).
-template <bool EMIT, bool BF16 = false>
+// PRE (with EMIT): the target logits are in s_uy already (fwd_sample_kernel<true>) and this kernel does not look for them in
+// its accumulators; the target entries go through the epilogue like any other, except that they are kept out of the block
+// exponents (form_dlogits, EXCL), and fwd_knock_kernel clears their bytes of G afterwards.
+template <bool EMIT, bool BF16 = false, bool PRE = false>
 __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
+  static_assert(!PRE || EMIT, "PRE belongs to the emitting kernel");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   FwdParams p = p_in;
   if (p.dc) { p.sc = p.dc->sc; p.k1 = p.dc->k1; }
@@ -270,6 +339,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
     for (int e = threadIdx.x; e < p.n_predict * 256; e += NTHREADS) {
       const int i = rt * 256 + (e & 255) + (e >> 8);
       tgt[e] = ((e & 255) + rt * 256 < p.N && target_valid(p.targets, p.ignore_index, i, p.N, p.V)) ? (int)p.targets[i] : -1;
+      if (PRE) reinterpret_cast<float*>(smem + FWD_UY_OFF)[e] = p.s_uy[(int64_t)(e >> 8) * p.Np + rt * 256 + (e & 255)];
     }
   }
   __syncthreads();
@@ -305,17 +375,45 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
       // (one code path for the epilogue: with a second one for the last tile of the vocabulary, each with its MFMAs, the
       // accumulators are spilled; columns that do not exist are struck out of the finished accumulators instead)
       const bool ragged = vlim < 256;
-      if (ragged) strike_columns_beyond<0, 1>(acc, vlim, wa, stat, p.em2cap);
-      take_target_logits<true, true, true, 256, 0, 1>(acc, tgt, p.n_predict, col0, row0, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2, p.em2cap);
-      uint32_t ew = form_dlogits<true, NTHREADS, 64, 0, 1>(acc, p.k1, p.c2, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, tail);
-      if (ragged) strike_columns_beyond<1, 2>(acc, vlim, wa, stat, p.em2cap);
-      take_target_logits<true, true, true, 256, 1, 2>(acc, tgt, p.n_predict, col0, row0, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2, p.em2cap);
-      ew |= form_dlogits<true, NTHREADS, 64, 1, 2>(acc, p.k1, p.c2, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, tail);
-      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // every wave has read its last fragment
-      prefetch();
-      if (ragged) strike_columns_beyond<2, 4>(acc, vlim, wa, stat, p.em2cap);
-      take_target_logits<true, true, true, 256, 2, 4>(acc, tgt, p.n_predict, col0, row0, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2, p.em2cap);
-      ew |= form_dlogits<true, NTHREADS, 64, 2, 4>(acc, p.k1, p.c2, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0);
+      uint32_t ew;
+      if (PRE) {
+        // which of the lane's values of row block b is a target of its row (one is looked for: two targets of a row in one
+        // lane's 64 columns are the same column, or rare enough that the second may set an exponent): its known value
+        const float* tuy = reinterpret_cast<const float*>(smem + FWD_UY_OFF) + wb * 128;
+        auto target_value = [&](int b) {
+          float v = __builtin_nanf("");
+          for (int k = 0; k < p.n_predict; ++k) {
+            const int rel = tgt[k * 256 + b * 32 + (lane_id() & 31)] - col0;
+            if ((unsigned)rel < 128u && ((rel >> 2) & 1) == (lane_id() >> 5)) v = tuy[k * 256 + b * 32 + (lane_id() & 31)];
+          }
+          return v;
+        };
+        float xc[4];
+        if (ragged) strike_columns_beyond<0, 1>(acc, vlim, wa, stat, p.em2cap);
+        xc[0] = target_value(0);
+        ew = form_dlogits<true, NTHREADS, 64, 0, 1, decltype(tail)&, true>(acc, p.k1, p.c2, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, tail, xc, p.sc);
+        if (ragged) strike_columns_beyond<1, 2>(acc, vlim, wa, stat, p.em2cap);
+        xc[1] = target_value(1);
+        ew |= form_dlogits<true, NTHREADS, 64, 1, 2, decltype(tail)&, true>(acc, p.k1, p.c2, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, tail, xc, p.sc);
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // every wave has read its last fragment
+        prefetch();
+        if (ragged) strike_columns_beyond<2, 4>(acc, vlim, wa, stat, p.em2cap);
+        xc[2] = target_value(2); xc[3] = target_value(3);
+        NoHook none;
+        ew |= form_dlogits<true, NTHREADS, 64, 2, 4, NoHook&, true>(acc, p.k1, p.c2, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, none, xc, p.sc);
+      } else {
+        if (ragged) strike_columns_beyond<0, 1>(acc, vlim, wa, stat, p.em2cap);
+        take_target_logits<true, true, true, 256, 0, 1>(acc, tgt, p.n_predict, col0, row0, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2, p.em2cap);
+        ew = form_dlogits<true, NTHREADS, 64, 0, 1>(acc, p.k1, p.c2, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, tail);
+        if (ragged) strike_columns_beyond<1, 2>(acc, vlim, wa, stat, p.em2cap);
+        take_target_logits<true, true, true, 256, 1, 2>(acc, tgt, p.n_predict, col0, row0, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2, p.em2cap);
+        ew |= form_dlogits<true, NTHREADS, 64, 1, 2>(acc, p.k1, p.c2, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, tail);
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // every wave has read its last fragment
+        prefetch();
+        if (ragged) strike_columns_beyond<2, 4>(acc, vlim, wa, stat, p.em2cap);
+        take_target_logits<true, true, true, 256, 2, 4>(acc, tgt, p.n_predict, col0, row0, p.sc, p.s_uy, p.Np, stat, p.k1, p.ic2, p.em2cap);
+        ew |= form_dlogits<true, NTHREADS, 64, 2, 4>(acc, p.k1, p.c2, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0);
+      }
       if (lane_id() == 0) p.gexp[(int64_t)(2 * ct + wa) * p.kbw + 2 * rt + wb] = ew;
     } else {
       float sum[4], amax[4];

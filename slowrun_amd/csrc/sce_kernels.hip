@@ -26,6 +26,7 @@
 #include <stdlib.h>
 #include <string.h>
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 #include <type_traits>
 #include <vector>
@@ -80,6 +81,7 @@ constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)8 << 20;
 static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
 
 static std::mutex g_mu;
+static std::atomic<int64_t> g_gather_limit{(int64_t)1 << 32};   // see sce_test_set_gather_limit
 static int g_arch_ok[64];   // 0 unknown, 1 gfx950, -1 other
 static void* g_scratch[64]; // device address of `scratch` on each device, filled with g_arch_ok
 static int g_cus[64];       // compute units, filled with g_arch_ok
@@ -140,7 +142,9 @@ static int check_device(int dev) {
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
-      HIP_TRY(hipFuncSetAttribute((const void*)fwd_sample_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_SAMPLE));
+      HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<true, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
+      HIP_TRY(hipFuncSetAttribute((const void*)fwd_sample_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_SAMPLE));
+      HIP_TRY(hipFuncSetAttribute((const void*)fwd_sample_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_SAMPLE));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_recompute_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_RECOMPUTE));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
@@ -265,6 +269,10 @@ static int dw_launches(const SavedLayout& S, int64_t Pw) {
 }
 
 extern "C" int sce_version(void) { return SCE_VERSION; }
+
+extern "C" int64_t sce_test_set_gather_limit(int64_t bytes) {
+  return g_gather_limit.exchange(bytes > 0 && bytes < ((int64_t)1 << 32) ? bytes : (int64_t)1 << 32);
+}
 
 extern "C" int sce_timing_enable(int on) {
   std::lock_guard<std::mutex> lk(g_timing_mu);
@@ -505,17 +513,27 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
   p.dc = bf16ops ? nullptr : dcp;
   p.want_argmax = a->argmax != nullptr;
   const int grid = 8 * nsplit * ((RT + 7) / 8);
+  // An emitting forward pass has its target logits computed ahead of the forward kernel (with the rows' boosts, from a tile
+  // of gathered rows of W_q^T) as long as that tile's 32-bit offsets reach every row of W_q^T; beyond, the forward kernel
+  // takes them out of its own accumulators, as the other kinds of forward pass do.
+  const bool pre = emit && !bf16ops && (int64_t)S.Vp * S.ldx < g_gather_limit;
   {
     // the exponent boosts of the rows, estimated from two tiles of their logits: only for a forward pass
     // that emits the dlogits (a backward pass that forms them again knows the rows' sums and takes the boosts from those)
     KernelTimer tm(SCE_K_QUANT, st);
     float* lam = (float*)(sv + S.off_lam);
     p.lam = lam;
-    if (!bf16ops && emit) fwd_sample_kernel<<<RT, NTHREADS, SMEM_SAMPLE, st>>>(p, CT / 2, lam);
+    if (!bf16ops && emit) {
+      if (pre) fwd_sample_kernel<true><<<RT, NTHREADS, SMEM_SAMPLE, st>>>(p, CT / 2, lam);
+      else fwd_sample_kernel<false><<<RT, NTHREADS, SMEM_SAMPLE, st>>>(p, CT / 2, lam);
+    }
   }
   {
     KernelTimer tm(SCE_K_FWD, st);
-    if (emit) fwd_kernel<true><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
+    if (emit && pre) {
+      fwd_kernel<true, false, true><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
+      fwd_knock_kernel<<<(int)(S.Np / 256), 256, 0, st>>>(p.ghat_t, p.kbv, a->targets, a->ignore_index, (int)N, (int)Vl, a->shape.n_predict);
+    } else if (emit) fwd_kernel<true><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
     else if (bf16ops) fwd_kernel<false, true><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
     else fwd_kernel<false><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
   }

@@ -653,3 +653,43 @@ def test_softcap_range(cap, keep):
     rep = pu.check_parity(ours, ref, "mean")
     assert rep["n_ignored"] > 0
     print(rep)
+
+
+@pytest.mark.parametrize("n_predict", [1, 3, 4])
+@pytest.mark.parametrize("shape", [(700, 272, 2049), (513, 64, 300), (256, 128, 1000), (1031, 528, 5000)])
+def test_target_logits_ahead_of_the_forward_kernel(shape, n_predict):
+    """A forward pass that emits the dlogits gets its target logits from a tile of gathered rows of W_q^T, computed before
+    the forward kernel (which then never looks for a target in its accumulators), or -- for a W_q^T beyond the gather's
+    32-bit offsets -- from the forward kernel's own accumulators.  sce_test_set_gather_limit forces the second way at a
+    size a test can afford.  The argmax of the two ways is the same; the row sums take the target's term in at a
+    different place (lse within 2 ulp, the losses with it), and the gradients agree up to the rounding of the
+    dlogits (the blocks' exponents are found differently)."""
+    from slowrun_amd import _lib, cuda_kernels as ck
+    N, d, V = shape
+    g = torch.Generator().manual_seed(N + n_predict)
+    from tests.test_gpu_parity_peaked import make_peaked
+    inp = make_peaked(N, d, V, 12.0, shared=True, seed=N, ignore=0.1)
+    x, w, y = inp.x.cuda(), inp.w.cuda(), inp.targets.cuda().clone()
+    y[5:9] = y[5]                                  # offsets of one row with the same target
+    y[N - 2] = -1
+    mw = torch.rand(n_predict, generator=g).cuda() + 0.1 if n_predict > 1 else None
+    go = (torch.rand(N, generator=g) / N).cuda()
+    res = []
+    lib = _lib.lib()
+    try:
+        for limit in (0, 1):
+            lib.sce_test_set_gather_limit(limit)
+            out, saved, lse, am, nv = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, "none", mtp_weights=mw, keep_dlogits=True, want_argmax=True)
+            dx, dw = ck.ce_backward(saved, y, go, N, d, V, inp.x_s, inp.w_s, inp.cap, 1.0, "none", torch.float32, torch.float32,
+                                    mtp_weights=mw, keep_dlogits=True)
+            torch.cuda.synchronize()
+            res.append((out.clone(), lse.clone(), am.clone(), nv.clone(), dx.clone(), dw.clone()))
+    finally:
+        lib.sce_test_set_gather_limit(0)
+    a, b = res
+    assert torch.equal(a[2], b[2]) and torch.equal(a[3], b[3])
+    assert float((a[1] - b[1]).abs().max()) <= 4e-6 * float(b[1].abs().max().clamp_min(1.0))
+    assert float((a[0] - b[0]).abs().max()) <= 2e-5
+    for name, u, v in (("dx", a[4], b[4]), ("dw", a[5], b[5])):
+        mr, cs = pu.maxrel(u, v), pu.cosine(u, v)
+        assert mr <= pu.GRAD_MAXREL and cs > pu.GRAD_COS, (name, mr, cs)

@@ -15,7 +15,8 @@ from slowrun_amd import build
 pytestmark = pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
 
 # one wave per SIMD, all accumulators in registers, nothing in scratch memory
-HOT = ["fwd_kernel<true, false>", "fwd_kernel<false, false>", "fwd_kernel<false, true>", "fwd_sample_kernel", "bwd_recompute_kernel",
+HOT = ["fwd_kernel<true, false, true>", "fwd_kernel<true, false, false>", "fwd_kernel<false, false, false>", "fwd_kernel<false, true, false>",
+       "fwd_sample_kernel<true>", "fwd_sample_kernel<false>", "bwd_recompute_kernel",
        "bwd_dx_kernel<bf16_t, false>", "bwd_dx_kernel<float, false>", "bwd_dx_kernel<bf16_t, true>", "bwd_dx_kernel<float, true>",
        "bwd_dw_kernel<false>", "bwd_dw_kernel<true>", "bwd_dw_tail_kernel", "bench_gemm_kernel", "floor_fwd_kernel", "floor_dx_kernel",
        "floor_dw_kernel"]
