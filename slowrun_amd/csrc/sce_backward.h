@@ -43,6 +43,8 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const float* __restrict__
     rowinfo[i] = __float_as_int(lam_i);
     for (int k = 0; k < 4; ++k)
       rowinfo[(int64_t)(1 + k) * Np + i] = (k < n_predict && i < N && target_valid(targets, ignore_index, i + k, N, V)) ? (int)targets[i + k] : -1;
+    for (int k = 0; k < 4; ++k)          // and the target logits as the forward pass saved them: the recompute kernel knows its targets by these values
+      rowinfo[(int64_t)(5 + k) * Np + i] = (k < n_predict && i < N) ? __float_as_int(s_zy[(int64_t)k * Np + i]) : 0x7fc00000;
   }
   if (i < N) {
     const float g = (per_row ? grad_output[i] : grad_output[0] / (float)hdr[0]) * grad_scale;
@@ -153,18 +155,18 @@ struct RecomputeParams {
   int64_t dp, ldx;             // K extent and row stride of xq / wqt
   int64_t kbw, kb0, kbv;       // blocks of 128 rows in the buffer (row stride of gexp), block of this panel's first row, blocks of 128 columns
   int RT, CT, V;
-  float k1, c2;          // as in FwdParams
-  const DevConsts* dc;   // non-NULL: k1 comes from here
+  float k1, c2, sc;      // as in FwdParams
+  const DevConsts* dc;   // non-NULL: k1 and sc come from here
 };
 
 // Recompute a 256 x 256 logit tile and leave its block-scaled dlogits in G (16-byte stores straight from the registers).
-constexpr int ROWINFO_PLANES = 5;                      // per row: exponent boost (a float), then the target column of each of 4 offsets (or -1)
+constexpr int ROWINFO_PLANES = 9;                      // per row: exponent boost (a float), the target column of each of 4 offsets (or -1), the target logits
 constexpr int SMEM_RECOMPUTE = SMEM_BYTES + 4 * ROWINFO_PLANES * 512;      // two K slots + the row data of 128 rows per wave
 
 __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p_in) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   RecomputeParams p = p_in;
-  if (p.dc) p.k1 = p.dc->k1;
+  if (p.dc) { p.k1 = p.dc->k1; p.sc = p.dc->sc; }
   int rt, ct;
   if (!map_tile(blockIdx.x, p.RT, p.CT, rt, ct)) return;
   // The tile order goes through the columns in groups of 8, and it does so from the last group to the first:
@@ -202,15 +204,30 @@ __global__ __launch_bounds__(256) void bwd_recompute_kernel(RecomputeParams p_in
   const int* tgt = reinterpret_cast<const int*>(smem + SMEM_BYTES) + wave * (ROWINFO_PLANES * 128) + 128;
   uint8_t* gq = const_cast<uint8_t*>(uniform_ptr(p.ghat_t + ((p.kb0 / 2 + rt) * p.kbv + 2 * ct + wa) * BLOCKED_KSTEP + wb * 128 * BK));      // the wave's quadrant of G
   const int col0 = ct * 256 + wa * 128;
+  // The target entries are not looked up in the accumulators (the compiler moves a row block's 64 accumulators around
+  // every such lookup): a lane knows the value of a target among its columns -- the forward pass saved it, and this
+  // kernel computes the same number -- and keeps it out of the block exponent by that (form_dlogits, EXCL); the bytes
+  // are cleared afterwards (fwd_knock_kernel).
+  const float* tval = reinterpret_cast<const float*>(tgt + 4 * 128);
+  auto target_value = [&](int b) {
+    float v = __builtin_nanf("");
+    for (int k = 0; k < p.n_predict; ++k) {
+      const int rel = tgt[k * 128 + b * 32 + (lane_id() & 31)] - col0;
+      if ((unsigned)rel < 128u && ((rel >> 2) & 1) == (lane_id() >> 5)) v = tval[k * 128 + b * 32 + (lane_id() & 31)];
+    }
+    return v;
+  };
+  float xc[4];
   if (ragged) strike_columns_beyond<0, 1>(acc, vlim, wa);
-  take_target_logits<false, true, false, 128, 0, 1>(acc, tgt, p.n_predict, col0, 0, 0.f, nullptr, 0, nullptr, 0.f, 0.f, 0.f);
-  uint32_t ew = form_dlogits<false, 32, 32, 0, 1>(acc, p.k1, p.c2, 0, gq, wa, wb, nullptr, lam, false, tail);
+  xc[0] = target_value(0);
+  uint32_t ew = form_dlogits<false, 32, 32, 0, 1, decltype(tail)&, true>(acc, p.k1, p.c2, 0, gq, wa, wb, nullptr, lam, false, tail, xc, p.sc);
   if (ragged) strike_columns_beyond<1, 2>(acc, vlim, wa);
-  take_target_logits<false, true, false, 128, 1, 2>(acc, tgt, p.n_predict, col0, 0, 0.f, nullptr, 0, nullptr, 0.f, 0.f, 0.f);
-  ew |= form_dlogits<false, 32, 32, 1, 2>(acc, p.k1, p.c2, 0, gq, wa, wb, nullptr, lam, false, tail);
+  xc[1] = target_value(1);
+  ew |= form_dlogits<false, 32, 32, 1, 2, decltype(tail)&, true>(acc, p.k1, p.c2, 0, gq, wa, wb, nullptr, lam, false, tail, xc, p.sc);
   if (ragged) strike_columns_beyond<2, 4>(acc, vlim, wa);
-  take_target_logits<false, true, false, 128, 2, 4>(acc, tgt, p.n_predict, col0, 0, 0.f, nullptr, 0, nullptr, 0.f, 0.f, 0.f);
-  ew |= form_dlogits<false, 32, 32, 2, 4>(acc, p.k1, p.c2, 0, gq, wa, wb, nullptr, lam, false);
+  xc[2] = target_value(2); xc[3] = target_value(3);
+  NoHook none;
+  ew |= form_dlogits<false, 32, 32, 2, 4, NoHook&, true>(acc, p.k1, p.c2, 0, gq, wa, wb, nullptr, lam, false, none, xc, p.sc);
   if (lane_id() == 0) p.gexp[(int64_t)(2 * ct + wa) * p.kbw + p.kb0 + 2 * rt + wb] = ew;
 }
 

@@ -165,8 +165,11 @@ __device__ __forceinline__ void take_target_logits(v16f (&acc)[4][4], const int*
 // tile's last rows point at targets of the next tile's rows: those (at most three) ride as the last columns of the
 // first tile, in place of the sampled columns there.
 constexpr int SMEM_SAMPLE = SMEM_BYTES + 2 * 256 * 4 + 8 * 256 * 4;      // the K slots, the gathered rows, the rows without a target, the first tile's results
-template <bool GATHER>
+// BOOST = false (with GATHER): the target logits only, for a forward pass that emits nothing (the first tile is then
+// computed only for the sake of its last columns, i.e. with more than one offset).
+template <bool GATHER, bool BOOST = true>
 __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct, float* __restrict__ lam_out) {
+  static_assert(GATHER || BOOST, "nothing to do");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   FwdParams p = p_in;
   if (p.dc) { p.sc = p.dc->sc; p.k1 = p.dc->k1; }
@@ -190,8 +193,11 @@ __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct,
     yraw[k] = (k < p.n_predict && row + k < p.N && row < p.N) ? p.targets[row + k] : p.ignore_index;
   }
   v16f acc[4][4];
-  if (GATHER) mfma_mainloop(p.wqt, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 0, 0, wave, NoHook(), 0, 0, nullptr, rows);
-  else mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 0, 0, wave);
+  const bool first_tile = BOOST || ntail > 0;
+  if (first_tile) {
+    if (GATHER) mfma_mainloop(p.wqt, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 0, 0, wave, NoHook(), 0, 0, nullptr, rows);
+    else mfma_mainloop(p.wqt + (int64_t)ct * 256 * p.ldx, p.ldx, p.xq + (int64_t)rt * 256 * p.ldx, p.ldx, (int)(p.dp / BK), smem, acc, 0, 0, wave);
+  }
   {
     bool any = false;
 #pragma unroll
@@ -200,7 +206,7 @@ __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct,
     dead[threadIdx.x] = !any;
   }
   const int lane = lane_id();
-  if (GATHER) {
+  if (GATHER && first_tile) {
     // columns 252 .. 255 are registers 12 .. 15 of A block 3 in the upper half-wave of the waves with wa = 1; rows 224 .. 255
     // are B block 3 of the waves with wb = 1
     const int i = 224 + (lane & 31);
@@ -216,6 +222,7 @@ __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct,
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
     gmin[b] = INFINITY; top[b] = -INFINITY;
+    if (!BOOST) continue;
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
       float sum = 0.f, cnt = 0.f;
@@ -240,12 +247,14 @@ __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct,
     keep = reinterpret_cast<float*>(smem + SMEM_BYTES + 2048) + wave * 64 + lane_id();
 #pragma unroll
     for (int b = 0; b < 4; ++b) { gmin[b] = keep[b * 256]; top[b] = keep[(4 + b) * 256]; }
+    if (BOOST) {
 #pragma unroll
-    for (int b = 0; b < 4; ++b)
+      for (int b = 0; b < 4; ++b)
 #pragma unroll
-      for (int a = 0; a < 4; ++a)
+        for (int a = 0; a < 4; ++a)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) top[b] = fmaxf(top[b], acc[a][b][r]);
+          for (int r = 0; r < 16; ++r) top[b] = fmaxf(top[b], acc[a][b][r]);
+    }
     // The band 0 <= column - row < n_predict lies in the 32 x 32 blocks on the diagonal and right of it: blocks (a, b) with
     // a - b = 0 or 1 of the waves with wa = wb, block (0, 3) of the wave with wa = 1, wb = 0.  (Stores under a lane
     // condition, no branches around the accumulators.)
@@ -265,6 +274,7 @@ __global__ __launch_bounds__(256) void fwd_sample_kernel(FwdParams p_in, int ct,
         __builtin_amdgcn_sched_barrier(0);      // (one block's accumulators at a time: all of them moved up front do not fit the registers)
       }
   }
+  if (!BOOST) return;
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
     gmin[b] = fminf(gmin[b], __shfl_xor(gmin[b], 32));
@@ -313,12 +323,12 @@ static_assert(SMEM_BYTES <= FWD_UY_OFF, "K slots and row data overlap");
 // EMIT: the epilogue also leaves the block-scaled dlogits of the tile in G (see form_dlogits), for a backward pass
 // that does not compute the logits again.
 // BF16 (without EMIT): bf16 operands, logits rounded to bf16 as the eager head's GEMM returns them (forward only).
-// PRE (with EMIT): the target logits are in s_uy already (fwd_sample_kernel<true>) and this kernel does not look for them in
-// its accumulators; the target entries go through the epilogue like any other, except that they are kept out of the block
-// exponents (form_dlogits, EXCL), and fwd_knock_kernel clears their bytes of G afterwards.
+// PRE: the target logits are in s_uy already (fwd_sample_kernel<true, .>) and this kernel does not look for them in
+// its accumulators.  With EMIT the target entries go through the epilogue like any other, except that they are kept out
+// of the block exponents (form_dlogits, EXCL), and fwd_knock_kernel clears their bytes of G afterwards.
 template <bool EMIT, bool BF16 = false, bool PRE = false>
 __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
-  static_assert(!PRE || EMIT, "PRE belongs to the emitting kernel");
+  static_assert(!PRE || !BF16, "PRE is for the fp8 kernels");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   FwdParams p = p_in;
   if (p.dc) { p.sc = p.dc->sc; p.k1 = p.dc->k1; }
@@ -339,7 +349,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
     for (int e = threadIdx.x; e < p.n_predict * 256; e += NTHREADS) {
       const int i = rt * 256 + (e & 255) + (e >> 8);
       tgt[e] = ((e & 255) + rt * 256 < p.N && target_valid(p.targets, p.ignore_index, i, p.N, p.V)) ? (int)p.targets[i] : -1;
-      if (PRE) reinterpret_cast<float*>(smem + FWD_UY_OFF)[e] = p.s_uy[(int64_t)(e >> 8) * p.Np + rt * 256 + (e & 255)];
+      if (PRE && EMIT) reinterpret_cast<float*>(smem + FWD_UY_OFF)[e] = p.s_uy[(int64_t)(e >> 8) * p.Np + rt * 256 + (e & 255)];
     }
   }
   __syncthreads();
@@ -438,7 +448,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
         stat[(0 + b) * NTHREADS] = sum[b]; stat[(4 + b) * NTHREADS] = amax[b]; stat[(8 + b) * NTHREADS] = __int_as_float(uarg[b]);
       }
     }
-    if (!EMIT) take_target_logits<true, false, false, 256>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, nullptr, 0.f, 0.f, 0.f);
+    if (!EMIT && !PRE) take_target_logits<true, false, false, 256>(acc, tgt, p.n_predict, ct * 256 + wa * 128, rt * 256 + wb * 128, p.sc, p.s_uy, p.Np, nullptr, 0.f, 0.f, 0.f);
   }
   float sum[4], amax[4];
   int uarg[4];

@@ -145,6 +145,8 @@ static int check_device(int dev) {
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<true, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_sample_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_SAMPLE));
       HIP_TRY(hipFuncSetAttribute((const void*)fwd_sample_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_SAMPLE));
+      HIP_TRY(hipFuncSetAttribute((const void*)fwd_sample_kernel<true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_SAMPLE));
+      HIP_TRY(hipFuncSetAttribute((const void*)fwd_kernel<false, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_FWD));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_recompute_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_RECOMPUTE));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<float, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
       HIP_TRY(hipFuncSetAttribute((const void*)bwd_dx_kernel<bf16_t, false>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_MAX));
@@ -513,10 +515,10 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
   p.dc = bf16ops ? nullptr : dcp;
   p.want_argmax = a->argmax != nullptr;
   const int grid = 8 * nsplit * ((RT + 7) / 8);
-  // An emitting forward pass has its target logits computed ahead of the forward kernel (with the rows' boosts, from a tile
-  // of gathered rows of W_q^T) as long as that tile's 32-bit offsets reach every row of W_q^T; beyond, the forward kernel
-  // takes them out of its own accumulators, as the other kinds of forward pass do.
-  const bool pre = emit && !bf16ops && (int64_t)S.Vp * S.ldx < g_gather_limit;
+  // An fp8 forward pass has its target logits computed ahead of the forward kernel (from a tile of gathered rows of W_q^T,
+  // together with the rows' boosts when it emits the dlogits) as long as that tile's 32-bit offsets reach every row of
+  // W_q^T; beyond, the forward kernel takes them out of its own accumulators, as the bf16 forward pass does.
+  const bool pre = !bf16ops && (int64_t)S.Vp * S.ldx < g_gather_limit;
   {
     // the exponent boosts of the rows, estimated from two tiles of their logits: only for a forward pass
     // that emits the dlogits (a backward pass that forms them again knows the rows' sums and takes the boosts from those)
@@ -526,7 +528,7 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
     if (!bf16ops && emit) {
       if (pre) fwd_sample_kernel<true><<<RT, NTHREADS, SMEM_SAMPLE, st>>>(p, CT / 2, lam);
       else fwd_sample_kernel<false><<<RT, NTHREADS, SMEM_SAMPLE, st>>>(p, CT / 2, lam);
-    }
+    } else if (pre) fwd_sample_kernel<true, false><<<RT, NTHREADS, SMEM_SAMPLE, st>>>(p, CT / 2, lam);
   }
   {
     KernelTimer tm(SCE_K_FWD, st);
@@ -535,6 +537,7 @@ static int forward_impl(const sce_args* a, void* ws, size_t ws_bytes, const char
       fwd_knock_kernel<<<(int)(S.Np / 256), 256, 0, st>>>(p.ghat_t, p.kbv, a->targets, a->ignore_index, (int)N, (int)Vl, a->shape.n_predict);
     } else if (emit) fwd_kernel<true><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
     else if (bf16ops) fwd_kernel<false, true><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
+    else if (pre) fwd_kernel<false, false, true><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
     else fwd_kernel<false><<<grid, NTHREADS, SMEM_FWD, st>>>(p);
   }
   KernelTimer tm_red(SCE_K_FWD_REDUCE, st);
@@ -688,7 +691,7 @@ extern "C" int sce_backward(const sce_args* a) {
     bwd_longlist_kernel<<<(int)((V + 255) / 256), 256, 0, st>>>(segoff, (int)V, longlist, longbase);
   }
   delete tm_prep;
-  const float k1 = (float)a->x_s * (float)a->w_s * 2.0f * LOG2E / a->cap, c2 = -2.0f * a->cap * LOG2E;
+  const float sc = (float)a->x_s * (float)a->w_s, k1 = sc * 2.0f * LOG2E / a->cap, c2 = -2.0f * a->cap * LOG2E;
   const int CTv = (int)(S.Vp / 256), CTd = (int)(S.dq / 256);
   int launch = 0;
   DwTail tail;
@@ -769,10 +772,13 @@ extern "C" int sce_backward(const sce_args* a) {
       const int64_t gorg = w0;                                    // the row that K block 0 of the dlogits buffer stands for
       RecomputeParams rp;
       rp.xq = xq + p0 * S.ldx; rp.wqt = wqt; rp.ghat_t = ghat_t; rp.gexp = gexp; rp.rowinfo = rowinfo + p0; rp.Np = S.Np; rp.n_predict = K;
-      rp.dp = S.dp; rp.ldx = S.ldx; rp.kbw = gkb; rp.kbv = S.Vp / BK; rp.kb0 = (p0 - gorg) / BK; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2; rp.dc = dcp;
+      rp.dp = S.dp; rp.ldx = S.ldx; rp.kbw = gkb; rp.kbv = S.Vp / BK; rp.kb0 = (p0 - gorg) / BK; rp.RT = RTp; rp.CT = CTv; rp.V = (int)Vl; rp.k1 = k1; rp.c2 = c2; rp.sc = sc; rp.dc = dcp;
       {
         KernelTimer tm(SCE_K_RECOMPUTE, st);
         bwd_recompute_kernel<<<map_tile_grid(RTp, CTv), NTHREADS, SMEM_RECOMPUTE, st>>>(rp);
+        if (p0 < N)       // the target entries of the panel's rows are cleared (rows p0 on: tiles (p0 - gorg) / 256 on of the buffer)
+          fwd_knock_kernel<<<(int)(prow / 256), 256, 0, st>>>(ghat_t + (size_t)((p0 - gorg) / 256) * (S.Vp / BK) * BLOCKED_KSTEP, S.Vp / BK, a->targets + p0,
+                                                          a->ignore_index, (int)(N - p0), (int)Vl, K);
       }
       dx_panel(p0, prow, gorg);
       const int64_t gathered = p0 + prow - w0;

@@ -655,15 +655,17 @@ def test_softcap_range(cap, keep):
     print(rep)
 
 
+@pytest.mark.parametrize("keep", [True, False])
 @pytest.mark.parametrize("n_predict", [1, 3, 4])
 @pytest.mark.parametrize("shape", [(700, 272, 2049), (513, 64, 300), (256, 128, 1000), (1031, 528, 5000)])
-def test_target_logits_ahead_of_the_forward_kernel(shape, n_predict):
-    """A forward pass that emits the dlogits gets its target logits from a tile of gathered rows of W_q^T, computed before
+def test_target_logits_ahead_of_the_forward_kernel(shape, n_predict, keep):
+    """An fp8 forward pass gets its target logits from a tile of gathered rows of W_q^T, computed before
     the forward kernel (which then never looks for a target in its accumulators), or -- for a W_q^T beyond the gather's
     32-bit offsets -- from the forward kernel's own accumulators.  sce_test_set_gather_limit forces the second way at a
     size a test can afford.  The argmax of the two ways is the same; the row sums take the target's term in at a
     different place (lse within 2 ulp, the losses with it), and the gradients agree up to the rounding of the
-    dlogits (the blocks' exponents are found differently)."""
+    dlogits (the blocks' exponents are found differently).  A forward pass that emits nothing does the same sums either
+    way, and the backward pass that follows it is the same code: everything is equal bit for bit."""
     from slowrun_amd import _lib, cuda_kernels as ck
     N, d, V = shape
     g = torch.Generator().manual_seed(N + n_predict)
@@ -679,14 +681,17 @@ def test_target_logits_ahead_of_the_forward_kernel(shape, n_predict):
     try:
         for limit in (0, 1):
             lib.sce_test_set_gather_limit(limit)
-            out, saved, lse, am, nv = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, "none", mtp_weights=mw, keep_dlogits=True, want_argmax=True)
+            out, saved, lse, am, nv = ck.ce_forward(x, w, y, inp.x_s, inp.w_s, inp.cap, "none", mtp_weights=mw, keep_dlogits=keep, want_argmax=True)
             dx, dw = ck.ce_backward(saved, y, go, N, d, V, inp.x_s, inp.w_s, inp.cap, 1.0, "none", torch.float32, torch.float32,
-                                    mtp_weights=mw, keep_dlogits=True)
+                                    mtp_weights=mw, keep_dlogits=keep)
             torch.cuda.synchronize()
             res.append((out.clone(), lse.clone(), am.clone(), nv.clone(), dx.clone(), dw.clone()))
     finally:
         lib.sce_test_set_gather_limit(0)
     a, b = res
+    if not keep:
+        assert all(torch.equal(u, v) for u, v in zip(a, b))
+        return
     assert torch.equal(a[2], b[2]) and torch.equal(a[3], b[3])
     assert float((a[1] - b[1]).abs().max()) <= 4e-6 * float(b[1].abs().max().clamp_min(1.0))
     assert float((a[0] - b[0]).abs().max()) <= 2e-5

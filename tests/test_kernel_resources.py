@@ -15,11 +15,13 @@ from slowrun_amd import build
 pytestmark = pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
 
 # one wave per SIMD, all accumulators in registers, nothing in scratch memory
-HOT = ["fwd_kernel<true, false, true>", "fwd_kernel<true, false, false>", "fwd_kernel<false, false, false>", "fwd_kernel<false, true, false>",
-       "fwd_sample_kernel<true>", "fwd_sample_kernel<false>", "bwd_recompute_kernel",
+HOT = ["fwd_kernel<true, false, true>", "fwd_kernel<true, false, false>", "fwd_kernel<false, false, true>", "fwd_kernel<false, false, false>",
+       "fwd_kernel<false, true, false>", "fwd_sample_kernel<true, true>", "fwd_sample_kernel<false, true>", "bwd_recompute_kernel",
        "bwd_dx_kernel<bf16_t, false>", "bwd_dx_kernel<float, false>", "bwd_dx_kernel<bf16_t, true>", "bwd_dx_kernel<float, true>",
        "bwd_dw_kernel<false>", "bwd_dw_kernel<true>", "bwd_dw_tail_kernel", "bench_gemm_kernel", "floor_fwd_kernel", "floor_dx_kernel",
        "floor_dw_kernel"]
+# the same, except that the compiler keeps part of the accumulators in architectural registers (its epilogue is a few stores)
+HOT_ANY_AGPRS = ["fwd_sample_kernel<true, false>"]
 # known to spill to scratch (a measurement aid); the bound is what was measured, so that it does not grow unseen
 SCRATCH_BOUND = {"bench_mfma_kernel": 16}
 
@@ -30,7 +32,7 @@ def table():
 
 
 def test_every_kernel_is_reported(table):
-    for k in HOT + list(SCRATCH_BOUND):
+    for k in HOT + HOT_ANY_AGPRS + list(SCRATCH_BOUND):
         assert k in table, f"{k} missing from the compiler's resource remarks: {sorted(table)}"
 
 
@@ -39,6 +41,12 @@ def test_hot_mfma_kernels_keep_everything_in_registers(table, kernel):
     r = table[kernel]
     assert r["scratch"] == 0 and r["vgpr_spill"] == 0, f"{kernel} spills to scratch memory: {r}"
     assert r["occupancy"] == 1 and r["agprs"] == 256, f"{kernel}: one wave per SIMD with 256 accumulation registers expected: {r}"
+
+
+@pytest.mark.parametrize("kernel", HOT_ANY_AGPRS)
+def test_other_mfma_kernels_keep_everything_in_registers(table, kernel):
+    r = table[kernel]
+    assert r["scratch"] == 0 and r["vgpr_spill"] == 0 and r["occupancy"] == 1, f"{kernel}: {r}"
 
 
 @pytest.mark.parametrize("kernel", sorted(SCRATCH_BOUND))
