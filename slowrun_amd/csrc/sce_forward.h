@@ -398,17 +398,16 @@ __global__ __launch_bounds__(256) void fwd_kernel(FwdParams p_in) {
           }
           return v;
         };
-        float xc[4];
+        float xc[4];                                   // (looked up a row block ahead of their use: the LDS reads have time)
         if (ragged) strike_columns_beyond<0, 1>(acc, vlim, wa, stat, p.em2cap);
-        xc[0] = target_value(0);
+        xc[0] = target_value(0); xc[1] = target_value(1);
         ew = form_dlogits<true, NTHREADS, 64, 0, 1, decltype(tail)&, true>(acc, p.k1, p.c2, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, tail, xc, p.sc);
         if (ragged) strike_columns_beyond<1, 2>(acc, vlim, wa, stat, p.em2cap);
-        xc[1] = target_value(1);
+        xc[2] = target_value(2); xc[3] = target_value(3);
         ew |= form_dlogits<true, NTHREADS, 64, 1, 2, decltype(tail)&, true>(acc, p.k1, p.c2, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, tail, xc, p.sc);
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // every wave has read its last fragment
         prefetch();
         if (ragged) strike_columns_beyond<2, 4>(acc, vlim, wa, stat, p.em2cap);
-        xc[2] = target_value(2); xc[3] = target_value(3);
         NoHook none;
         ew |= form_dlogits<true, NTHREADS, 64, 2, 4, NoHook&, true>(acc, p.k1, p.c2, vbase, gq, wa, wb, stat, lam, p.want_argmax != 0, none, xc, p.sc);
       } else {
