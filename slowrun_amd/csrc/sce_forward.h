@@ -13,7 +13,7 @@ struct FwdParams {
   const uint8_t* wqt;      // [Vp][dp]
   float4* partials;        // [S][Np]: sum exp(z - cap), max u, argmax u (bits), unused
   const int64_t* targets;  // (N,)
-  float* s_uy;             // [n_predict][Np]: raw logit u at the target of (offset, row), written by the workgroup that meets it
+  float* s_uy;             // [n_predict][Np]: raw logit u at the target of (offset, row): from fwd_sample_kernel (PRE), else written by the workgroup that meets it
   uint8_t* ghat_t;         // EMIT: G, all Np rows, tile by tile (kbv blocks of 128 columns per tile of 256 rows)
   uint32_t* gexp;          // EMIT: its block exponents [Vp / 128][kbw]
   const float* lam;        // EMIT: exponent boost of every row
@@ -86,7 +86,10 @@ __device__ __forceinline__ bool target_valid(const int64_t* __restrict__ targets
 // to the largest and drops what falls below about 2^-12 of it: about 2e-5 low on a sum of like-signed terms at K = 2560), and a z_y from a separate fp32 dot product would leave that bias in z_y - lse, i.e. in
 // 1 - p_y, where rows the model is sure of cannot afford it.  tgt (LDS): [4 offsets][TGT_STRIDE rows] target column or
 // -1, already at the wave's first row.  A lane looks at its four rows; the 64-way select runs only when some lane of
-// the wave has a hit (a few per cent of the tiles).
+// the wave has a hit (a few per cent of the tiles) -- but the compiler moves the row block's 64 accumulators out of the
+// accumulation registers around every offset's lookup, hit or not, which is why the fp8 kernels take their target
+// logits from fwd_sample_kernel where they can (PRE) and this function serves the rest: the bf16 kernel, and W_q^T
+// beyond that kernel's reach.
 // STORE: the logit goes to s_uy_tile[offset][row] (global).
 // KNOCK: the accumulator of the target is then set to -inf, for the dlogits epilogue that follows: the target takes
 //        no part in the stored dlogits (its column is handled in fp32, see bwd_prep_kernel) and must not set the
