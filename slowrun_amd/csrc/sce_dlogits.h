@@ -119,12 +119,19 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
       // offers the largest of the others
       const bool is_target = tmax * sc == xc[b];
       if (__builtin_amdgcn_ballot_w64(is_target) != 0) {
+        // (a value that occurs twice among the lane's 64 is not the target alone -- all logits are equal under a head
+        // that starts at zero -- and stays in: the other one needs the exponent)
         float tsec = -INFINITY;
+        int ties = 0;
 #pragma unroll
         for (int a = 0; a < 4; ++a)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) tsec = fmaxf(tsec, acc[a][b][r] == tmax ? -INFINITY : acc[a][b][r]);
-        texp = is_target ? tsec : tmax;
+          for (int r = 0; r < 16; ++r) {
+            const bool same = acc[a][b][r] == tmax;
+            ties += same ? 1 : 0;
+            tsec = fmaxf(tsec, same ? -INFINITY : acc[a][b][r]);
+          }
+        texp = (is_target && ties == 1) ? tsec : tmax;
       }
     }
     const float lamb = lam[b * LAM_STRIDE + (lane_id() & (LAM_LANES - 1))];      // (index taken anew: see lane_id)

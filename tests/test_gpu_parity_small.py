@@ -698,3 +698,56 @@ def test_target_logits_ahead_of_the_forward_kernel(shape, n_predict, keep):
     for name, u, v in (("dx", a[4], b[4]), ("dw", a[5], b[5])):
         mr, cs = pu.maxrel(u, v), pu.cosine(u, v)
         assert mr <= pu.GRAD_MAXREL and cs > pu.GRAD_COS, (name, mr, cs)
+
+
+@pytest.mark.parametrize("keep", [True, False])
+@pytest.mark.parametrize("n_predict", [1, 3])
+def test_head_that_starts_at_zero(keep, n_predict):
+    """All logits are equal (W = 0, as a zero-initialised lm_head has it at the first step; here also a W with a few
+    repeated columns): the target is then not the only one of a lane's values with its value, and the kernels that know
+    their targets by value must not take the others for it."""
+    from slowrun_amd import cuda_kernels as ck
+    from oracle import eager
+    N, d, V = 600, 128, 1500
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(N, d, generator=g).cuda()
+    y = torch.randint(0, V, (N,), generator=g).cuda()
+    y[7] = -1
+    mw = torch.tensor([1.0, 0.5, 0.25][:n_predict]).cuda() if n_predict > 1 else None
+    go = (torch.rand(N, generator=g) / N).cuda()
+    x_s, w_s = float(x.abs().max()) / 448.0, 1.6 / 448.0
+    for w in (torch.zeros(d, V).cuda(), (torch.randn(d, 1, generator=g) * d ** -0.5).expand(d, V).contiguous().cuda()):
+        out, saved, lse, am, nv = ck.ce_forward(x, w, y, x_s, w_s, 15.0, "none", mtp_weights=mw, keep_dlogits=keep)
+        dx, dw = ck.ce_backward(saved, y, go, N, d, V, x_s, w_s, 15.0, 1.0, "none", torch.float32, torch.float32, mtp_weights=mw,
+                                keep_dlogits=keep)
+        torch.cuda.synchronize()
+        assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(dx).all()) and bool(torch.isfinite(dw).all())
+        ref = eager.softcapped_ce_mtp(x, w, y, [1.0, 0.5, 0.25][:n_predict], x_s, w_s, cap=15.0, grad_output=go)
+        assert float((out - ref["loss"]).abs().max() / ref["loss"].abs().max()) < pu.LOSS_RTOL
+        # dX is zero in exact arithmetic (every column of W is the same vector w: sum_v p_v w - w = 0); what comes out is the
+        # rounding of the dlogits, all of a row's alike here, against the scale g w of its two terms
+        scale = float(go.max()) * float(w.abs().max()) * (float(mw.sum()) if mw is not None else 1.0)
+        assert float(dx.abs().max()) <= 0.0625 * scale
+        mr, cs = pu.maxrel(dw, ref["dw"]), pu.cosine(dw, ref["dw"])
+        assert mr <= pu.GRAD_MAXREL and cs > pu.GRAD_COS, ("dw", mr, cs)
+
+
+@pytest.mark.parametrize("keep", [True, False])
+def test_a_column_that_ties_with_the_target(keep):
+    """Two identical columns of W, one of them a row's target and both that row's largest logits by far: the kernels know
+    the target among a lane's values by its value, and the twin has the same value -- it must keep its say in the
+    block's exponent (without it the twin's dlogit overflows the block's range)."""
+    N, d, V = 512, 128, 1024
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(N, d, generator=g)
+    w = torch.randn(d, V, generator=g) * d ** -0.5
+    y = torch.randint(0, V, (N,), generator=g)
+    for i0, c1, c2 in ((3, 8, 16), (200, 300, 308), (411, 900, 1016)):      # same block of 128 columns, same half of the lanes
+        w[:, c1] = w[:, c2] = 10.0 * x[i0] / x[i0].pow(2).sum()
+        y[i0] = c1
+    inp = configs.HeadInputs("twins", x, w, y, float(x.abs().max()) / 448.0, float(w.abs().max()) / 448.0, 15.0)
+    go = torch.full((N,), 1.0 / N, device="cuda")
+    ours = pu.run_ours(inp, "none", x_dtype=torch.float32, w_dtype=torch.float32, grad_output=go, keep_dlogits=keep)
+    assert bool(torch.isfinite(ours["dx"]).all()) and bool(torch.isfinite(ours["dw"]).all())
+    ref = pu.run_oracle(inp, ours, "none", grad_output=go)
+    pu.check_parity(ours, ref, "none")
