@@ -113,7 +113,7 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
       for (int r = 0; r < 16; ++r) {
         tmax = fmaxf(tmax, acc[a][b][r]);
       }
-    float texp = tmax;
+    float texp = tmax, lfloor = -INFINITY;
     if (EXCL) {
       // some lane's largest value is its row's target (seldom, unless the rows are sure of their targets): that lane
       // offers the largest of the others
@@ -131,11 +131,17 @@ __device__ __forceinline__ uint32_t form_dlogits(const v16f (&acc)[4][4], float 
             ties += same ? 1 : 0;
             tsec = fmaxf(tsec, same ? -INFINITY : acc[a][b][r]);
           }
-        texp = (is_target && ties == 1) ? tsec : tmax;
+        if (is_target && ties == 1) {
+          // (the exponent stays within 2^90 of the target all the same: the target's own e^{z - cap}, scaled like the rest,
+          // still goes into the row sum, and must not leave the floats' range when everything else is at -cap under a large cap)
+          texp = tsec;
+          lfloor = c2 * fast_rcp(1.0f + fast_exp2(tmax * k1)) - 90.0f;
+        }
       }
     }
     const float lamb = lam[b * LAM_STRIDE + (lane_id() & (LAM_LANES - 1))];      // (index taken anew: see lane_id)
-    const float lg = wave_max_dpp(fmaf(c2, fast_rcp(1.0f + fast_exp2(texp * k1)), lamb));      // over the block: log2 of the largest boosted e^{z - cap}
+    const float rexp = fast_rcp(1.0f + fast_exp2(texp * k1));
+    const float lg = wave_max_dpp(EXCL ? fmaxf(c2 * rexp, lfloor) + lamb : fmaf(c2, rexp, lamb));      // over the block: log2 of the largest boosted e^{z - cap}
     const float sb = fminf(floorf(8.8f - lg), 126.f);         // from -112 (boost <= 120) to 8 + 2 cap log2(e) - boost, held to what the exponent byte has
     const float cs = sb + 2.0f + lamb;                        // the 4 of 4 r (1 - r) and the row's boost ride along
     expword |= (uint32_t)(127 - (int)sb) << (8 * b);

@@ -751,3 +751,34 @@ def test_a_column_that_ties_with_the_target(keep):
     assert bool(torch.isfinite(ours["dx"]).all()) and bool(torch.isfinite(ours["dw"]).all())
     ref = pu.run_oracle(inp, ours, "none", grad_output=go)
     pu.check_parity(ours, ref, "none")
+
+
+@pytest.mark.parametrize("keep", [True, False])
+def test_saturated_logits_under_the_largest_cap(keep):
+    """cap = 40 and logits that saturate it: every row's target at +cap, everything else at -cap, so that e^{z - cap} spans
+    e^{-80}.  The target, kept out of its block's exponent, still goes into the row sum at the block's scale: the sum
+    must stay finite."""
+    from slowrun_amd import cuda_kernels as ck
+    from oracle import eager
+    N, d, V = 300, 64, 700
+    g = torch.Generator().manual_seed(2)
+    y = torch.randint(0, V, (N,), generator=g)
+    x = torch.zeros(N, d); x[:, 0] = 1.0
+    w = torch.full((d, V), 0.0); w[0, :] = -400.0
+    x, w, y = x.cuda(), w.cuda(), y.cuda()
+    x = x + 0.0
+    # row i gets +400 at its own target through hidden unit 1 + (i % 32): rows of one block of 32 have different units
+    for i in range(N):
+        x[i, 1 + (i % 32)] = 1.0
+    w[1:33, :] = 0.0
+    for i in range(N):
+        w[1 + (i % 32), y[i]] = 800.0
+    x_s, w_s, cap = 1.0 / 448.0 * 2.0, 800.0 / 448.0, 40.0
+    go = torch.full((N,), 1.0 / N, device="cuda")
+    out, saved, lse, am, nv = ck.ce_forward(x, w, y, x_s, w_s, cap, "none", keep_dlogits=keep)
+    dx, dw = ck.ce_backward(saved, y, go, N, d, V, x_s, w_s, cap, 1.0, "none", torch.float32, torch.float32, keep_dlogits=keep)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(lse).all())
+    assert bool(torch.isfinite(dx).all()) and bool(torch.isfinite(dw).all())
+    ref = eager.softcapped_ce(x, w, y, x_s, w_s, cap=cap, reduction="none", grad_output=go)
+    assert float((lse - ref["lse"]).abs().max()) <= 1e-3 * float(ref["lse"].abs().max())
